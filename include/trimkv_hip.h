@@ -1,0 +1,210 @@
+/*
+ * trimkv_hip.h -- C ABI of libtrimkv_hip.so: the TRIM-KV cache hot path on MI355X (gfx950).
+ *
+ * Every pointer that is not marked "host" is a DEVICE pointer.  No function allocates, frees,
+ * synchronises the host or throws; all work is enqueued on `stream` (a hipStream_t passed as
+ * void*, NULL = the default stream).  Every function returns 0 on success, a negative
+ * trimkv_status on an argument error (nothing was launched) or a positive hipError_t when the
+ * launch itself failed.  trimkv_last_error() returns a thread-local description of the last
+ * non-zero return.
+ *
+ * Storage model ("slabs").  One layer of the cache is four arrays shared by all
+ * nseg = batch * kv_heads segments, segment id seg = b * kv_heads + h:
+ *
+ *     k_slab, v_slab   [nseg][cap][head_dim]   bf16/fp16 rows, oldest token first
+ *     lb_slab          [nseg][cap]             log-retention log(beta) (f32 / bf16 / f16)
+ *     pos_slab         [nseg][cap]             absolute token position, int64
+ *     seg_len          [nseg]                  int32, rows in use per segment
+ *
+ * Rows [0, seg_len[seg]) of a segment are live, the rest is slack that appends fill and
+ * evictions free.  A dense cache is the special case in which every seg_len is equal; a ragged
+ * cache is the same storage with unequal lengths.  Kernels that only read K/V also accept a
+ * packed layout through `seg_start` (row offset of every segment, e.g. cu_seqlens_k).
+ *
+ * Reference citations are to yejun-yun/trimkv, paths relative to its repository root.
+ */
+#ifndef TRIMKV_HIP_H
+#define TRIMKV_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    TRIMKV_OK = 0,
+    TRIMKV_ERR_NULL = -1,        /* a required pointer is NULL                              */
+    TRIMKV_ERR_SHAPE = -2,       /* a size is non-positive or unsupported                   */
+    TRIMKV_ERR_DTYPE = -3,       /* unknown dtype code                                      */
+    TRIMKV_ERR_CAPACITY = -4,    /* the operation would overflow the slab capacity          */
+    TRIMKV_ERR_WORKSPACE = -5,   /* workspace missing or too small                          */
+    TRIMKV_ERR_UNSUPPORTED = -6  /* valid arguments this build has no kernel for            */
+} trimkv_status;
+
+typedef enum { TRIMKV_F32 = 0, TRIMKV_BF16 = 1, TRIMKV_F16 = 2 } trimkv_dtype;
+
+/* Eviction score (cache_utils.py:176-184): alpha = log(beta)*age, knorm_alpha adds log||k||. */
+typedef enum { TRIMKV_SCORE_ALPHA = 0, TRIMKV_SCORE_KNORM_ALPHA = 1 } trimkv_strategy;
+
+/* How the score is rounded.
+ *  UPCAST : fp32(log beta) * fp32(age), one fp32 multiply -- the dense class, cache_utils.py:172-174.
+ *  NATIVE : the product in log beta's own dtype, as the ragged classes compute it
+ *           (cache_utils.py:386, 441, 755, 874); identical to UPCAST for f32 log beta, and
+ *           round_lb(fp32(round_lb(age)) * fp32(log beta)) for a 16-bit log beta.
+ *  knorm:  UPCAST adds log(norm) with norm and log rounded to K's dtype and no clamp (:178-180);
+ *          NATIVE clamps the norm at 1e-12 first (:390, 450, 759, 878).                          */
+typedef enum { TRIMKV_ROUND_UPCAST = 0, TRIMKV_ROUND_NATIVE = 1 } trimkv_score_rounding;
+
+/* Library version (major*10000 + minor*100 + patch).  No reference counterpart. */
+int trimkv_version(void);
+
+/* Thread-local text for the last non-zero status returned on this thread ("" if none). */
+const char* trimkv_last_error(void);
+
+/*
+ * trimkv_append -- append s_new tokens to every segment.
+ * Replaces TrimKVCache.update's four torch.cat calls (src/trimkv/cache_utils.py:104-107) and,
+ * for the flat caches, the four update_flatten_view_triton re-packs
+ * (src/trimkv/cache_utils.py:646-676, src/trimkv/triton/db_cache_utils.py:86-186).
+ *
+ * New rows come from strided [batch][kv_heads][s_new][...] tensors; strides are in ELEMENTS,
+ * the innermost head_dim axis of k_new/v_new is contiguous.  pos strides may be 0 (broadcast).
+ * Row j of segment seg is written at slab row seg_len[seg] + j; afterwards seg_len += s_new.
+ * cu_seqlens (optional, [nseg+1] int32) is advanced as the reference does:
+ * cu[i] += i * s_new (cache_utils.py:678-680).
+ * The caller guarantees seg_len[seg] + s_new <= cap for every segment (max_len_after is the
+ * caller's upper bound on the new maximum length and is checked against cap).
+ */
+int trimkv_append(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                  int32_t* cu_seqlens, int nseg, int kv_heads, int cap, int head_dim,
+                  int kv_dtype, int lb_dtype,
+                  const void* k_new, const void* v_new,
+                  int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                  const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h, int64_t lb_stride_s,
+                  const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h, int64_t pos_stride_s,
+                  int s_new, int max_len_after, void* stream);
+
+/*
+ * trimkv_gate_hidden -- first half of the `rg` retention gate, for the tokens of one append:
+ *     part[j][t][h] = sum over the j-th slice of intermediate units u of
+ *                     W2[h][u] * silu( W1[u][:] . x[t][:] + b1[u] )
+ * (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:171-176).  x [ntok][hidden], w1
+ * [inter][hidden], b1 [inter] (nullable), w2 [kv_heads][inter], all `dtype` (bf16);
+ * part is f32 [nslice][ntok][kv_heads] with nslice = trimkv_gate_slices(inter).
+ * The second half (sum of slices + bias, logsigmoid, :177-179) is fused into
+ * trimkv_append_gated.
+ */
+int trimkv_gate_slices(int inter);
+int trimkv_gate_hidden(const void* x, const void* w1, const void* b1, const void* w2, float* part,
+                       int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
+
+/*
+ * trimkv_append_gated -- trimkv_append whose log(beta) is produced inside the append kernel:
+ *     lb[b][h][s] = logsigmoid( sum_j part[j][b*s_new + s][h] + gate_bias[h] )
+ * rounded to lb_dtype (modeling_trimkv_qwen3.py:177-179, then the transpose at :333).
+ * gate_bias is f32 [kv_heads].  Everything else as trimkv_append.
+ */
+int trimkv_append_gated(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                        int32_t* cu_seqlens, int nseg, int kv_heads, int cap, int head_dim,
+                        int kv_dtype, int lb_dtype,
+                        const void* k_new, const void* v_new,
+                        int64_t kv_stride_b, int64_t kv_stride_h, int64_t kv_stride_s,
+                        const float* gate_part, int gate_nslice, const float* gate_bias,
+                        const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h, int64_t pos_stride_s,
+                        int s_new, int max_len_after, void* stream);
+
+/*
+ * trimkv_evict -- per-segment top-k eviction with in-place, order-preserving compaction.
+ * Replaces TrimKVCache.compress_layer (src/trimkv/cache_utils.py:160-198: score, topk, sort,
+ * four gathers) and the per-head top-k of the flat caches (cache_utils.py:508-521).
+ *
+ * For every segment with n = seg_len[seg] and k = keep_per_seg ? keep_per_seg[seg] : keep:
+ * if n < k + slack or n <= k the segment is left alone; otherwise the k tokens with the
+ * largest score are kept in their original order in rows [0, k) and seg_len[seg] = k.
+ *     score_i = log_beta_i * (q_idx - pos_i)            (see trimkv_score_rounding)
+ * The last `sliding_window` tokens score +inf (cache_utils.py:186-187).  Equal scores at the
+ * cut are resolved towards the older token (torch.topk leaves that order unspecified).
+ * max_len: caller's upper bound on seg_len (sizes on-chip storage; <= cap).
+ * kept_idx (optional, int32 [nseg][kept_stride]): the kept source rows, ascending.
+ * workspace: trimkv_evict_workspace(nseg, max_len) bytes (0 when the scores fit on chip).
+ */
+size_t trimkv_evict_workspace(int nseg, int max_len);
+int trimkv_evict(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                 int nseg, int cap, int head_dim, int kv_dtype, int lb_dtype,
+                 int keep, const int32_t* keep_per_seg, int slack,
+                 int64_t q_idx, int strategy, int rounding, int sliding_window, int max_len,
+                 int32_t* kept_idx, int kept_stride,
+                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * trimkv_group_threshold -- shared-budget selection over groups of segments.
+ * Replaces the concatenate-then-topk of the flat caches: one budget per batch element over its
+ * kv_heads segments (cache_utils.py:771-787), or over all its layers (cache_utils.py:862-898),
+ * or one budget over everything for a single sequence (cache_utils.py:397, 458).
+ *
+ * Group g owns segments [g*segs_per_group, (g+1)*segs_per_group) of each of the nlayers layers
+ * whose slabs are given by the device pointer tables lb_slabs / pos_slabs / k_slabs / seg_lens
+ * (nlayers entries each; k_slabs only read for knorm).  Per group it finds the budget-th
+ * largest score over all those tokens (budget clamped to the group's token count) and writes,
+ * for every (layer, segment), new_len[layer*nseg + seg] = number of its tokens that are kept.
+ * thr_key [ngroups] receives the order-preserving key of the cut score and tie_take [ngroups]
+ * how many tokens equal to it are kept (oldest layer/segment/row first); tie_base
+ * [nlayers*nseg] receives how many equal-to-cut tokens precede each segment in that order.
+ * With use_threshold != 0 no selection is done: a token is kept iff score >= threshold_score
+ * (cache_utils.py:462, 893; -inf keeps everything) and budget is ignored.
+ */
+int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+                           const void* const* k_slabs, const int32_t* const* seg_lens,
+                           int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
+                           int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
+                           int64_t q_idx, int strategy, int rounding,
+                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                           void* stream);
+
+/*
+ * trimkv_compact_threshold -- in-place compaction of one layer against group thresholds:
+ * keeps token i of segment seg iff key_i > thr_key[g] or (key_i == thr_key[g] and its rank
+ * among equal keys, tie_base[seg] + rank inside the segment, is < tie_take[g]); g =
+ * seg / segs_per_group.  Replaces the boolean-mask indexing of the flat caches
+ * (cache_utils.py:401-404, 469-472, 808-811, 922-925) and their head_lens popcounts.
+ * thr_key/tie_take are [ngroups]; tie_base [nseg] for THIS layer; seg_len is updated.
+ */
+int trimkv_compact_threshold(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                             int nseg, int segs_per_group, int cap, int head_dim, int kv_dtype, int lb_dtype,
+                             const uint32_t* thr_key, const int32_t* tie_take, const int32_t* tie_base,
+                             int64_t q_idx, int strategy, int rounding, int max_len,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * trimkv_build_cu_seqlens -- cu[0] = 0, cu[i+1] = cu[i] + seg_len[i] (int32), the offsets the
+ * reference rebuilds with torch.cumsum after every eviction (cache_utils.py:412-416, 830-834).
+ */
+int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlens, void* stream);
+
+/*
+ * trimkv_decode_attn -- single-query GQA attention over every segment's retained K/V:
+ *     out[seg*group + g][:] = softmax( q[seg*group + g] . K_seg^T * scale ) V_seg
+ * Replaces flash_attn_varlen_func as called at src/trimkv/attn/flash_attn.py:61-71 and 135-145
+ * (Q_LEN == 1), HF flash_attention_2 on the dense cache (src/trimkv/attn/__init__.py:15-26) and
+ * eager_attention_forward (src/trimkv/attn/eager_attn.py:48-73) at decode time.
+ *
+ * q and out are [nseg*group][head_dim], contiguous, kv dtype -- i.e. [B][Hq][1][D] and
+ * [B][1][Hq][D].  Segment rows start at seg_start[seg] (int32 row offsets, e.g. cu_seqlens_k)
+ * or, when seg_start is NULL, at seg*cap.  A segment of length 0 yields zeros.
+ * Split-K: every segment is cut into chunks of `chunk` rows (0 = chosen from nseg/max_len);
+ * partial (max, sum, accumulator) triples go through `workspace`
+ * (trimkv_decode_attn_workspace bytes) and are merged by a second kernel.
+ * head_dim must be 128; group in [1, 8]; dtype bf16.
+ */
+size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim, int max_len, int chunk);
+int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
+                       const int32_t* seg_len, const int32_t* seg_start,
+                       int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                       int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRIMKV_HIP_H */

@@ -1,0 +1,92 @@
+"""ctypes binding of libtrimkv_hip.so -- the only way Python reaches the HIP kernels.
+
+There is no fallback: if the library is missing or a call fails, a ``TrimKVLibraryError`` is
+raised.  Argument and return types mirror ``include/trimkv_hip.h`` one to one.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtrimkv_hip.so")
+
+F32, BF16, F16 = 0, 1, 2
+SCORE_ALPHA, SCORE_KNORM_ALPHA = 0, 1
+ROUND_UPCAST, ROUND_NATIVE = 0, 1
+
+
+class TrimKVLibraryError(RuntimeError):
+    pass
+
+
+_p, _i, _i64, _sz, _f = C.c_void_p, C.c_int, C.c_int64, C.c_size_t, C.c_float
+
+# name -> (restype, argtypes); must list every symbol trimkv_hip.h declares
+SIGNATURES = {
+    "trimkv_version": (_i, []),
+    "trimkv_last_error": (C.c_char_p, []),
+    "trimkv_append": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64, _i64,
+                           _p, _i64, _i64, _i64, _p, _i64, _i64, _i64, _i, _i, _p]),
+    "trimkv_gate_slices": (_i, [_i]),
+    "trimkv_gate_hidden": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "trimkv_append_gated": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64, _i64,
+                                 _p, _i, _p, _p, _i64, _i64, _i64, _i, _i, _p]),
+    "trimkv_evict_workspace": (_sz, [_i, _i]),
+    "trimkv_evict": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _i64, _i, _i, _i, _i,
+                          _p, _i, _p, _sz, _p]),
+    "trimkv_group_threshold": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
+                                    _p, _p, _p, _p, _p]),
+    "trimkv_compact_threshold": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i, _i, _i,
+                                      _p, _sz, _p]),
+    "trimkv_build_cu_seqlens": (_i, [_p, _i, _p, _p]),
+    "trimkv_decode_attn_workspace": (_sz, [_i, _i, _i, _i, _i]),
+    "trimkv_decode_attn": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p]),
+}
+
+_lib = None
+
+
+def load():
+    """Load (once) and return the ctypes handle; raises if the library has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise TrimKVLibraryError(
+            f"{LIB_PATH} is missing: build it with `python -m trimkv_amd.build` (hipcc, gfx950). "
+            "There is no CPU fallback.")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = load().trimkv_last_error().decode("utf-8", "replace")
+        raise TrimKVLibraryError(f"{what} failed with status {rc}: {msg}")
+
+
+def dtype_code(dt) -> int:
+    import torch
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    if dt == torch.float16:
+        return F16
+    raise TrimKVLibraryError(f"unsupported dtype {dt}")
+
+
+def ptr(t) -> int:
+    """Device (or host) address of a tensor, or None."""
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device) -> int:
+    import torch
+    return torch.cuda.current_stream(device).cuda_stream

@@ -1,0 +1,378 @@
+// Single-query GQA attention over ragged per-segment K/V (split-K + merge), gfx950.
+//
+// Replaces flash_attn_varlen_func at Q_LEN == 1 (src/trimkv/attn/flash_attn.py:61-71, 135-145),
+// HF flash_attention_2 on the dense cache (src/trimkv/attn/__init__.py:15-26) and
+// eager_attention_forward (src/trimkv/attn/eager_attn.py:48-73) at decode time.
+//
+// The op is HBM-bound (about 4 flop per byte of K/V), so the kernel is built around the stream:
+//   * a wavefront reads whole 256-byte rows, 16 lanes x 16 bytes per row, 4 rows per load
+//     instruction (1 KiB contiguous), always with the next tile already in flight;
+//   * q.K uses v_dot2_f32_bf16 on the bytes as loaded; the 16-lane partial sums of one tile are
+//     reduced with a transposing DPP butterfly that leaves ONE (row, head) score per lane, so the
+//     softmax costs one exp per lane per tile;
+//   * a wavefront takes 128 rows at a time: all their scores first, one running-max update, then
+//     the V rows; probabilities reach the lanes that hold the matching V rows through LDS as
+//     packed bf16 pairs, and P.V is v_dot2_f32_bf16 over two rows at a time (v_perm_b32
+//     interleaves the rows);
+//   * the four wavefronts of a workgroup own disjoint quarters of the workgroup's rows and merge
+//     (max, sum, accumulator) in LDS; workgroups of one segment merge in a second tiny kernel.
+#include "common.hip.h"
+
+namespace trimkv {
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int AT_THREADS = 256;
+constexpr int AT_WAVES = 4;
+constexpr int AT_D = 128;            // head_dim
+constexpr int AT_BLOCK_ROWS = 128;   // rows one wavefront scores before it touches V
+constexpr float AT_NEG = -1.0e30f;   // "minus infinity" that stays finite under subtraction
+
+template <int G>
+struct AttnCfg {
+    static constexpr int NJ = G <= 2 ? 8 : (G <= 4 ? 4 : 2);  // load instructions (of 4 rows) per tile
+    static constexpr int NV = NJ * G;                          // scores per tile per 16-lane row group (<= 16)
+    static constexpr int TILE_ROWS = NJ * 4;
+    static constexpr int NT = AT_BLOCK_ROWS / TILE_ROWS;       // tiles per block
+    static constexpr int PSTRIDE = NV <= 8 ? 8 : 16;           // bf16 slots per (tile, row group) in LDS
+};
+
+typedef uint32_t __attribute__((may_alias)) u32_alias;  // LDS words written as bf16 halves, read as pairs
+typedef uint16_t __attribute__((may_alias)) u16_alias;
+#define DPP_MOV(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), 0xf, 0xf, false))
+constexpr int DPP_QUAD_XOR1 = 0xB1;       // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;       // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_ROR8 = 0x128;
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+
+// Sum 16 per-lane values over the 16 lanes of a row group, leaving value x(c) in lane c, where
+// x(c) = bit2(c)<<3 | bit0(c)<<2 | bit1(c)<<1 | bit3(c).  Each step halves the values a lane
+// carries: the lane keeps the half its lane bit names and adds the partner's copy of that half.
+__device__ __forceinline__ float reduce16_transposed(float (&v)[16], int c) {
+    const bool b0 = c & 1, b1 = c & 2, b2 = c & 4, b3 = c & 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float keep = b2 ? v[i + 8] : v[i], send = b2 ? v[i] : v[i + 8];
+        v[i] = keep + DPP_MOV(send, DPP_ROW_HALF_MIRROR);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float keep = b0 ? v[i + 4] : v[i], send = b0 ? v[i] : v[i + 4];
+        v[i] = keep + DPP_MOV(send, DPP_QUAD_XOR1);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float keep = b1 ? v[i + 2] : v[i], send = b1 ? v[i] : v[i + 2];
+        v[i] = keep + DPP_MOV(send, DPP_QUAD_XOR2);
+    }
+    const float keep = b3 ? v[1] : v[0], send = b3 ? v[0] : v[1];
+    return keep + DPP_MOV(send, DPP_ROW_ROR8);
+}
+
+struct AttnArgs {
+    const uint4* q; void* out; const uint4* k; const uint4* v;
+    const int32_t* seg_len; const int32_t* seg_start;
+    int nseg, cap, max_len, chunk, nsplit, direct;
+    float scale_log2;
+    float* ws_o; float* ws_ml;
+};
+
+template <int G>
+__global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
+    using C = AttnCfg<G>;
+    constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
+
+    __shared__ u32_alias p_lds[AT_WAVES][NT][4][PS / 2];
+    __shared__ uint32_t smax[AT_WAVES][8];
+    __shared__ float so[AT_WAVES][G][AT_D];
+    __shared__ float sm[AT_WAVES][8];
+    __shared__ float sl[AT_WAVES][8];
+
+    const int seg = blockIdx.y, split = blockIdx.x;
+    int n = a.seg_len[seg];
+    n = max(0, min(n, a.max_len));
+    const int nsp = (n + a.chunk - 1) / a.chunk;
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int c = lane & 15, r = lane >> 4;
+
+    if (split >= nsp) {
+        if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
+            for (int i = tid; i < G * AT_D; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * AT_D + i] = 0;
+        }
+        return;
+    }
+    const int rps = (n + nsp - 1) / nsp;
+    const int t0 = split * rps, t1 = min(n, t0 + rps);
+    const int pw = (t1 - t0 + AT_WAVES - 1) / AT_WAVES;
+    const int w0 = t0 + w * pw, w1 = min(t1, w0 + pw);
+
+    const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
+    const uint4* kp = a.k + row0 * 16 + c;  // 16 uint4 per 256-byte row; this lane's 16-byte column
+    const uint4* vp = a.v + row0 * 16 + c;
+
+    uint4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) qv[g] = a.q[((int64_t)seg * G + g) * 16 + c];
+
+    // which (row-in-tile, head) this lane owns after the transposing reduction
+    const int my_x = ((c & 4) << 1) | ((c & 1) << 2) | (c & 2) | ((c & 8) >> 3);
+    const bool my_valid = my_x < NV;
+    const int my_j = my_x / G, my_g = my_x - my_j * G;
+
+    float o[G][8];
+    float m_run[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m_run[g] = AT_NEG;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = 0.0f;
+    }
+    float l_lane = 0.0f;
+
+    auto load_tile = [&](const uint4* base, int row_begin, uint4 (&dst)[NJ]) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int row = min(row_begin + j * 4 + r, w1 - 1);  // rows past the end re-read the last one (weight 0)
+            dst[j] = base[(int64_t)row * 16];
+        }
+    };
+
+    if (w0 < w1) {
+        // Two register buffers per operand, indexed by tile parity (the tile loops are fully
+        // unrolled, so the parity is static): while tile t is being consumed, tile t+1 -- or the
+        // first tile of the next phase -- is in flight.  NT is even, so tile 0 always sits in [0].
+        uint4 kb[2][NJ], vb[2][NJ];
+        load_tile(kp, w0, kb[0]);
+#pragma unroll 1
+        for (int blk = w0; blk < w1; blk += AT_BLOCK_ROWS) {
+            const int nrows = min(AT_BLOCK_ROWS, w1 - blk);
+            float s[NT];
+            // ---- scores of up to 128 rows ----
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                s[t] = AT_NEG;
+                if (t * TILE_ROWS < nrows) {
+                    if (t + 1 < NT && (t + 1) * TILE_ROWS < nrows) load_tile(kp, blk + (t + 1) * TILE_ROWS, kb[(t + 1) & 1]);
+                    else load_tile(vp, blk, vb[0]);
+                    float part[16];
+#pragma unroll
+                    for (int x = 0; x < 16; ++x) part[x] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                        for (int g = 0; g < G; ++g) {
+                            float acc = dot2_bf16(kb[t & 1][j].x, qv[g].x, 0.0f);
+                            acc = dot2_bf16(kb[t & 1][j].y, qv[g].y, acc);
+                            acc = dot2_bf16(kb[t & 1][j].z, qv[g].z, acc);
+                            acc = dot2_bf16(kb[t & 1][j].w, qv[g].w, acc);
+                            part[j * G + g] = acc;
+                        }
+                    }
+                    const float val = reduce16_transposed(part, c);
+                    const int row = blk + t * TILE_ROWS + my_j * 4 + r;
+                    if (my_valid && row < w1) s[t] = val * a.scale_log2;
+                }
+            }
+            // ---- running max, probabilities ----
+            float lmax = AT_NEG;
+#pragma unroll
+            for (int t = 0; t < NT; ++t) lmax = fmaxf(lmax, s[t]);
+            if (lane < 8) smax[w][lane] = float_key(AT_NEG);
+            if (my_valid) atomicMax(&smax[w][my_g], float_key(lmax));
+            float alpha_mine = 1.0f, m_mine = AT_NEG;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float mb = key_float(smax[w][g]);
+                const float m_new = fmaxf(m_run[g], mb);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_new);
+                m_run[g] = m_new;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[g][e] *= alpha;
+                if (g == my_g) { alpha_mine = alpha; m_mine = m_new; }
+            }
+            l_lane *= alpha_mine;
+            u16_alias* pw16 = (u16_alias*)&p_lds[w][0][0][0];
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if (t * TILE_ROWS < nrows) {
+                    const float p = my_valid ? __builtin_amdgcn_exp2f(s[t] - m_mine) : 0.0f;
+                    l_lane += p;
+                    if (my_valid) pw16[(t * 4 + r) * PS + my_g * NJ + my_j] = f32_to_bf16_bits(p);
+                }
+            }
+            // ---- P.V over the same rows ----
+#pragma unroll
+            for (int t = 0; t < NT; ++t) {
+                if (t * TILE_ROWS < nrows) {
+                    if (t + 1 < NT && (t + 1) * TILE_ROWS < nrows) load_tile(vp, blk + (t + 1) * TILE_ROWS, vb[(t + 1) & 1]);
+                    else if (blk + AT_BLOCK_ROWS < w1) load_tile(kp, blk + AT_BLOCK_ROWS, kb[0]);
+                    uint32_t pd[NV / 2];
+#pragma unroll
+                    for (int i = 0; i < NV / 2; ++i) pd[i] = p_lds[w][t][r][i];
+#pragma unroll
+                    for (int u = 0; u < NJ / 2; ++u) {
+                        const uint4 ra = vb[t & 1][2 * u], rb = vb[t & 1][2 * u + 1];
+                        const uint32_t va[4] = {ra.x, ra.y, ra.z, ra.w};
+                        const uint32_t vv[4] = {rb.x, rb.y, rb.z, rb.w};
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t lo = __builtin_amdgcn_perm(vv[i], va[i], 0x05040100u);  // rows (2u, 2u+1), element 2i
+                            const uint32_t hi = __builtin_amdgcn_perm(vv[i], va[i], 0x07060302u);  // rows (2u, 2u+1), element 2i+1
+#pragma unroll
+                            for (int g = 0; g < G; ++g) {
+                                const uint32_t pp = pd[(g * NJ) / 2 + u];
+                                o[g][2 * i] = dot2_bf16(lo, pp, o[g][2 * i]);
+                                o[g][2 * i + 1] = dot2_bf16(hi, pp, o[g][2 * i + 1]);
+                            }
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- merge the four row groups of a wavefront, then the four wavefronts ----
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float x = o[g][e];
+            x += __shfl_xor(x, 16, 64);
+            x += __shfl_xor(x, 32, 64);
+            o[g][e] = x;
+        }
+    }
+    if (lane < 8) sl[w][lane] = 0.0f;
+    if (my_valid && l_lane != 0.0f) atomicAdd(&sl[w][my_g], l_lane);
+    if (r == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) so[w][g][c * 8 + e] = o[g][e];
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) sm[w][g] = m_run[g];
+    }
+    __syncthreads();
+    for (int i = tid; i < G * AT_D; i += AT_THREADS) {
+        const int g = i / AT_D, d = i - g * AT_D;
+        float mx = AT_NEG;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) mx = fmaxf(mx, sm[ww][g]);
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) {
+            const float f = __builtin_amdgcn_exp2f(sm[ww][g] - mx);
+            acc += f * so[ww][g][d];
+            lsum += f * sl[ww][g];
+        }
+        if (a.direct) {
+            const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+            ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
+        } else {
+            const int64_t slot = ((int64_t)seg * a.nsplit + split) * G + g;
+            a.ws_o[slot * AT_D + d] = acc;
+            if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
+        }
+    }
+}
+
+template <int G>
+__global__ __launch_bounds__(AT_D) void decode_attn_merge_kernel(AttnArgs a) {
+    const int seg = blockIdx.x, d = threadIdx.x;
+    int n = a.seg_len[seg];
+    n = max(0, min(n, a.max_len));
+    const int nsp = (n + a.chunk - 1) / a.chunk;
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        float mx = AT_NEG;
+        for (int s = 0; s < nsp; ++s) mx = fmaxf(mx, a.ws_ml[(((int64_t)seg * a.nsplit + s) * G + g) * 2]);
+        float acc = 0.0f, lsum = 0.0f;
+        for (int s = 0; s < nsp; ++s) {
+            const int64_t slot = ((int64_t)seg * a.nsplit + s) * G + g;
+            const float f = __builtin_amdgcn_exp2f(a.ws_ml[slot * 2] - mx);
+            acc += f * a.ws_o[slot * AT_D + d];
+            lsum += f * a.ws_ml[slot * 2 + 1];
+        }
+        const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+        ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
+    }
+}
+
+static int pick_chunk(int nseg, int max_len) {
+    // Aim for about 8 workgroups per CU (256 CUs) so the tail of the grid is short, but keep a
+    // workgroup's share at 256 rows or more so the merge traffic stays below 1 % of the K/V bytes.
+    const int64_t rows = (int64_t)nseg * max_len;
+    int64_t chunk = (rows + 2047) / 2048;
+    chunk = ((chunk + 127) / 128) * 128;
+    if (chunk < 256) chunk = 256;
+    if (chunk > 2048) chunk = 2048;
+    return (int)chunk;
+}
+
+template <int G>
+static void launch_attn(const AttnArgs& a, hipStream_t st) {
+    hipLaunchKernelGGL(decode_attn_kernel<G>, dim3(a.nsplit, a.nseg), dim3(AT_THREADS), 0, st, a);
+    if (!a.direct) hipLaunchKernelGGL(decode_attn_merge_kernel<G>, dim3(a.nseg), dim3(AT_D), 0, st, a);
+}
+
+}  // namespace trimkv
+
+using namespace trimkv;
+
+extern "C" size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim, int max_len, int chunk) {
+    if (nseg <= 0 || group <= 0 || head_dim <= 0 || max_len <= 0) return 0;
+    if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
+    const int nsplit = (max_len + chunk - 1) / chunk;
+    if (nsplit <= 1) return 0;
+    return (size_t)nseg * nsplit * group * (head_dim + 2) * sizeof(float);
+}
+
+extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
+                                  const int32_t* seg_len, const int32_t* seg_start,
+                                  int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                                  int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_decode_attn";
+    if (!q || !out || !k_slab || !v_slab || !seg_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
+    if (head_dim != AT_D) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be %d (got %d)", fn, AT_D, head_dim);
+    if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
+    if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
+    if (nseg > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nseg=%d exceeds the grid limit 65535", fn, nseg);
+    if (max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
+    if (((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_slab | (uintptr_t)v_slab) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: q/out/K/V must be 16-byte aligned", fn);
+    if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
+    if (chunk % 64) return fail(TRIMKV_ERR_SHAPE, "%s: chunk must be a multiple of 64 (got %d)", fn, chunk);
+    AttnArgs a;
+    a.q = (const uint4*)q; a.out = out; a.k = (const uint4*)k_slab; a.v = (const uint4*)v_slab;
+    a.seg_len = seg_len; a.seg_start = seg_start; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
+    a.nsplit = (max_len + chunk - 1) / chunk;
+    a.direct = a.nsplit <= 1;
+    a.scale_log2 = scale * 1.4426950408889634f;
+    a.ws_o = nullptr; a.ws_ml = nullptr;
+    if (!a.direct) {
+        const size_t need = trimkv_decode_attn_workspace(nseg, group, head_dim, max_len, chunk);
+        if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+        a.ws_o = (float*)workspace;
+        a.ws_ml = a.ws_o + (size_t)nseg * a.nsplit * group * AT_D;
+    }
+    hipStream_t st = (hipStream_t)stream;
+    switch (group) {
+        case 1: launch_attn<1>(a, st); break;
+        case 2: launch_attn<2>(a, st); break;
+        case 3: launch_attn<3>(a, st); break;
+        case 4: launch_attn<4>(a, st); break;
+        case 5: launch_attn<5>(a, st); break;
+        case 6: launch_attn<6>(a, st); break;
+        case 7: launch_attn<7>(a, st); break;
+        default: launch_attn<8>(a, st); break;
+    }
+    return launch_status(fn);
+}

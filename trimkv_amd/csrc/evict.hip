@@ -1,0 +1,539 @@
+// Eviction kernels: retention score -> per-segment (or per-group) top-k -> in-place compaction.
+//
+// Replaces TrimKVCache.compress_layer (src/trimkv/cache_utils.py:160-198), the per-head top-k of
+// the flat caches (:508-521) and their concatenate/topk/boolean-mask pipelines (:397-416,
+// :771-834, :862-943).  One workgroup owns one segment: scores become order-preserving 32-bit
+// keys staged in LDS, the cut is found by a 4-pass 8-bit radix select, a block scan turns the
+// keep flags into the ascending list of kept source rows (written over the keys), and rows are
+// moved tile by tile inside the slab (destination row <= source row, so a tile is read in full
+// before it is written).
+#include "common.hip.h"
+
+namespace trimkv {
+
+constexpr int EV_THREADS = 256;
+constexpr int EV_ITEMS = 4;             // consecutive elements per thread in the compaction scan
+constexpr int EV_ROW_PASSES = 4;        // rows held in registers per thread while a tile moves
+constexpr int EV_LDS_KEY_BYTES = 128 * 1024;  // largest key array kept in LDS (32768 tokens)
+constexpr int GT_THREADS = 1024;        // group-threshold workgroup
+
+struct ScoreArgs {
+    const void* lb; const int64_t* pos; const char* k;  // bases of ONE segment
+    int lb_dtype, kv_dtype, row_bytes, strategy, rounding, sliding_window;
+    int64_t q_idx;
+};
+
+// ||k_row|| and its log, rounded as torch rounds them for a 16-bit K (norm -> K dtype, log -> K dtype).
+__device__ __forceinline__ float knorm_term(const ScoreArgs& s, int i) {
+    const uint16_t* row = (const uint16_t*)(s.k + (int64_t)i * s.row_bytes);
+    const int d = s.row_bytes >> 1;
+    float acc = 0.0f;
+    for (int e = 0; e < d; ++e) {
+        const float x = s.kv_dtype == TRIMKV_BF16 ? bf16_bits_to_f32(row[e]) : f16_bits_to_f32(row[e]);
+        acc = __fmaf_rn(x, x, acc);
+    }
+    float nrm = round_to_dtype(__fsqrt_rn(acc), s.kv_dtype);
+    if (s.rounding == TRIMKV_ROUND_NATIVE) nrm = fmaxf(nrm, round_to_dtype(1e-12f, s.kv_dtype));
+    return round_to_dtype(logf(nrm), s.kv_dtype);
+}
+
+// Order-preserving key of token i's score; n = segment length (for the sliding window).
+__device__ __forceinline__ uint32_t score_key(const ScoreArgs& s, int i, int n) {
+    if (s.sliding_window > 0 && i >= n - s.sliding_window) return float_key(__builtin_inff());
+    const float lb = load_as_f32(s.lb, i, s.lb_dtype);
+    const float age = (float)(s.q_idx - s.pos[i]);  // int64 -> fp32, round to nearest even
+    float sc;
+    if (s.rounding == TRIMKV_ROUND_NATIVE && s.lb_dtype != TRIMKV_F32) {
+        sc = round_to_dtype(__fmul_rn(round_to_dtype(age, s.lb_dtype), lb), s.lb_dtype);
+        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = round_to_dtype(__fadd_rn(sc, knorm_term(s, i)), s.lb_dtype);
+    } else {
+        sc = __fmul_rn(lb, age);
+        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = __fadd_rn(sc, knorm_term(s, i));
+    }
+    return float_key(sc);
+}
+
+// ---- 4-pass radix select: the `want`-th largest of keys[0..n) -------------------------------
+// Returns the key at the cut and, through *take_eq, how many elements equal to it are kept.
+// hist: 256 words of LDS; scratch: EV_THREADS/64 + 3 words of LDS.
+__device__ __forceinline__ uint32_t radix_select(const uint32_t* keys, int n, int want, uint32_t* hist, uint32_t* scratch,
+                                                 int* take_eq) {
+    uint32_t prefix = 0;
+    uint32_t remaining = (uint32_t)want;
+    uint32_t* sel = scratch + EV_THREADS / 64 + 1;  // [0] = chosen bin, [1] = remaining after it
+#pragma unroll 1
+    for (int pass = 0; pass < 4; ++pass) {
+        const int shift = 24 - 8 * pass;
+        for (int b = threadIdx.x; b < 256; b += EV_THREADS) hist[b] = 0;
+        __syncthreads();
+        const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+        for (int i = threadIdx.x; i < n; i += EV_THREADS) {
+            const uint32_t key = keys[i];
+            if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        // thread t looks at bin 255-t: an inclusive scan walks the bins from the largest down
+        uint32_t cnt = threadIdx.x < 256 ? hist[255 - threadIdx.x] : 0u, tot;
+        const uint32_t incl = block_scan_inclusive<EV_THREADS>(cnt, scratch, &tot);
+        if (threadIdx.x < 256 && incl >= remaining && incl - cnt < remaining) {
+            sel[0] = 255u - threadIdx.x;
+            sel[1] = remaining - (incl - cnt);
+        }
+        __syncthreads();
+        prefix |= sel[0] << shift;
+        remaining = sel[1];
+        __syncthreads();
+    }
+    *take_eq = (int)remaining;
+    return prefix;
+}
+
+// ---- keep flags -> ascending list of kept source rows, written over keys[0..kept) ------------
+// keep(i) = key > thr  or  (key == thr and eq_base + (rank among equal keys before i) < take_eq).
+// Returns the number kept; *first_evicted = smallest i not kept (n if none).
+__device__ __forceinline__ int compact_indices(uint32_t* keys, int n, uint32_t thr, int take_eq, int eq_base,
+                                               uint32_t* scratch, int* first_evicted_lds) {
+    int gt_base = 0;
+    const int eq_kept0 = min(eq_base, take_eq);  // ties already granted to earlier segments of the group
+    if (threadIdx.x == 0) *first_evicted_lds = n;
+    __syncthreads();
+    for (int base = 0; base < n; base += EV_THREADS * EV_ITEMS) {
+        const int i0 = base + threadIdx.x * EV_ITEMS;
+        uint32_t k[EV_ITEMS];
+        uint32_t gt = 0, eq = 0;
+#pragma unroll
+        for (int j = 0; j < EV_ITEMS; ++j) {
+            k[j] = (i0 + j < n) ? keys[i0 + j] : 0u;
+            const bool valid = i0 + j < n;
+            gt += (valid && k[j] > thr) ? 1u : 0u;
+            eq += (valid && k[j] == thr) ? 1u : 0u;
+        }
+        uint32_t tot;
+        const uint32_t incl = block_scan_inclusive<EV_THREADS>(gt | (eq << 16), scratch, &tot);  // <= 1024 each
+        // (the scan's first barrier separates every thread's reads of this chunk from the writes below)
+        int gt_before = gt_base + (int)((incl & 0xffffu) - gt);
+        int eq_before = eq_base + (int)((incl >> 16) - eq);
+        int my_first_evicted = n;
+#pragma unroll
+        for (int j = 0; j < EV_ITEMS; ++j) {
+            if (i0 + j < n) {
+                const bool is_gt = k[j] > thr, is_eq = k[j] == thr;
+                const bool keep = is_gt || (is_eq && eq_before < take_eq);
+                if (keep) keys[gt_before + min(eq_before, take_eq) - eq_kept0] = (uint32_t)(i0 + j);
+                else my_first_evicted = min(my_first_evicted, i0 + j);
+                gt_before += is_gt ? 1 : 0;
+                eq_before += is_eq ? 1 : 0;
+            }
+        }
+        if (my_first_evicted < n) atomicMin(first_evicted_lds, my_first_evicted);
+        gt_base += (int)(tot & 0xffffu);
+        eq_base += (int)(tot >> 16);
+    }
+    __syncthreads();
+    return gt_base + min(eq_base, take_eq) - eq_kept0;
+}
+
+// A use the compiler cannot see through: the value must sit in its register here, so every load
+// that feeds it has completed (s_waitcnt) before execution moves on.
+__device__ __forceinline__ void land(uint4& v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+__device__ __forceinline__ void land(uint32_t& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void land(int64_t& v) { asm volatile("" : "+v"(v)); }
+
+// ---- move kept rows and metadata to the front of the segment, in place ----------------------
+// idx[r] (ascending, idx[r] >= r) is the source row of destination row r.  Tile t's destinations
+// [t*R, (t+1)*R) can only overlap sources of tiles <= t, so each tile is loaded whole, the
+// workgroup meets at a barrier with its loads complete, and only then is the tile stored.
+__device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg, int64_t* posseg, const uint32_t* idx,
+                                             int kept, int first_moved, int row_bytes, int lpr_shift, int lb_bytes) {
+    const int lpr = 1 << lpr_shift;
+    const int rpp = EV_THREADS >> lpr_shift;  // rows per pass
+    const int piece = threadIdx.x & (lpr - 1), rl = threadIdx.x >> lpr_shift;
+    const int tile_rows = rpp * EV_ROW_PASSES;
+    for (int base = (first_moved / tile_rows) * tile_rows; base < kept; base += tile_rows) {
+        uint4 kk[EV_ROW_PASSES], vv[EV_ROW_PASSES];
+        bool mv[EV_ROW_PASSES];
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) {
+            const int r = base + p * rpp + rl;
+            mv[p] = false;
+            kk[p] = make_uint4(0, 0, 0, 0);
+            vv[p] = make_uint4(0, 0, 0, 0);
+            if (r < kept) {
+                const int src = (int)idx[r];
+                if (src != r) {
+                    mv[p] = true;
+                    const int64_t o = (int64_t)src * row_bytes + (piece << 4);
+                    kk[p] = *(const uint4*)(kseg + o);
+                    vv[p] = *(const uint4*)(vseg + o);
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) { land(kk[p]); land(vv[p]); }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) {
+            if (mv[p]) {
+                const int r = base + p * rpp + rl;
+                const int64_t o = (int64_t)r * row_bytes + (piece << 4);
+                *(uint4*)(kseg + o) = kk[p];
+                *(uint4*)(vseg + o) = vv[p];
+            }
+        }
+    }
+    __syncthreads();
+    const int mtile = EV_THREADS * EV_ROW_PASSES;
+    for (int base = (first_moved / mtile) * mtile; base < kept; base += mtile) {
+        uint32_t lbv[EV_ROW_PASSES];
+        int64_t pv[EV_ROW_PASSES];
+        bool mv[EV_ROW_PASSES];
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) {
+            const int r = base + p * EV_THREADS + threadIdx.x;
+            mv[p] = false;
+            lbv[p] = 0;
+            pv[p] = 0;
+            if (r < kept) {
+                const int src = (int)idx[r];
+                if (src != r) {
+                    mv[p] = true;
+                    lbv[p] = lb_bytes == 4 ? ((const uint32_t*)lbseg)[src] : (uint32_t)((const uint16_t*)lbseg)[src];
+                    pv[p] = posseg[src];
+                }
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) { land(lbv[p]); land(pv[p]); }
+        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < EV_ROW_PASSES; ++p) {
+            if (mv[p]) {
+                const int r = base + p * EV_THREADS + threadIdx.x;
+                if (lb_bytes == 4) ((uint32_t*)lbseg)[r] = lbv[p];
+                else ((uint16_t*)lbseg)[r] = (uint16_t)lbv[p];
+                posseg[r] = pv[p];
+            }
+        }
+    }
+}
+
+struct EvictArgs {
+    char* k_slab; char* v_slab; char* lb_slab; int64_t* pos_slab; int32_t* seg_len;
+    int nseg, cap, row_bytes, lpr_shift, kv_dtype, lb_dtype;
+    int keep; const int32_t* keep_per_seg; int slack;
+    int64_t q_idx; int strategy, rounding, sliding_window;
+    int32_t* kept_idx; int kept_stride;
+    uint32_t* ws_keys; int ws_stride;  // used when the keys do not fit in LDS
+    // threshold mode (trimkv_compact_threshold)
+    const uint32_t* thr_key; const int32_t* tie_take; const int32_t* tie_base; int segs_per_group;
+};
+
+// SELECT = true: find the cut inside the segment (trimkv_evict).
+// SELECT = false: the cut comes from thr_key/tie_take/tie_base (trimkv_compact_threshold).
+template <bool LDS_KEYS, bool SELECT>
+__global__ __launch_bounds__(EV_THREADS) void evict_kernel(EvictArgs a) {
+    extern __shared__ uint32_t lds_keys[];
+    __shared__ uint32_t hist[256];
+    __shared__ uint32_t scratch[EV_THREADS / 64 + 4];
+    __shared__ int first_evicted;
+
+    const int seg = blockIdx.x;
+    const int n = a.seg_len[seg];
+    if (n <= 0 || n > a.cap) return;  // nothing cached, or a corrupt length: touch nothing
+    int want = 0;
+    if (SELECT) {
+        want = a.keep_per_seg ? a.keep_per_seg[seg] : a.keep;
+        if (want < 0) want = 0;
+        if (n <= want || n < want + a.slack) return;  // uniform across the workgroup
+    }
+    uint32_t* keys = LDS_KEYS ? lds_keys : a.ws_keys + (int64_t)seg * a.ws_stride;
+
+    const int lb_bytes = a.lb_dtype == TRIMKV_F32 ? 4 : 2;
+    char* kseg = a.k_slab + (int64_t)seg * a.cap * a.row_bytes;
+    char* vseg = a.v_slab + (int64_t)seg * a.cap * a.row_bytes;
+    char* lbseg = a.lb_slab + (int64_t)seg * a.cap * lb_bytes;
+    int64_t* posseg = a.pos_slab + (int64_t)seg * a.cap;
+
+    ScoreArgs s;
+    s.lb = lbseg; s.pos = posseg; s.k = kseg; s.lb_dtype = a.lb_dtype; s.kv_dtype = a.kv_dtype; s.row_bytes = a.row_bytes;
+    s.strategy = a.strategy; s.rounding = a.rounding; s.sliding_window = a.sliding_window; s.q_idx = a.q_idx;
+    for (int i = threadIdx.x; i < n; i += EV_THREADS) keys[i] = score_key(s, i, n);
+    __syncthreads();
+
+    uint32_t thr;
+    int take_eq, eq_base = 0;
+    if (SELECT) {
+        thr = radix_select(keys, n, want, hist, scratch, &take_eq);
+    } else {
+        const int g = seg / a.segs_per_group;
+        thr = a.thr_key[g];
+        take_eq = a.tie_take[g];
+        eq_base = a.tie_base[seg];
+    }
+    const int kept = compact_indices(keys, n, thr, take_eq, eq_base, scratch, &first_evicted);
+    const int first_moved = first_evicted;
+    if (a.kept_idx) {
+        for (int r = threadIdx.x; r < kept && r < a.kept_stride; r += EV_THREADS)
+            a.kept_idx[(int64_t)seg * a.kept_stride + r] = (int32_t)keys[r];
+    }
+    if (first_moved < kept)
+        move_segment(kseg, vseg, lbseg, posseg, keys, kept, first_moved, a.row_bytes, a.lpr_shift, lb_bytes);
+    if (threadIdx.x == 0) a.seg_len[seg] = kept;
+}
+
+// ---- shared-budget selection over groups of segments ----------------------------------------
+struct GroupArgs {
+    const void* const* lb_slabs; const int64_t* const* pos_slabs; const void* const* k_slabs; const int32_t* const* seg_lens;
+    int nlayers, nseg, segs_per_group, cap, row_bytes, kv_dtype, lb_dtype;
+    int64_t budget; int use_threshold; float threshold_score;
+    int64_t q_idx; int strategy, rounding;
+    uint32_t* thr_key; int32_t* tie_take; int32_t* tie_base; int32_t* new_len;
+};
+
+__device__ __forceinline__ ScoreArgs group_segment(const GroupArgs& a, int layer, int seg) {
+    const int lb_bytes = a.lb_dtype == TRIMKV_F32 ? 4 : 2;
+    ScoreArgs s;
+    s.lb = (const char*)a.lb_slabs[layer] + (int64_t)seg * a.cap * lb_bytes;
+    s.pos = a.pos_slabs[layer] + (int64_t)seg * a.cap;
+    s.k = a.k_slabs ? (const char*)a.k_slabs[layer] + (int64_t)seg * a.cap * a.row_bytes : nullptr;
+    s.lb_dtype = a.lb_dtype; s.kv_dtype = a.kv_dtype; s.row_bytes = a.row_bytes;
+    s.strategy = a.strategy; s.rounding = a.rounding; s.sliding_window = 0; s.q_idx = a.q_idx;
+    return s;
+}
+
+__device__ __forceinline__ uint64_t block_sum_u64(uint64_t v, uint64_t* scratch) {
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_down(v, d, 64);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();
+    if (lane == 0) scratch[wave] = v;
+    __syncthreads();
+    uint64_t t = 0;
+    for (int w = 0; w < GT_THREADS / 64; ++w) t += scratch[w];
+    return t;
+}
+
+__global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a) {
+    __shared__ unsigned long long hist[256];
+    __shared__ uint64_t red[GT_THREADS / 64];
+    __shared__ unsigned long long sel[2];
+    const int g = blockIdx.x;
+    const int seg0 = g * a.segs_per_group;
+
+    uint32_t thr;
+    int64_t take;
+    if (a.use_threshold) {
+        thr = float_key(a.threshold_score);
+        take = INT32_MAX;  // every token equal to the threshold passes (score >= threshold)
+    } else {
+        uint64_t total = 0;
+        for (int l = 0; l < a.nlayers; ++l)
+            for (int s = 0; s < a.segs_per_group; ++s) total += (uint64_t)max(0, min(a.seg_lens[l][seg0 + s], a.cap));
+        uint64_t remaining = (uint64_t)max((int64_t)0, a.budget);
+        if (remaining >= total) {  // the budget covers everything: keep all
+            thr = 0u;
+            take = INT32_MAX;
+        } else if (remaining == 0) {
+            thr = 0xffffffffu;
+            take = 0;
+        } else {
+            uint32_t prefix = 0;
+            for (int pass = 0; pass < 4; ++pass) {
+                const int shift = 24 - 8 * pass;
+                const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+                for (int b = threadIdx.x; b < 256; b += GT_THREADS) hist[b] = 0ull;
+                __syncthreads();
+                for (int l = 0; l < a.nlayers; ++l)
+                    for (int s = 0; s < a.segs_per_group; ++s) {
+                        const int n = max(0, min(a.seg_lens[l][seg0 + s], a.cap));
+                        const ScoreArgs sa = group_segment(a, l, seg0 + s);
+                        for (int i = threadIdx.x; i < n; i += GT_THREADS) {
+                            const uint32_t key = score_key(sa, i, n);
+                            if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1ull);
+                        }
+                    }
+                __syncthreads();
+                if (threadIdx.x == 0) {  // 256 bins, walked from the largest down
+                    uint64_t acc = 0;
+                    int b = 255;
+                    for (; b > 0; --b) {
+                        if (acc + hist[b] >= remaining) break;
+                        acc += hist[b];
+                    }
+                    sel[0] = (unsigned long long)b;
+                    sel[1] = remaining - acc;
+                }
+                __syncthreads();
+                prefix |= (uint32_t)sel[0] << shift;
+                remaining = sel[1];
+                __syncthreads();
+            }
+            thr = prefix;
+            take = (int64_t)remaining;
+        }
+    }
+    // per-segment kept counts and tie bookkeeping, in (layer, segment) order
+    int64_t eq_seen = 0;
+    for (int l = 0; l < a.nlayers; ++l)
+        for (int s = 0; s < a.segs_per_group; ++s) {
+            const int n = max(0, min(a.seg_lens[l][seg0 + s], a.cap));
+            const ScoreArgs sa = group_segment(a, l, seg0 + s);
+            uint64_t cnt = 0;  // low 32 bits: greater, high 32 bits: equal
+            for (int i = threadIdx.x; i < n; i += GT_THREADS) {
+                const uint32_t key = score_key(sa, i, n);
+                cnt += (key > thr ? 1ull : 0ull) + (key == thr ? (1ull << 32) : 0ull);
+            }
+            cnt = block_sum_u64(cnt, red);
+            const int64_t gt = (int64_t)(cnt & 0xffffffffull), eq = (int64_t)(cnt >> 32);
+            const int64_t eq_kept = max((int64_t)0, min(eq, take - eq_seen));
+            if (threadIdx.x == 0) {
+                a.new_len[(int64_t)l * a.nseg + seg0 + s] = (int32_t)(gt + eq_kept);
+                a.tie_base[(int64_t)l * a.nseg + seg0 + s] = (int32_t)min(eq_seen, (int64_t)INT32_MAX);
+            }
+            eq_seen += eq;
+        }
+    if (threadIdx.x == 0) {
+        a.thr_key[g] = thr;
+        a.tie_take[g] = (int32_t)min(take, (int64_t)INT32_MAX);
+    }
+}
+
+__global__ void cu_seqlens_kernel(const int32_t* seg_len, int nseg, int32_t* cu) {
+    __shared__ uint32_t scratch[1024 / 64 + 1];
+    int32_t running = 0;
+    if (threadIdx.x == 0) cu[0] = 0;
+    for (int base = 0; base < nseg; base += 1024) {
+        const int i = base + threadIdx.x;
+        uint32_t tot;
+        const uint32_t incl = block_scan_inclusive<1024>(i < nseg ? (uint32_t)max(seg_len[i], 0) : 0u, scratch, &tot);
+        if (i < nseg) cu[i + 1] = running + (int32_t)incl;
+        running += (int32_t)tot;
+        __syncthreads();
+    }
+}
+
+static int lpr_shift_of(int row_bytes) {
+    const int lpr = row_bytes / 16;
+    if (row_bytes % 16 || lpr <= 0 || (lpr & (lpr - 1)) || lpr > 64) return -1;
+    int s = 0;
+    while ((1 << s) < lpr) ++s;
+    return s;
+}
+
+template <bool SELECT>
+static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st) {
+    const size_t key_bytes = (size_t)max_len * 4;
+    if (key_bytes <= (size_t)EV_LDS_KEY_BYTES) {
+        static bool attr_set = false;
+        if (!attr_set) {  // allow more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per workgroup)
+            hipError_t e = hipFuncSetAttribute((const void*)evict_kernel<true, SELECT>, hipFuncAttributeMaxDynamicSharedMemorySize, EV_LDS_KEY_BYTES);
+            if (e != hipSuccess) return fail((int)e, "%s: hipFuncSetAttribute: %s", fn, hipGetErrorString(e));
+            attr_set = true;
+        }
+        hipLaunchKernelGGL((evict_kernel<true, SELECT>), dim3(a.nseg), dim3(EV_THREADS), key_bytes, st, a);
+    } else {
+        const size_t need = (size_t)a.nseg * max_len * 4;
+        if (!workspace || workspace_bytes < need)
+            return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed for max_len=%d, got %zu", fn, need, max_len, workspace_bytes);
+        a.ws_keys = (uint32_t*)workspace;
+        a.ws_stride = max_len;
+        hipLaunchKernelGGL((evict_kernel<false, SELECT>), dim3(a.nseg), dim3(EV_THREADS), 0, st, a);
+    }
+    return launch_status(fn);
+}
+
+}  // namespace trimkv
+
+using namespace trimkv;
+
+extern "C" size_t trimkv_evict_workspace(int nseg, int max_len) {
+    if (nseg <= 0 || max_len <= 0) return 0;
+    if ((size_t)max_len * 4 <= (size_t)EV_LDS_KEY_BYTES) return 0;
+    return (size_t)nseg * max_len * 4;
+}
+
+static int check_slab_args(const char* fn, const void* k, const void* v, const void* lb, const void* pos, const void* len,
+                           int nseg, int cap, int head_dim, int kv_dtype, int lb_dtype, int max_len, int* lpr_shift) {
+    if (!k || !v || !lb || !pos || !len) return fail(TRIMKV_ERR_NULL, "%s: null slab pointer", fn);
+    if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0)
+        return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
+    if (nseg <= 0 || cap <= 0 || head_dim <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d head_dim=%d max_len=%d", fn, nseg, cap, head_dim, max_len);
+    if (max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
+    *lpr_shift = lpr_shift_of(head_dim * 2);
+    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be 16 * a power of two <= 1024 (head_dim=%d)", fn, head_dim);
+    if (((uintptr_t)k & 15) || ((uintptr_t)v & 15)) return fail(TRIMKV_ERR_SHAPE, "%s: slabs must be 16-byte aligned", fn);
+    return TRIMKV_OK;
+}
+
+extern "C" int trimkv_evict(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                            int nseg, int cap, int head_dim, int kv_dtype, int lb_dtype,
+                            int keep, const int32_t* keep_per_seg, int slack,
+                            int64_t q_idx, int strategy, int rounding, int sliding_window, int max_len,
+                            int32_t* kept_idx, int kept_stride,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_evict";
+    int lpr_shift;
+    int rc = check_slab_args(fn, k_slab, v_slab, lb_slab, pos_slab, seg_len, nseg, cap, head_dim, kv_dtype, lb_dtype, max_len, &lpr_shift);
+    if (rc) return rc;
+    if (!keep_per_seg && keep < 0) return fail(TRIMKV_ERR_SHAPE, "%s: keep=%d", fn, keep);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    if (rounding != TRIMKV_ROUND_UPCAST && rounding != TRIMKV_ROUND_NATIVE) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown rounding %d", fn, rounding);
+    if (kept_idx && kept_stride <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: kept_stride=%d", fn, kept_stride);
+    EvictArgs a = {};
+    a.k_slab = (char*)k_slab; a.v_slab = (char*)v_slab; a.lb_slab = (char*)lb_slab; a.pos_slab = pos_slab; a.seg_len = seg_len;
+    a.nseg = nseg; a.cap = cap; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
+    a.keep = keep; a.keep_per_seg = keep_per_seg; a.slack = slack < 0 ? 0 : slack;
+    a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding; a.sliding_window = sliding_window < 0 ? 0 : sliding_window;
+    a.kept_idx = kept_idx; a.kept_stride = kept_stride; a.segs_per_group = 1;
+    return launch_evict<true>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int trimkv_compact_threshold(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len,
+                                        int nseg, int segs_per_group, int cap, int head_dim, int kv_dtype, int lb_dtype,
+                                        const uint32_t* thr_key, const int32_t* tie_take, const int32_t* tie_base,
+                                        int64_t q_idx, int strategy, int rounding, int max_len,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_compact_threshold";
+    int lpr_shift;
+    int rc = check_slab_args(fn, k_slab, v_slab, lb_slab, pos_slab, seg_len, nseg, cap, head_dim, kv_dtype, lb_dtype, max_len, &lpr_shift);
+    if (rc) return rc;
+    if (!thr_key || !tie_take || !tie_base) return fail(TRIMKV_ERR_NULL, "%s: null threshold pointer", fn);
+    if (segs_per_group <= 0 || nseg % segs_per_group) return fail(TRIMKV_ERR_SHAPE, "%s: segs_per_group=%d does not divide nseg=%d", fn, segs_per_group, nseg);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    EvictArgs a = {};
+    a.k_slab = (char*)k_slab; a.v_slab = (char*)v_slab; a.lb_slab = (char*)lb_slab; a.pos_slab = pos_slab; a.seg_len = seg_len;
+    a.nseg = nseg; a.cap = cap; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
+    a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding; a.sliding_window = 0;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.segs_per_group = segs_per_group;
+    return launch_evict<false>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+                                      const void* const* k_slabs, const int32_t* const* seg_lens,
+                                      int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
+                                      int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
+                                      int64_t q_idx, int strategy, int rounding,
+                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                      void* stream) {
+    const char* fn = "trimkv_group_threshold";
+    if (!lb_slabs || !pos_slabs || !seg_lens || !thr_key || !tie_take || !tie_base || !new_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if (strategy == TRIMKV_SCORE_KNORM_ALPHA && !k_slabs) return fail(TRIMKV_ERR_NULL, "%s: knorm_alpha needs k_slabs", fn);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0) return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
+    if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0 || nseg % segs_per_group || cap <= 0 || head_dim <= 0)
+        return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d segs_per_group=%d cap=%d head_dim=%d", fn, nlayers, nseg, segs_per_group, cap, head_dim);
+    GroupArgs a;
+    a.lb_slabs = lb_slabs; a.pos_slabs = pos_slabs; a.k_slabs = strategy == TRIMKV_SCORE_KNORM_ALPHA ? k_slabs : nullptr; a.seg_lens = seg_lens;
+    a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
+    a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
+    a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len;
+    hipLaunchKernelGGL(group_threshold_kernel, dim3(nseg / segs_per_group), dim3(GT_THREADS), 0, (hipStream_t)stream, a);
+    return launch_status(fn);
+}
+
+extern "C" int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlens, void* stream) {
+    if (!seg_len || !cu_seqlens) return fail(TRIMKV_ERR_NULL, "trimkv_build_cu_seqlens: null pointer argument");
+    if (nseg <= 0) return fail(TRIMKV_ERR_SHAPE, "trimkv_build_cu_seqlens: nseg=%d", nseg);
+    hipLaunchKernelGGL(cu_seqlens_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seg_len, nseg, cu_seqlens);
+    return launch_status("trimkv_build_cu_seqlens");
+}
