@@ -192,7 +192,9 @@ int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlen
  *
  * q and out are [nseg*group][head_dim], contiguous, kv dtype -- i.e. [B][Hq][1][D] and
  * [B][1][Hq][D].  Segment rows start at seg_start[seg] (int32 row offsets, e.g. cu_seqlens_k)
- * or, when seg_start is NULL, at seg*cap.  A segment of length 0 yields zeros.
+ * or, when seg_start is NULL, at seg*cap.  seg_len may be NULL: every segment then holds max_len
+ * rows (a dense cache).  max_len is the caller's upper bound on seg_len (longer segments are
+ * truncated to it).  A segment of length 0 yields zeros.
  * Split-K: every segment is cut into chunks of `chunk` rows (0 = chosen from nseg/max_len);
  * partial (max, sum, accumulator) triples go through `workspace`
  * (trimkv_decode_attn_workspace bytes) and are merged by a second kernel.

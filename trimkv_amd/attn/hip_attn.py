@@ -1,0 +1,159 @@
+"""Attention over the retained KV on the HIP kernels of libtrimkv_hip.so.
+
+Three callables with the reference's attention-interface signature
+(``fn(module, query, key, value, attention_mask, scaling=..., flash_attn_kwargs=..., **kw)
+-> (out [B,Q,Hq,D], None, None)``, src/trimkv/attn/flash_attn.py:10-20, 79-89):
+
+* ``dense_attention_forward`` -- K/V ``[B,Hkv,n,D]`` (views of a dense cache's slabs, or any tensors)
+* ``batched_dynamic_kv_budget_attention_forward`` / ``dynamic_kv_budget_attention_forward`` --
+  K/V flat ``[rows, D]`` with ``head_lens`` / ``cu_seqlens_k`` (and ``seg_start`` when the rows
+  are a ragged cache's slabs) in ``flash_attn_kwargs``; segment ``b*Hkv+h`` is attended by query
+  heads ``h*G .. h*G+G-1`` of batch element ``b`` (flash_attn.py:120-125, 147-149).
+
+Q_LEN == 1 runs ``trimkv_decode_attn``.  Longer query blocks (prompt chunks) are computed with
+torch ops on the same device until the chunk-prefill kernel exists.  As in the reference the
+ragged entry points ignore ``attention_mask`` and ``scaling`` (flash_attn.py:15, 85; the scale is
+``D**-0.5``) and apply a bottom-right causal mask when Q_LEN > 1.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional, Tuple
+
+import torch
+from torch import nn
+
+from .. import _lib
+
+_WS: Dict[Tuple[str, int], torch.Tensor] = {}
+
+
+def _workspace(device, nbytes: int) -> Optional[torch.Tensor]:
+    if nbytes <= 0:
+        return None
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    ws = _WS.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        _WS[key] = ws
+    return ws
+
+
+def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, nseg: int, group: int,
+                     seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
+                     scale: float, chunk: int = 0) -> torch.Tensor:
+    """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``."""
+    if not query.is_cuda:
+        raise _lib.TrimKVLibraryError("decode attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
+    lib = _lib.load()
+    d = query.shape[-1]
+    out = torch.empty_like(query)
+    ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, max_len, chunk)
+    ws = _workspace(query.device, ws_bytes)
+    rc = lib.trimkv_decode_attn(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(),
+                                _lib.ptr(seg_len), _lib.ptr(seg_start), nseg, cap, d, group, _lib.dtype_code(query.dtype),
+                                float(scale), max_len, chunk, _lib.ptr(ws), 0 if ws is None else ws.numel(),
+                                _lib.current_stream(query.device))
+    _lib.check(rc, "trimkv_decode_attn")
+    return out
+
+
+def _causal_bottom_right(qlen: int, n: int, device) -> torch.Tensor:
+    t = torch.arange(qlen, device=device)[:, None]
+    j = torch.arange(n, device=device)[None, :]
+    return j <= (n - qlen + t)
+
+
+def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                            attention_mask: Optional[torch.Tensor] = None, scaling: Optional[float] = None,
+                            dropout: float = 0.0, flash_attn_kwargs: Optional[dict] = None, **kwargs):
+    """Dense-cache attention.  query [B,Hq,Q,D], key/value [B,Hkv,n,D] -> ([B,Q,Hq,D], None, None)."""
+    B, Hq, Q, D = query.shape
+    Hkv, n = key.shape[1], key.shape[2]
+    G = Hq // Hkv
+    scale = D ** -0.5 if scaling is None else scaling
+    if Q == 1 and attention_mask is None:
+        ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
+              and value.stride() == key.stride() and key.stride(1) % D == 0)
+        if not ok:
+            key, value = key.contiguous(), value.contiguous()
+        cap = key.stride(1) // D
+        q2 = query.reshape(B * Hq, D)
+        if not q2.is_contiguous():
+            q2 = q2.contiguous()
+        seg_len = (flash_attn_kwargs or {}).get("seg_len")
+        if seg_len is not None and (seg_len.numel() != B * Hkv or (flash_attn_kwargs or {}).get("max_len") != n):
+            seg_len = None
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale)
+        return out.view(B, 1, Hq, D), None, None
+    # prompt chunks and masked batches: torch ops (bottom-right causal, as flash-attn aligns it)
+    k = key.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
+    v = value.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
+    w = torch.matmul(query, k.transpose(2, 3)).float() * scale
+    if attention_mask is not None:
+        w = w + attention_mask[:, :, :, :n].float()
+    elif Q > 1:
+        w = w.masked_fill(~_causal_bottom_right(Q, n, query.device), float("-inf"))
+    w = torch.softmax(w, dim=-1).to(query.dtype)
+    return torch.matmul(w, v).transpose(1, 2).contiguous(), None, None
+
+
+def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_heads):
+    kw = flash_attn_kwargs or {}
+    head_lens, cu = kw.get("head_lens"), kw.get("cu_seqlens_k")
+    if head_lens is None or cu is None:
+        raise ValueError("flash_attn_kwargs must carry head_lens and cu_seqlens_k")
+    B, Hq, Q, D = query.shape
+    nseg = head_lens.shape[0]
+    if batch_size is None:
+        batch_size = B
+    if num_kv_heads is None:
+        num_kv_heads = nseg // batch_size
+    G = Hq // num_kv_heads
+    seg_start = kw.get("seg_start")
+    if seg_start is None:  # packed rows, as the reference stores them
+        seg_start = cu[:-1]
+        if not seg_start.is_contiguous():
+            seg_start = seg_start.contiguous()
+        max_len = kw.get("max_len")
+        if max_len is None:
+            max_len = int(head_lens.max().item())  # the reference synchronises here as well (flash_attn.py:58, 133)
+        cap = max_len
+    else:
+        max_len, cap = kw["max_len"], kw["seg_cap"]
+    if Q == 1:
+        q2 = query.reshape(B * Hq, D)  # [B,Hq,1,D]: row seg*G+g is query head h*G+g of batch b
+        if not q2.is_contiguous():
+            q2 = q2.contiguous()
+        out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5)
+        return out.view(B, 1, Hq, D), None, None
+    # prompt chunks: per-segment torch ops with the bottom-right causal mask of flash-attn's causal=True
+    out = torch.zeros(B, Q, Hq, D, dtype=query.dtype, device=query.device)
+    starts = seg_start.tolist()
+    lens = head_lens.tolist()
+    for seg in range(nseg):
+        b, h = divmod(seg, num_kv_heads)
+        n = lens[seg]
+        if n == 0:
+            continue
+        k = key[starts[seg]:starts[seg] + n].float()
+        v = value[starts[seg]:starts[seg] + n].float()
+        qs = query[b, h * G:(h + 1) * G].float()
+        s = torch.einsum("gqd,nd->gqn", qs, k) * (D ** -0.5)
+        s = s.masked_fill(~_causal_bottom_right(Q, n, query.device), float("-inf"))
+        p = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
+        out[b, :, h * G:(h + 1) * G] = torch.einsum("gqn,nd->qgd", p, v).to(query.dtype)
+    return out, None, None
+
+
+def batched_dynamic_kv_budget_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                                attention_mask: Optional[torch.Tensor] = None, scaling: float = None,
+                                                dropout_p: float = 0.0, flash_attn_kwargs: dict = {}, **kwargs):
+    kw = flash_attn_kwargs or {}
+    return _ragged_common(query, key, value, kw, kw.get("batch_size"), kw.get("num_kv_heads"))
+
+
+def dynamic_kv_budget_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                        attention_mask: Optional[torch.Tensor] = None, scaling: float = None,
+                                        dropout_p: float = 0.0, flash_attn_kwargs: dict = {}, **kwargs):
+    assert query.shape[0] == 1, "Batch size greater than 1 not supported in dynamic KV budget attention."
+    return _ragged_common(query, key, value, flash_attn_kwargs, 1, None)

@@ -1,0 +1,818 @@
+"""TRIM-KV caches on MI355X: same classes, signatures and results as the reference's
+``src/trimkv/cache_utils.py``, backed by capacity slabs in HBM and the HIP kernels of
+``libtrimkv_hip.so``.
+
+Storage.  Every layer owns four slabs shared by its ``nseg = B * Hkv`` segments::
+
+    K, V   [nseg, cap, D]  bf16/fp16      log beta [nseg, cap]      positions [nseg, cap] int64
+    seg_len [nseg] int32 (device)
+
+``update`` writes only the new rows (``trimkv_append``), ``compress`` selects and compacts in
+place (``trimkv_evict`` / ``trimkv_group_threshold`` + ``trimkv_compact_threshold``): nothing is
+re-allocated or re-packed per step, which is where the reference spends its bandwidth
+(``torch.cat`` at cache_utils.py:104-107, four Triton re-packs at :646-676).  Tensors handed out
+are views of the slabs: valid until the next ``update``/``compress`` of that layer.
+
+There is no CPU path: tensors must live on the GPU and the library must be built.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Dict, Iterable, List, Optional, Tuple
+
+import numpy as np
+import torch
+
+from . import _lib
+
+try:  # the reference subclasses HF's DynamicCache so that isinstance(x, Cache) holds (cache_utils.py:8-11)
+    from transformers.cache_utils import DynamicCache as _CacheBase
+except Exception:  # pragma: no cover - transformers is optional for the cache itself
+    class _CacheBase:  # type: ignore
+        def __init__(self, *a, **k) -> None:
+            pass
+
+__all__ = ["TrimKVCache", "DynamicBudgetTrimKVCache", "BatchedDynamicBudgetTrimKVCache", "LazyLogBeta"]
+
+_EMPTY = lambda: torch.tensor([])  # what the reference stores for a skipped layer (cache_utils.py:84-87)
+
+
+class LazyLogBeta:
+    """log(beta) that has not been finished yet: per-slice partial sums of the `rg` gate's second
+    linear plus its bias.  ``update`` hands it to ``trimkv_append_gated`` so that the sum, the
+    bias, the logsigmoid and the write into the slab happen in the append kernel.  It quacks like
+    the ``[B, S, Hkv]`` tensor the gate would return where the caller only transposes it
+    (modeling_trimkv_qwen3.py:333)."""
+
+    def __init__(self, part: torch.Tensor, bias_f32: torch.Tensor, batch: int, seq: int, heads: int, dtype, transposed=False):
+        self.part, self.bias_f32 = part, bias_f32
+        self.batch, self.seq, self.heads, self.dtype, self.transposed = batch, seq, heads, dtype, transposed
+
+    @property
+    def shape(self):
+        return (self.batch, self.heads, self.seq) if self.transposed else (self.batch, self.seq, self.heads)
+
+    def dim(self) -> int:
+        return 3
+
+    def transpose(self, a: int, b: int) -> "LazyLogBeta":
+        if {a % 3, b % 3} != {1, 2}:
+            raise ValueError("LazyLogBeta only supports transpose(1, 2)")
+        return LazyLogBeta(self.part, self.bias_f32, self.batch, self.seq, self.heads, self.dtype, not self.transposed)
+
+    def materialize(self) -> torch.Tensor:
+        """The finished tensor, computed with torch ops (for callers that need the values)."""
+        acc = self.part.sum(dim=0).view(self.batch, self.seq, self.heads)
+        if self.dtype != torch.float32:
+            acc = acc.to(self.dtype).float()
+            acc = (acc + self.bias_f32).to(self.dtype).float()
+        else:
+            acc = acc + self.bias_f32
+        out = torch.nn.functional.logsigmoid(acc).to(self.dtype)
+        return out.transpose(1, 2) if self.transposed else out
+
+
+class _Slab:
+    """Device storage of one layer."""
+
+    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len")
+
+    def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
+        nseg = B * H
+        self.B, self.H, self.D, self.cap = B, H, D, cap
+        self.k = torch.empty(nseg, cap, D, dtype=kv_dtype, device=device)
+        self.v = torch.empty(nseg, cap, D, dtype=kv_dtype, device=device)
+        self.lb = torch.empty(nseg, cap, dtype=lb_dtype, device=device)
+        self.pos = torch.empty(nseg, cap, dtype=torch.int64, device=device)
+        self.seg_len = torch.zeros(nseg, dtype=torch.int32, device=device)
+        self.cu = torch.zeros(nseg + 1, dtype=torch.int32, device=device) if ragged else None
+        self.lens = np.zeros(nseg, dtype=np.int64)  # exact host mirror of seg_len
+        self.max_len = 0
+
+    @property
+    def nseg(self) -> int:
+        return self.B * self.H
+
+    def regrow(self, new_cap: int) -> None:
+        """Move to slabs of another capacity (rare: first right-sizing, or an unbounded cache)."""
+        keep = min(self.max_len, new_cap)
+        for name in ("k", "v", "lb", "pos"):
+            old = getattr(self, name)
+            new = torch.empty((old.shape[0], new_cap) + tuple(old.shape[2:]), dtype=old.dtype, device=old.device)
+            if keep:
+                new[:, :keep] = old[:, :keep]
+            setattr(self, name, new)
+        self.cap = new_cap
+
+
+def _require_cuda(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise _lib.TrimKVLibraryError(
+            f"{what} is on {t.device}: this cache runs on the GPU through libtrimkv_hip.so only (no CPU path)")
+
+
+class _SlabBacked(_CacheBase):
+    """What the three cache classes share: slabs, append, bookkeeping."""
+
+    _ragged = False
+
+    def __init__(self, max_seq_len: int = 20480, _distributed_cache_data: Iterable = None, device: str = "cuda") -> None:
+        try:
+            super().__init__()
+        except Exception:  # a DynamicCache whose constructor wants a config: the base is only a marker here
+            pass
+        if _distributed_cache_data is not None:
+            raise NotImplementedError(f"Distributed cache data is not supported for {type(self).__name__}")
+        self.max_seq_len = max_seq_len
+        self._seen_tokens = 0
+        self._slabs: List[Optional[_Slab]] = []
+        self.n_seen_tokens: List[int] = []
+        self.device = device
+        self.offset = torch.tensor(0, dtype=torch.int64)
+        self.block_mask = None
+        self.sliding_window_size = 0
+        self._budget_hint: Optional[int] = None  # memory_size + buffer_size of the last compress()
+        self._ws: Dict[Any, torch.Tensor] = {}
+
+    # ---- storage helpers -------------------------------------------------------------------
+    def _workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
+        if nbytes <= 0:
+            return None
+        key = ("evict", str(device))
+        ws = self._ws.get(key)
+        if ws is None or ws.numel() < nbytes:
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+            self._ws[key] = ws
+        return ws
+
+    def _new_capacity(self, slab: Optional[_Slab], need: int, s_new: int) -> int:
+        if self._budget_hint is not None and need <= self._budget_hint:
+            return self._budget_hint
+        if slab is None:
+            return need + max(128, need // 8)
+        return max(need + max(128, s_new), int(slab.cap * 1.5))
+
+    def _append(self, layer: int, k, v, lb, pos) -> _Slab:
+        B, H, S, D = k.shape
+        _require_cuda(k, "key_states")
+        slab = self._slabs[layer]
+        lazy = isinstance(lb, LazyLogBeta)
+        lb_dtype = lb.dtype
+        if slab is None:
+            slab = _Slab(B, H, D, self._new_capacity(None, S, S), k.dtype, lb_dtype, k.device, self._ragged)
+            self._slabs[layer] = slab
+        else:
+            if (B, H, D) != (slab.B, slab.H, slab.D):
+                raise ValueError(f"layer {layer}: got K of shape {tuple(k.shape)}, cache holds B={slab.B} Hkv={slab.H} D={slab.D}")
+            if slab.max_len + S > slab.cap:
+                slab.regrow(self._new_capacity(slab, slab.max_len + S, S))
+        if v.shape != k.shape or v.dtype != k.dtype:
+            raise ValueError("value_states must match key_states in shape and dtype")
+        if k.stride(3) != 1 or (k.stride(0) * 2) % 16 or (k.stride(1) * 2) % 16 or (k.stride(2) * 2) % 16 or k.data_ptr() % 16:
+            k = k.contiguous()
+        if v.stride() != k.stride() or v.data_ptr() % 16:
+            v = v.contiguous()
+            if v.stride() != k.stride():
+                k = k.contiguous()
+        if pos.dtype != torch.int64:
+            pos = pos.to(torch.int64)
+        if pos.device != k.device:
+            pos = pos.to(k.device)
+        if pos.dim() == 1:
+            ps = (0, 0, pos.stride(0))
+        else:
+            if tuple(pos.shape) != (B, H, S):
+                raise ValueError(f"cache_positions must be [S] or [B,Hkv,S], got {tuple(pos.shape)}")
+            ps = pos.stride()
+        lib = _lib.load()
+        st = _lib.current_stream(k.device)
+        common = (slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                  _lib.ptr(slab.cu), slab.nseg, H, slab.cap, D, _lib.dtype_code(k.dtype), _lib.dtype_code(slab.lb.dtype),
+                  k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2))
+        if lazy:
+            if not lb.transposed or lb.shape != (B, H, S):
+                raise ValueError("a lazy log-beta must be the [B,Hkv,S] transpose of the gate output")
+            rc = lib.trimkv_append_gated(*common, lb.part.data_ptr(), lb.part.shape[0], lb.bias_f32.data_ptr(),
+                                         pos.data_ptr(), ps[0], ps[1], ps[2], S, slab.max_len + S, st)
+            _lib.check(rc, "trimkv_append_gated")
+        else:
+            _require_cuda(lb, "retention_weights")
+            if tuple(lb.shape) != (B, H, S):
+                raise ValueError(f"retention_weights must be [B,Hkv,S], got {tuple(lb.shape)}")
+            if lb.dtype != slab.lb.dtype:
+                lb = lb.to(slab.lb.dtype)
+            rc = lib.trimkv_append(*common, lb.data_ptr(), lb.stride(0), lb.stride(1), lb.stride(2),
+                                   pos.data_ptr(), ps[0], ps[1], ps[2], S, slab.max_len + S, st)
+            _lib.check(rc, "trimkv_append")
+        slab.lens += S
+        slab.max_len += S
+        return slab
+
+    def _ensure_layer(self, layer: int) -> None:
+        while len(self._slabs) <= layer:
+            self._slabs.append(None)
+            self.n_seen_tokens.append(0)
+
+    # ---- bookkeeping shared by all three classes (cache_utils.py:35-54) ---------------------
+    def __len__(self) -> int:
+        return len(self._slabs)
+
+    def get_seq_length(self, layer_idx: Optional[int] = None) -> int:
+        """Tokens SEEN: in total when ``layer_idx`` is None, else by that layer (cache_utils.py:48-54)."""
+        if layer_idx is None:
+            return self._seen_tokens
+        return self.n_seen_tokens[layer_idx] if layer_idx < len(self.n_seen_tokens) else 0
+
+    def memory_bytes(self) -> int:
+        """Bytes of HBM held by the slabs (no reference counterpart)."""
+        tot = 0
+        for s in self._slabs:
+            if s is not None:
+                tot += sum(t.numel() * t.element_size() for t in (s.k, s.v, s.lb, s.pos))
+        return tot
+
+
+class _DenseViews:
+    """List-like ``cache.key_cache`` etc.: item ``l`` is the live ``[B,Hkv,n,...]`` view of layer l."""
+
+    def __init__(self, cache: "TrimKVCache", which: str):
+        self._c, self._w = cache, which
+
+    def __len__(self) -> int:
+        return len(self._c._slabs)
+
+    def __getitem__(self, layer: int) -> torch.Tensor:
+        if isinstance(layer, slice):
+            return [self[i] for i in range(*layer.indices(len(self)))]
+        if layer < 0:
+            layer += len(self)
+        s = self._c._slabs[layer]
+        if s is None:
+            return _EMPTY()
+        n = s.max_len
+        t = getattr(s, self._w)
+        if self._w in ("k", "v"):
+            return t.view(s.B, s.H, s.cap, s.D)[:, :, :n]
+        return t.view(s.B, s.H, s.cap)[:, :, :n]
+
+    def __iter__(self):
+        return (self[i] for i in range(len(self)))
+
+
+class TrimKVCache(_SlabBacked):
+    """Dense cache: every (batch, kv-head) pair holds the same number of tokens.
+
+    Drop-in for the reference's ``TrimKVCache`` (src/trimkv/cache_utils.py:11-223).
+    """
+
+    def __init__(self, max_seq_len: int = 20480, _distributed_cache_data: Iterable = None, device: str = "cuda") -> None:
+        super().__init__(max_seq_len, _distributed_cache_data, device)
+
+    # The reference exposes four per-layer lists; here they are live views of the slabs.
+    @property
+    def key_cache(self):
+        return _DenseViews(self, "k")
+
+    @property
+    def value_cache(self):
+        return _DenseViews(self, "v")
+
+    @property
+    def retention_weights(self):
+        return _DenseViews(self, "lb")
+
+    @property
+    def kv_positions(self):
+        return _DenseViews(self, "pos")
+
+    def _layer_tuple(self, layer: int):
+        return (self.key_cache[layer], self.value_cache[layer], self.retention_weights[layer], self.kv_positions[layer])
+
+    def __getitem__(self, layer_idx: int):
+        if layer_idx < len(self):
+            return self._layer_tuple(layer_idx)
+        raise KeyError(f"Cache only has {len(self)} layers, attempted to access layer with index {layer_idx}")
+
+    def __iter__(self):
+        for layer_idx in range(len(self)):
+            yield self._layer_tuple(layer_idx)
+
+    def get_cache_length(self, layer_idx: int = 0) -> int:
+        """Tokens currently CACHED per head in ``layer_idx`` (cache_utils.py:134-138)."""
+        if layer_idx >= len(self._slabs) or self._slabs[layer_idx] is None:
+            return 0
+        return self._slabs[layer_idx].max_len
+
+    def get_total_cached_tokens(self, num_key_value_heads: Optional[int] = None) -> int:
+        if num_key_value_heads is None:
+            num_key_value_heads = self._slabs[0].H if self._slabs and self._slabs[0] is not None else 0
+        return sum(self.get_cache_length(l) * num_key_value_heads for l in range(len(self)))
+
+    def update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int,
+               cache_kwargs: Optional[Dict[str, Any]] = None):
+        """Append ``[B,Hkv,S,D]`` keys/values, ``[B,Hkv,S]`` log beta and positions to ``layer_idx``.
+
+        Returns ``(K, V, log_beta, positions, kernel_kwargs)`` for the whole layer, as the
+        reference does (cache_utils.py:62-110).  ``kernel_kwargs`` is empty in the reference;
+        here it carries the device-side segment lengths so that the attention call needs no
+        extra launch.
+        """
+        if key_states is not None:
+            seq_len = key_states.shape[-2]
+            if layer_idx == 0:
+                self._seen_tokens += seq_len
+            self._ensure_layer(layer_idx)
+            slab = self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
+            self.n_seen_tokens[layer_idx] += seq_len
+        slab = self._slabs[layer_idx]
+        extra = {} if slab is None else {"seg_len": slab.seg_len, "max_len": slab.max_len, "seg_cap": slab.cap}
+        return (*self._layer_tuple(layer_idx), extra)
+
+    def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
+                 floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
+                 num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
+        """Evict every layer that holds ``memory_size + buffer_size`` tokens or more down to
+        ``memory_size`` per head (cache_utils.py:140-158)."""
+        num_layers = len(self._slabs) if num_layers is None else num_layers
+        assert num_layers == len(self._slabs), "All caches must have the same number of layers"
+        first = self._slabs[0] if self._slabs else None
+        heads = first.H if first is not None else 0
+        num_key_value_heads = heads if num_key_value_heads is None else num_key_value_heads
+        assert num_key_value_heads == heads, "Key and value caches must have the same number of heads"
+        self._budget_hint = memory_size + buffer_size
+        for layer_idx in range(skip_layers, num_layers):
+            if memory_size + buffer_size <= self.get_cache_length(layer_idx):
+                self.compress_layer(layer_idx, memory_size, strategy, self.sliding_window_size)
+                slab = self._slabs[layer_idx]
+                if slab.cap > 2 * self._budget_hint:  # a long prefill left a slab far larger than steady state needs
+                    slab.regrow(self._budget_hint)
+
+    def compress_layer(self, layer_idx: int, memory_size: int, comrpess_strategy: str = "alpha", sliding_window_size: int = 0,
+                       return_indices: bool = False):
+        """Keep, per (batch, head), the ``memory_size`` tokens with the largest
+        ``fp32(log beta) * (seen + 1 - position)`` in temporal order (cache_utils.py:160-198)."""
+        if comrpess_strategy == "alpha":
+            strat = _lib.SCORE_ALPHA
+        elif comrpess_strategy == "knorm_alpha":
+            strat = _lib.SCORE_KNORM_ALPHA
+        else:
+            raise ValueError(f"Unknown compression strategy: {comrpess_strategy}")
+        slab = self._slabs[layer_idx]
+        n = slab.max_len
+        if memory_size > n:
+            raise RuntimeError(f"selected index k out of range: k={memory_size} > cached tokens {n}")
+        lib = _lib.load()
+        ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, n), slab.k.device)
+        kept = torch.empty(slab.nseg, memory_size, dtype=torch.int32, device=slab.k.device) if return_indices else None
+        rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                              slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                              memory_size, None, 0, self.get_seq_length(layer_idx) + 1, strat, _lib.ROUND_UPCAST,
+                              sliding_window_size, n, _lib.ptr(kept), memory_size,
+                              _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(slab.k.device))
+        _lib.check(rc, "trimkv_evict")
+        slab.lens[:] = memory_size
+        slab.max_len = memory_size
+        if return_indices:
+            return kept.view(slab.B, slab.H, memory_size)
+
+    # ---- batch utilities used by HF generation modes (cache_utils.py:112-132) ---------------
+    def batch_select_indices(self, indices: torch.Tensor):
+        """Only keep ``indices`` along the batch axis (contrastive / beam search)."""
+        for slab in self._slabs:
+            if slab is None:
+                continue
+            idx = indices.to(slab.k.device).long()
+            nb = idx.numel()
+            for name in ("k", "v", "lb", "pos"):
+                t = getattr(slab, name)
+                setattr(slab, name, t.view((slab.B, slab.H) + tuple(t.shape[1:]))[idx].reshape((nb * slab.H,) + tuple(t.shape[1:])).contiguous())
+            slab.seg_len = slab.seg_len.view(slab.B, slab.H)[idx].reshape(-1).contiguous()
+            slab.lens = slab.lens.reshape(slab.B, slab.H)[idx.cpu().numpy()].reshape(-1).copy()
+            slab.B = nb
+
+    def batch_split(self, full_batch_size: int, split_size: int) -> List["TrimKVCache"]:
+        out = []
+        for i in range(0, full_batch_size, split_size):
+            part = TrimKVCache(max_seq_len=self.max_seq_len, device=self.device)
+            part._seen_tokens = self._seen_tokens
+            part.n_seen_tokens = list(self.n_seen_tokens)
+            for slab in self._slabs:
+                if slab is None:
+                    part._slabs.append(None)
+                    continue
+                nb = min(split_size, slab.B - i)
+                new = _Slab.__new__(_Slab)
+                new.B, new.H, new.D, new.cap = nb, slab.H, slab.D, slab.cap
+                lo, hi = i * slab.H, (i + nb) * slab.H
+                new.k, new.v, new.lb, new.pos = slab.k[lo:hi], slab.v[lo:hi], slab.lb[lo:hi], slab.pos[lo:hi]
+                new.seg_len, new.cu = slab.seg_len[lo:hi], None
+                new.lens, new.max_len = slab.lens[lo:hi].copy(), slab.max_len
+                part._slabs.append(new)
+            out.append(part)
+        return out
+
+    # ---- observability (cache_utils.py:200-223) ---------------------------------------------
+    def log(self, layer_idx: int = None):
+        logs = {}
+        if layer_idx is None:
+            for l in range(len(self._slabs)):
+                logs[l] = {"seen_tokens": self.get_seq_length(l), "kv_positions": self.kv_positions[l].detach().cpu()}
+        else:
+            logs["seen_tokens"] = self.get_seq_length(layer_idx)
+            logs["kv_positions"] = self.kv_positions[layer_idx].detach().cpu()
+        return logs
+
+    def copy_to_device(self, device: str):
+        new = TrimKVCache(max_seq_len=self.max_seq_len, device=device)
+        new._seen_tokens = self._seen_tokens
+        new.offset = self.offset.to(device)
+        new.block_mask = self.block_mask.to(device) if self.block_mask is not None else None
+        new.n_seen_tokens = self.n_seen_tokens.copy()
+        new._budget_hint = self._budget_hint
+        for slab in self._slabs:
+            if slab is None:
+                new._slabs.append(None)
+                continue
+            c = _Slab.__new__(_Slab)
+            c.B, c.H, c.D, c.cap = slab.B, slab.H, slab.D, slab.cap
+            c.k, c.v, c.lb, c.pos = (t.to(device, copy=True) for t in (slab.k, slab.v, slab.lb, slab.pos))
+            c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
+            c.lens, c.max_len = slab.lens.copy(), slab.max_len
+            new._slabs.append(c)
+        return new
+
+
+# ==============================================================================================
+# Ragged caches
+# ==============================================================================================
+class _PackedViews:
+    """List-like ``cache.key_cache`` of a ragged cache: item ``l`` is the PACKED ``[sum(n), ...]``
+    tensor the reference stores, gathered from the slab on demand (introspection, tests)."""
+
+    def __init__(self, cache: "_RaggedCache", which: str):
+        self._c, self._w = cache, which
+
+    def __len__(self) -> int:
+        return len(self._c._slabs)
+
+    def __getitem__(self, layer: int) -> torch.Tensor:
+        s = self._c._slabs[layer]
+        if s is None:
+            return _EMPTY()
+        valid = torch.arange(s.cap, device=s.k.device)[None, :] < s.seg_len[:, None]
+        t = getattr(s, self._w)[valid]
+        return t if self._w in ("k", "v") else t.unsqueeze(-1)
+
+    def __iter__(self):
+        return (self[i] for i in range(len(self)))
+
+
+class _RaggedCache(_SlabBacked):
+    """Flat per-head variable-length cache; segments ordered ``seq = b * Hkv + h``."""
+
+    _ragged = True
+
+    def __init__(self, max_seq_len: int = 20480, _distributed_cache_data: Iterable = None, device: str = "cuda") -> None:
+        super().__init__(max_seq_len, _distributed_cache_data, device)
+        self.batch_size: Optional[int] = None
+        self.num_kv_heads: Optional[int] = None
+        self._tables: Dict[Any, torch.Tensor] = {}
+
+    key_cache = property(lambda self: _PackedViews(self, "k"))
+    value_cache = property(lambda self: _PackedViews(self, "v"))
+    retention_weights = property(lambda self: _PackedViews(self, "lb"))
+    kv_positions = property(lambda self: _PackedViews(self, "pos"))
+
+    @property
+    def head_lens(self) -> List[torch.Tensor]:
+        return [_EMPTY() if s is None else s.seg_len for s in self._slabs]
+
+    @property
+    def cu_seqlens_k(self) -> List[torch.Tensor]:
+        return [_EMPTY() if s is None else s.cu for s in self._slabs]
+
+    def get_total_cached_tokens(self) -> int:  # cache_utils.py:253-254, 593-594
+        return int(sum(int(s.lens.sum()) for s in self._slabs if s is not None))
+
+    def _layer_tokens(self, layer: int) -> int:
+        s = self._slabs[layer]
+        return 0 if s is None else int(s.lens.sum())
+
+    def _update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int):
+        if key_states is not None:
+            S = key_states.shape[2]
+            if layer_idx == 0:
+                self._seen_tokens += S
+            self._ensure_layer(layer_idx)
+            slab = self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
+            # on the first call cu starts as zeros and the kernel's "cu[i] += i*S" yields
+            # arange(0, nseg*S+1, S), what the reference builds at cache_utils.py:297, 643
+            self.n_seen_tokens[layer_idx] += S
+        slab = self._slabs[layer_idx]
+        kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu,
+              "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len}
+        flat = (slab.k.view(-1, slab.D), slab.v.view(-1, slab.D), slab.lb.view(-1, 1), slab.pos.view(-1, 1))
+        return flat, kw
+
+    def _seg_start(self, slab: _Slab) -> torch.Tensor:
+        key = ("seg_start", slab.nseg, slab.cap, str(slab.k.device))
+        t = self._tables.get(key)
+        if t is None:
+            t = torch.arange(slab.nseg, dtype=torch.int32, device=slab.k.device) * slab.cap
+            self._tables[key] = t
+        return t
+
+    # ---- selection plumbing ----------------------------------------------------------------
+    @staticmethod
+    def _strategy_code(strategy: str) -> int:
+        base = strategy.replace("_threshold", "")
+        if base == "alpha":
+            return _lib.SCORE_ALPHA
+        if base == "knorm_alpha":
+            return _lib.SCORE_KNORM_ALPHA
+        raise ValueError(f"Unknown compression strategy: {strategy}")
+
+    def _ptr_table(self, tensors: List[torch.Tensor], device) -> torch.Tensor:
+        return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64).to(device)
+
+    def _group_select(self, layers: List[int], segs_per_group: int, budget: int, strategy: str,
+                      threshold: Optional[float] = None):
+        """Run ``trimkv_group_threshold`` over ``layers`` (all of one shape); returns the device
+        tensors (thr_key, tie_take, tie_base [L,nseg], new_len [L,nseg])."""
+        slabs = [self._slabs[l] for l in layers]
+        s0 = slabs[0]
+        for s in slabs:
+            if (s.nseg, s.cap, s.D, s.k.dtype, s.lb.dtype) != (s0.nseg, s0.cap, s0.D, s0.k.dtype, s0.lb.dtype):
+                raise _lib.TrimKVLibraryError("cross-layer selection needs layers of one shape and capacity")
+        dev = s0.k.device
+        L = len(slabs)
+        ngroups = s0.nseg // segs_per_group
+        thr = torch.empty(ngroups, dtype=torch.int32, device=dev)
+        take = torch.empty(ngroups, dtype=torch.int32, device=dev)
+        tie_base = torch.empty(L, s0.nseg, dtype=torch.int32, device=dev)
+        new_len = torch.empty(L, s0.nseg, dtype=torch.int32, device=dev)
+        lb_t = self._ptr_table([s.lb for s in slabs], dev)
+        pos_t = self._ptr_table([s.pos for s in slabs], dev)
+        k_t = self._ptr_table([s.k for s in slabs], dev)
+        len_t = self._ptr_table([s.seg_len for s in slabs], dev)
+        lib = _lib.load()
+        rc = lib.trimkv_group_threshold(lb_t.data_ptr(), pos_t.data_ptr(), k_t.data_ptr(), len_t.data_ptr(),
+                                        L, s0.nseg, segs_per_group, s0.cap, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                        int(budget), 0 if threshold is None else 1, 0.0 if threshold is None else float(threshold),
+                                        self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE,
+                                        thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(),
+                                        _lib.current_stream(dev))
+        _lib.check(rc, "trimkv_group_threshold")
+        self._keepalive = (lb_t, pos_t, k_t, len_t)  # the launch reads these tables asynchronously
+        return thr, take, tie_base, new_len
+
+    def _compact(self, layer: int, segs_per_group: int, thr, take, tie_base_l, strategy: str) -> None:
+        slab = self._slabs[layer]
+        lib = _lib.load()
+        ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
+        rc = lib.trimkv_compact_threshold(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                                          slab.nseg, segs_per_group, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                                          thr.data_ptr(), take.data_ptr(), tie_base_l.data_ptr(),
+                                          self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE, slab.max_len,
+                                          _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(slab.k.device))
+        _lib.check(rc, "trimkv_compact_threshold")
+
+    def _evict_per_segment(self, layer: int, keep: np.ndarray, strategy: str) -> None:
+        slab = self._slabs[layer]
+        keep_dev = torch.from_numpy(np.ascontiguousarray(keep, dtype=np.int32)).to(slab.k.device)
+        lib = _lib.load()
+        ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
+        rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                              slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                              0, keep_dev.data_ptr(), 0, self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE,
+                              0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(slab.k.device))
+        _lib.check(rc, "trimkv_evict")
+        self._keepalive2 = keep_dev
+
+    def _refresh(self, layers: List[int]) -> None:
+        """After an eviction: rebuild cu_seqlens on the device and bring the new lengths to the
+        host -- the one synchronisation an eviction costs (the reference pays O(B*L*Hkv))."""
+        lib = _lib.load()
+        for l in layers:
+            slab = self._slabs[l]
+            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
+            _lib.check(rc, "trimkv_build_cu_seqlens")
+        if layers:
+            lens = torch.stack([self._slabs[l].seg_len for l in layers]).cpu().numpy().astype(np.int64)
+            for i, l in enumerate(layers):
+                self._slabs[l].lens = lens[i].copy()
+                self._slabs[l].max_len = int(lens[i].max())
+
+    def set_budgets(self, budgets) -> None:
+        """Give every segment its own token budget: ``budgets`` is ``[nseg]`` (all layers alike) or
+        ``[num_layers][nseg]`` integers.  Used by :meth:`evict_to_budgets`."""
+        arr = np.asarray(budgets.cpu() if torch.is_tensor(budgets) else budgets, dtype=np.int64)
+        self._budgets_host = arr
+        self._budgets_dev: Dict[Any, torch.Tensor] = {}
+
+    def evict_to_budgets(self, buffer_size: int = 0, strategy: str = "alpha", layers: Optional[List[int]] = None) -> None:
+        """Per-head budgets: segment ``seg`` of every listed layer is cut to its ``budget[seg]`` best
+        tokens once it holds ``budget[seg] + buffer_size`` or more.  This is the per-head
+        variable-k select the reference reaches through its floor branch
+        (cache_utils.py:508-521).  The trigger is evaluated on the host mirror of the lengths and
+        again per segment on the device; no host synchronisation happens here."""
+        layers = [l for l in range(len(self._slabs)) if self._slabs[l] is not None] if layers is None else layers
+        lib = _lib.load()
+        code = self._strategy_code(strategy)
+        for l in layers:
+            slab = self._slabs[l]
+            kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[l]
+            hit = (slab.lens > kh) & (slab.lens >= kh + buffer_size)
+            if not hit.any():
+                continue
+            key = (l if self._budgets_host.ndim == 2 else -1, str(slab.k.device))
+            keep = self._budgets_dev.get(key)
+            if keep is None:
+                keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(slab.k.device)
+                self._budgets_dev[key] = keep
+            st = _lib.current_stream(slab.k.device)
+            ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
+            rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                                  slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                                  0, keep.data_ptr(), buffer_size, self.get_seq_length() + 1, code, _lib.ROUND_NATIVE,
+                                  0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(), st)
+            _lib.check(rc, "trimkv_evict")
+            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), st)
+            _lib.check(rc, "trimkv_build_cu_seqlens")
+            slab.lens = np.where(hit, kh, slab.lens)
+            slab.max_len = int(slab.lens.max())
+
+    def segment_positions(self):
+        """Per layer, per segment: retained absolute positions (host tensors)."""
+        out = []
+        for s in self._slabs:
+            pos = s.pos.cpu()
+            out.append([pos[i, : int(s.lens[i])].clone() for i in range(s.nseg)])
+        return out
+
+    def copy_to_device(self, device):
+        raise NotImplementedError(f"copy_to_device not implemented for {type(self).__name__}")
+
+
+class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
+    """Drop-in for the reference's ``BatchedDynamicBudgetTrimKVCache`` (cache_utils.py:563-971)."""
+
+    def update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int,
+               cache_kwargs: Optional[Dict[str, Any]] = None):
+        if key_states is not None:
+            B, H, S, D = key_states.shape
+            if self.batch_size is None:
+                self.batch_size, self.num_kv_heads = B, H
+            else:
+                assert B == self.batch_size, f"Batch size changed: {self.batch_size} -> {B}"
+                assert H == self.num_kv_heads, f"Num KV heads changed: {self.num_kv_heads} -> {H}"
+        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx)
+        kw["batch_size"], kw["num_kv_heads"] = self.batch_size, self.num_kv_heads
+        return (*flat, kw)
+
+    def get_cache_length(self, layer_idx: int = 0, batch_idx: int = 0, head_idx: int = 0) -> int:
+        if layer_idx >= len(self._slabs) or self._slabs[layer_idx] is None:
+            return 0
+        return int(self._slabs[layer_idx].lens[batch_idx * self.num_kv_heads + head_idx])
+
+    @torch.inference_mode()
+    def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
+                 floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
+                 num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
+        num_layers = len(self._slabs) if num_layers is None else num_layers
+        H = self.num_kv_heads if num_key_value_heads is None else num_key_value_heads
+        B = self.batch_size
+        if self.get_total_cached_tokens() <= B * H * (memory_size + buffer_size) * num_layers and "threshold" not in strategy:
+            return  # cache_utils.py:714-717
+        if "layer_wise" in strategy:  # cache_utils.py:719-729, 740-834
+            base = strategy.replace("layer_wise_", "")
+            if base not in ("alpha", "knorm_alpha"):
+                raise ValueError(f"Unknown compression strategy: {base}")
+            todo = [l for l in range(num_layers) if self._layer_tokens(l) > B * H * (memory_size + buffer_size)]
+            for l in todo:
+                if floor_budget_ratio > 0:
+                    budget = int(memory_size * H * (1 - floor_budget_ratio))
+                    _, _, _, new_len = self._group_select([l], H, budget, base)
+                    chosen = new_len[0].cpu().numpy().astype(np.int64)
+                    floor_per_head = int(memory_size * floor_budget_ratio)
+                    # top-up (:789-806): a head keeps its best max(chosen, floor) tokens, at most all of them
+                    keep = np.minimum(np.maximum(chosen, floor_per_head), self._slabs[l].lens)
+                    self._evict_per_segment(l, keep, base)
+                else:
+                    thr, take, tie_base, _ = self._group_select([l], H, memory_size * H, base)
+                    self._compact(l, H, thr, take, tie_base[0], base)
+            self._refresh(todo)
+        else:  # cache_utils.py:836-945; floor_budget_ratio is not used by this variant
+            tokens_per_batch = sum(self._layer_tokens(l) for l in range(num_layers)) // B
+            if tokens_per_batch <= num_layers * H * (memory_size + buffer_size) and "threshold" not in strategy:
+                return
+            if strategy not in ("alpha", "knorm_alpha", "alpha_threshold", "knorm_alpha_threshold"):
+                raise ValueError(f"Unknown compression strategy: {strategy}")
+            layers = list(range(num_layers))
+            threshold = None
+            if "threshold" in strategy:
+                threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
+            thr, take, tie_base, _ = self._group_select(layers, H, num_layers * H * memory_size, strategy, threshold)
+            for i, l in enumerate(layers):
+                self._compact(l, H, thr, take, tie_base[i], strategy)
+            self._refresh(layers)
+
+    def log(self):
+        positions = self.segment_positions()
+        return {"batch_size": self.batch_size, "num_kv_heads": self.num_kv_heads,
+                "head_wise_kv_positions": [p for layer in positions for p in layer],
+                "flat_head_lens": np.concatenate([s.lens for s in self._slabs]).astype(np.int32)}
+
+
+class DynamicBudgetTrimKVCache(_RaggedCache):
+    """Drop-in for the reference's ``DynamicBudgetTrimKVCache`` (cache_utils.py:226-560): batch size 1."""
+
+    def update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int,
+               cache_kwargs: Optional[Dict[str, Any]] = None):
+        if key_states is not None:
+            assert key_states.shape[0] == 1, "Batch size greater than 1 is not supported for DynamicBudgetTrimKVCache"
+            self.batch_size, self.num_kv_heads = 1, key_states.shape[1]
+        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx)
+        return (*flat, kw)
+
+    def get_cache_length(self, layer_idx: int = 0, head_idx: int = 0) -> int:
+        if layer_idx >= len(self._slabs) or self._slabs[layer_idx] is None:
+            return 0
+        return int(self._slabs[layer_idx].lens[head_idx])
+
+    @torch.inference_mode()
+    def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
+                 floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
+                 num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
+        num_layers = len(self._slabs) if num_layers is None else num_layers
+        H = self._slabs[0].nseg if num_key_value_heads is None else num_key_value_heads
+        if "layer_wise" in strategy:  # cache_utils.py:356-369, 371-416: one top-k over the whole layer
+            base = strategy.replace("layer_wise_", "")
+            todo = [l for l in range(num_layers) if not H * (memory_size + buffer_size) >= self._layer_tokens(l)]
+            if todo and base not in ("alpha", "knorm_alpha"):
+                raise ValueError(f"Unknown compression strategy: {base}")
+            for l in todo:
+                thr, take, tie_base, _ = self._group_select([l], H, H * memory_size, base)
+                self._compact(l, H, thr, take, tie_base[0], base)
+            self._refresh(todo)
+            return
+        # all layers at once, cache_utils.py:418-536
+        total_budget = num_layers * H * memory_size
+        if num_layers * H * (memory_size + buffer_size) > self.get_total_cached_tokens() and "threshold" not in strategy:
+            return
+        if strategy not in ("alpha", "knorm_alpha", "alpha_threshold", "knorm_alpha_threshold"):
+            raise ValueError(f"Unknown compression strategy: {strategy}")
+        layers = list(range(num_layers))
+        if floor_budget_ratio == 0:
+            threshold = None
+            if "threshold" in strategy:
+                threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
+            thr, take, tie_base, _ = self._group_select(layers, H, total_budget, strategy, threshold)
+            for i, l in enumerate(layers):
+                self._compact(l, H, thr, take, tie_base[i], strategy)
+            self._refresh(layers)
+            return
+        assert "threshold" not in strategy, "Thresholding strategy is not compatible with floor_budget_ratio > 0"
+        adaptive = int(total_budget * (1 - floor_budget_ratio))
+        thr, take, tie_base, new_len = self._group_select(layers, H, adaptive, strategy)
+        chosen = new_len.cpu().numpy().astype(np.int64).reshape(-1)          # per (layer, head), flattened
+        first_sel = self._first_token_selected(layers, thr, take, tie_base, strategy).reshape(-1)
+        lens = np.concatenate([self._slabs[l].lens for l in layers])
+        # bucketize against the inclusive cumsum with right=False (cache_utils.py:496): a chosen
+        # token that is the FIRST row of head j >= 1 is counted for head j-1.
+        credited = chosen.copy()
+        moved = first_sel.copy()
+        moved[0] = 0
+        moved[lens == 0] = 0
+        credited -= moved
+        credited[:-1] += moved[1:]
+        head_cnt = credited + int(memory_size * floor_budget_ratio)
+        for i, l in enumerate(layers):
+            self._evict_per_segment(l, head_cnt[i * H:(i + 1) * H], strategy)  # k >= len keeps all (:514-516)
+        self._refresh(layers)
+
+    def _first_token_selected(self, layers, thr, take, tie_base, strategy) -> np.ndarray:
+        """For every (layer, head): is its oldest token among the globally chosen ones?"""
+        thr_key = int(thr.cpu().numpy().astype(np.uint32)[0])
+        take_n = int(take.cpu()[0])
+        tb = tie_base.cpu().numpy()
+        q_idx = self.get_seq_length() + 1
+        out = np.zeros((len(layers), self._slabs[layers[0]].nseg), dtype=np.int64)
+        for i, l in enumerate(layers):
+            s = self._slabs[l]
+            lb0, pos0 = s.lb[:, 0], s.pos[:, 0]
+            score = (q_idx - pos0) * lb0  # the ragged classes' own expression (cache_utils.py:441)
+            if "knorm" in strategy:
+                score = score + torch.log(s.k[:, 0].norm(dim=-1).clamp_min(1e-12))
+            f = score.float().cpu().numpy().astype(np.float32)
+            f = np.where(f == 0, np.float32(0), f)
+            u = f.view(np.uint32)
+            key = np.where(u & np.uint32(0x80000000), ~u, u | np.uint32(0x80000000)).astype(np.uint64)
+            sel = (key > thr_key) | ((key == thr_key) & (tb[i] < take_n))
+            out[i] = sel & (s.lens > 0)
+        return out
+
+    def log(self):
+        positions = self.segment_positions()
+        return {"head_wise_kv_positions": [p for layer in positions for p in layer],
+                "flat_head_lens": np.concatenate([s.lens for s in self._slabs]).astype(np.int32)}

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     __shared__ float sl[AT_WAVES][8];
 
     const int seg = blockIdx.y, split = blockIdx.x;
-    int n = a.seg_len[seg];
+    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int nsp = (n + a.chunk - 1) / a.chunk;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
 template <int G>
 __global__ __launch_bounds__(AT_D) void decode_attn_merge_kernel(AttnArgs a) {
     const int seg = blockIdx.x, d = threadIdx.x;
-    int n = a.seg_len[seg];
+    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int nsp = (n + a.chunk - 1) / a.chunk;
 #pragma unroll
@@ -340,13 +340,13 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
                                   int nseg, int cap, int head_dim, int group, int dtype, float scale,
                                   int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_decode_attn";
-    if (!q || !out || !k_slab || !v_slab || !seg_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
     if (head_dim != AT_D) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be %d (got %d)", fn, AT_D, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
     if (nseg > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nseg=%d exceeds the grid limit 65535", fn, nseg);
-    if (max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
+    if (!seg_start && max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
     if (((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_slab | (uintptr_t)v_slab) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: q/out/K/V must be 16-byte aligned", fn);
     if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
     if (chunk % 64) return fail(TRIMKV_ERR_SHAPE, "%s: chunk must be a multiple of 64 (got %d)", fn, chunk);
