@@ -1,0 +1,260 @@
+#!/usr/bin/env python3
+"""Decode-step benchmark of the TRIM-KV cache hot path on one MI355X.
+
+One "step" = for every layer: append one token per (batch, kv-head) segment + single-query GQA
+attention over the retained K/V; then, after the last layer, evict every layer that reached
+memory_size + buffer_size.  Inputs are synthetic (K, V ~ N(0,1) in bf16, log beta =
+logsigmoid(N(mu, sigma)) in fp32, random bf16 queries) and resident in HBM before the clock starts.
+
+    python bench.py [--gpus 1] [--steps 1024] [--warmup 128] [--config 3]
+
+prints ONE JSON line.  `value` = batch * steps / seconds (decode tokens/s for the whole job).
+`roofline` prices the dominant kernel (decode attention) against the 8 TB/s HBM peak using its
+algorithmic bytes and HIP-event durations sampled inside the timed region; `cpu_baseline` times the
+CPU oracle (the reference's pure-PyTorch path restated) on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "decode tokens/s (evict+append+varlen attn) & % of 8 TB/s HBM, Qwen3-8B shape"
+HBM_PEAK_GBS = 8000.0
+
+# BASELINE.json configs that fit one GPU as a steady-state decode loop (index = order in BASELINE.json)
+CONFIGS = {
+    2: dict(name="qwen3-1.7b", L=28, B=16, Hkv=8, Hq=16, M=2048, buf=128, mu=3.0, sigma=1.0),
+    3: dict(name="qwen3-8b", L=36, B=64, Hkv=8, Hq=32, M=4096, buf=128, mu=3.0, sigma=1.5),
+    5: dict(name="qwen3-14b", L=40, B=8, Hkv=8, Hq=40, M=8192, buf=512, mu=2.0, sigma=2.0),
+}
+D = 128
+
+
+def algorithmic_bytes(c):
+    """Bytes one decode step has to move (per layer, then total): every retained K and V row read
+    once, q read and o written, one K/V row + 12 bytes of metadata written per segment, and the
+    eviction (12 bytes of score inputs per cached token, kept rows and metadata read and
+    written) amortised over the buffer_size steps between evictions."""
+    nseg, G, e = c["B"] * c["Hkv"], c["Hq"] // c["Hkv"], 2
+    nbar = c["M"] + (c["buf"] + 1) / 2
+    attn_kv = nseg * 2 * nbar * D * e
+    attn_qo = nseg * 2 * G * D * e
+    append = nseg * (2 * D * e + 12)
+    evict = nseg * (12 * (c["M"] + c["buf"]) + 2 * 12 * c["M"] + 2 * 2 * c["M"] * D * e) / c["buf"]
+    return dict(attn=attn_kv + attn_qo, append=append, evict=evict, step=c["L"] * (attn_kv + attn_qo + append + evict))
+
+
+def cpu_baseline(c, budget_s=20.0):
+    """The oracle (the reference's pure-PyTorch CPU path restated) on ONE layer at full shape,
+    extrapolated to the full step: t_step = L * (B / b) * (t_append_attend + t_evict / buffer)."""
+    import torch
+    from oracle.attn_ref import eager_attention
+    from oracle.dense_ref import DenseCacheRef
+
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    b = c["B"]  # one layer at its full shape
+    G = c["Hq"] // c["Hkv"]
+    gen = torch.Generator().manual_seed(1234)
+    n0 = c["M"] + c["buf"] - 3
+    ref = DenseCacheRef()
+    k = torch.randn(b, c["Hkv"], n0, D, generator=gen).to(torch.bfloat16)
+    v = torch.randn(b, c["Hkv"], n0, D, generator=gen).to(torch.bfloat16)
+    lb = torch.nn.functional.logsigmoid(torch.randn(b, c["Hkv"], n0, generator=gen) * c["sigma"] + c["mu"])
+    ref.update(k, v, lb, torch.arange(n0), 0)
+    t_steps = []
+    t_start = time.perf_counter()
+    for i in range(3):
+        kn = torch.randn(b, c["Hkv"], 1, D, generator=gen).to(torch.bfloat16)
+        vn = torch.randn(b, c["Hkv"], 1, D, generator=gen).to(torch.bfloat16)
+        lbn = torch.nn.functional.logsigmoid(torch.randn(b, c["Hkv"], 1, generator=gen) * c["sigma"] + c["mu"])
+        q = torch.randn(b, c["Hq"], 1, D, generator=gen).to(torch.bfloat16)
+        t0 = time.perf_counter()
+        kk, vv, _, _, _ = ref.update(kn, vn, lbn, torch.arange(n0 + i, n0 + i + 1), 0)
+        eager_attention(q, kk, vv, G, D ** -0.5)
+        t_steps.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_start > budget_s and i >= 1:
+            break
+    t0 = time.perf_counter()
+    ref.compress("alpha", c["M"], c["buf"])
+    t_evict = time.perf_counter() - t0
+    assert ref.get_cache_length(0) == c["M"]
+    t_aa = min(t_steps[1:]) if len(t_steps) > 1 else t_steps[0]  # first step warms the allocator
+    t_step = c["L"] * (c["B"] / b) * (t_aa + t_evict / c["buf"])
+    return {"value": c["B"] / t_step, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"1 of {c['L']} layers, batch {b} of {c['B']}: {len(t_steps)} append+attend steps at n~{n0} "
+                      f"({t_aa * 1e3:.0f} ms) + 1 eviction ({t_evict * 1e3:.0f} ms); extrapolated "
+                      f"t_step = L*(B/b)*(t_append_attend + t_evict/buffer)",
+            "os_cpu_count": cores}
+
+
+def parity_gate(cache, c, attn_fn, mod):
+    """Outside the timed region: one more step on layer 0 checked against the oracle (positions
+    bit-exact for every segment; attention of a few segments against fp32)."""
+    import torch
+    from oracle.dense_ref import keep_indices, retention_scores
+
+    slab = cache._slabs[0]
+    n = slab.max_len
+    lb = slab.lb[:, :n].cpu()
+    pos = slab.pos[:, :n].cpu()
+    k = slab.k[:8, :n].float().cpu()
+    v = slab.v[:8, :n].float().cpu()
+    G = c["Hq"] // c["Hkv"]
+    q = torch.randn(c["B"], c["Hq"], 1, D, device=slab.k.device).to(torch.bfloat16)
+    out, _, _ = attn_fn(mod, q, cache.key_cache[0], cache.value_cache[0], None, scaling=D ** -0.5,
+                        flash_attn_kwargs={"seg_len": slab.seg_len, "max_len": n})
+    q8 = q.reshape(-1, G, D)[:8].float().cpu()
+    s = torch.einsum("sgd,snd->sgn", q8, k) * D ** -0.5
+    want = torch.einsum("sgn,snd->sgd", torch.softmax(s, -1), v)
+    got = out.reshape(-1, G, D)[:8].float().cpu()
+    err = (got - want).abs()
+    attn_ok = bool((err <= 2e-2 + 1e-2 * want.abs()).all())
+    result = {"attention_max_abs_err": float(err.max()), "attention_within_2e-2_abs_1e-2_rel": attn_ok}
+    if n > c["M"]:
+        q_idx = cache.get_seq_length(0) + 1
+        sc = retention_scores(lb, pos, q_idx)
+        top = torch.topk(sc, c["M"] + 1, dim=-1).values
+        ties = int((top[:, c["M"] - 1] == top[:, c["M"]]).sum())
+        want_idx = keep_indices(sc, c["M"])
+        got_idx = cache.compress_layer(0, c["M"], return_indices=True).view(-1, c["M"]).cpu().long()
+        same = (got_idx == want_idx).all(dim=-1)
+        result.update({"evicted_segments_checked": int(same.numel()), "retained_index_mismatches": int((~same).sum()),
+                       "boundary_tie_rows": ties})
+    return result
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=128)
+    ap.add_argument("--config", type=int, default=3, choices=sorted(CONFIGS))
+    ap.add_argument("--chunk", type=int, default=0, help="split-K rows per workgroup for decode attention (0 = library default)")
+    ap.add_argument("--layers", type=int, default=0, help="override the number of layers (smoke runs only; makes the result invalid)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--event-every", type=int, default=8, help="sample attention launches with HIP events every N steps")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures ONE GPU: the path shards by batch or KV head without communication, "
+              "so a multi-GPU figure is N independent copies of this run; --gpus must be 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    from trimkv_amd.attn import hip_attn
+
+    c = dict(CONFIGS[args.config])
+    if args.layers:
+        c["L"] = args.layers
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, B, Hkv, Hq, M, buf = c["L"], c["B"], c["Hkv"], c["Hq"], c["M"], c["buf"]
+    G = Hq // Hkv
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    class Mod:
+        training = False
+        num_key_value_groups = G
+
+    mod = Mod()
+    attn_fn = get_attention_interface("trimkv_hip")
+    if args.chunk:
+        _orig = hip_attn.decode_attention
+        hip_attn.decode_attention = lambda *a, **k: _orig(*a, **{**k, "chunk": args.chunk})
+
+    # steady-state cache: M + buf tokens per head, so the first step appends, attends and evicts
+    cache = TrimKVCache()
+    n0 = M + buf
+    pos0 = torch.arange(n0, device=dev)
+    for l in range(L):
+        k = torch.randn(B, Hkv, n0, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        v = torch.randn(B, Hkv, n0, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
+        lb = torch.nn.functional.logsigmoid(torch.randn(B, Hkv, n0, generator=gen, device=dev) * c["sigma"] + c["mu"])
+        cache.update(k, v, lb, pos0, l)
+        del k, v, lb
+    POOL = 4
+    pool = []
+    for l in range(L):
+        per = []
+        for _ in range(POOL):
+            per.append((torch.randn(B, Hkv, 1, D, generator=gen, device=dev).to(torch.bfloat16),
+                        torch.randn(B, Hkv, 1, D, generator=gen, device=dev).to(torch.bfloat16),
+                        torch.nn.functional.logsigmoid(torch.randn(B, Hkv, 1, generator=gen, device=dev) * c["sigma"] + c["mu"]),
+                        torch.randn(B, Hq, 1, D, generator=gen, device=dev).to(torch.bfloat16)))
+        pool.append(per)
+    torch.cuda.synchronize()
+
+    T = n0
+    events = []
+
+    def step(t, sample):
+        nonlocal T
+        pos = torch.full((1,), T, dtype=torch.int64, device=dev)
+        for l in range(L):
+            kn, vn, lbn, q = pool[l][t % POOL]
+            K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
+            if sample:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+                e1.record()
+                events.append((e0, e1, cache.get_cache_length(l)))
+            else:
+                attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+        T += 1
+        cache.compress("alpha", M, buf)
+
+    for t in range(args.warmup):
+        step(t, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(args.steps):
+        step(args.warmup + t, args.event_every > 0 and t % args.event_every == 0)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+
+    ms_per_step = seconds * 1e3 / args.steps
+    value = B * args.steps / seconds
+    ab = algorithmic_bytes(c)
+    nseg = B * Hkv
+    roof = None
+    if events:
+        durs = [e0.elapsed_time(e1) * 1e-3 for e0, e1, _ in events]
+        lens = [n for _, _, n in events]
+        avg_s = sum(durs) / len(durs)
+        avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
+        achieved = avg_bytes / avg_s / 1e9
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}> (+ split-K merge)", "achieved": round(achieved, 1),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
+                "algorithmic_bytes_per_launch": int(avg_bytes)}
+    parity = parity_gate(cache, c, attn_fn, mod)
+    out = {
+        "metric": METRIC, "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"BASELINE config {args.config} ({c['name']} shape): {L} layers, batch {B}, {Hkv} KV heads, {Hq} query heads, "
+                               f"head_dim {D}, memory_size {M}, buffer_size {buf}, steady-state decode (append + attend per layer, "
+                               f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
+                   "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(), "evictions_in_timed_region": args.steps // buf if args.warmup % buf == 0 else None},
+        "step_hbm": {"algorithmic_bytes_per_step": int(ab["step"]), "achieved_GBps": round(ab["step"] / (seconds / args.steps) / 1e9, 1),
+                     "frac_of_8TBps": round(ab["step"] / (seconds / args.steps) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": roof,
+        "parity": parity,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(c)
+    if args.layers:
+        out["config"]["note"] = "layer count overridden: not the BASELINE configuration"
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
