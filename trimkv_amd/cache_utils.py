@@ -478,6 +478,10 @@ class _RaggedCache(_SlabBacked):
         self.num_kv_heads: Optional[int] = None
         self._tables: Dict[Any, torch.Tensor] = {}
 
+    # plain attributes in the reference; a property here because newer HF Cache classes define a
+    # read-only `batch_size` of their own
+    batch_size = property(lambda self: self._batch_size, lambda self, v: setattr(self, "_batch_size", v))
+
     key_cache = property(lambda self: _PackedViews(self, "k"))
     value_cache = property(lambda self: _PackedViews(self, "v"))
     retention_weights = property(lambda self: _PackedViews(self, "lb"))
