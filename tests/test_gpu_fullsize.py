@@ -1,0 +1,170 @@
+"""BASELINE.json's full sizes (one layer of each config), checked through properties that do not need
+the CPU oracle at that size: kept-set threshold property, temporal order, idempotence, agreement
+with torch's own topk/sort/gather on the device, split invariance, exact linearity in V, permutation
+invariance, and fp32 attention on sampled segments."""
+import numpy as np
+import pytest
+import torch
+
+from tests.gpu_util import DEV, attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+class _Mod:
+    training = False
+
+
+def _fill_dense(B, H, n, mu, sigma, seed):
+    from trimkv_amd import TrimKVCache
+    gen = torch.Generator(device=DEV).manual_seed(seed)
+    k = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    v = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    lb = torch.nn.functional.logsigmoid(torch.randn(B, H, n, generator=gen, device=DEV) * sigma + mu)
+    cache = TrimKVCache()
+    cache.update(k, v, lb, torch.arange(n, device=DEV), 0)
+    return cache, k, v, lb, gen
+
+
+def _check_eviction(cache, k, v, lb, n, M, seen):
+    pos = torch.arange(n, device=DEV).expand_as(lb)
+    sc = lb.float() * (seen + 1 - pos)                       # the reference's expression, on the device
+    top = torch.topk(sc, M + 1, dim=-1).values
+    tie = top[..., M - 1] == top[..., M]
+    want = torch.sort(torch.topk(sc, M, dim=-1).indices, dim=-1).values
+    got = cache.compress_layer(0, M, return_indices=True).long()
+    assert cache.get_cache_length(0) == M and (cache._slabs[0].seg_len == M).all()
+    assert (got[..., 1:] > got[..., :-1]).all()               # temporal order, no duplicates
+    kept_min = torch.gather(sc, -1, got).min(-1).values
+    mask = torch.ones_like(sc, dtype=torch.bool).scatter_(-1, got, False)
+    evicted_max = sc.masked_fill(~mask, float("-inf")).max(-1).values
+    assert (kept_min >= evicted_max).all()                    # nothing evicted outranks anything kept
+    assert torch.equal(got[~tie], want[~tie]), "retained indices differ from torch.topk on rows without a boundary tie"
+    K, V, LB, POS = cache[0]
+    idx = got.unsqueeze(-1).expand(-1, -1, -1, 128)
+    assert torch.equal(K, k.gather(2, idx)) and torch.equal(V, v.gather(2, idx))
+    assert torch.equal(LB, lb.gather(2, got)) and torch.equal(POS, got)
+    before = [t.clone() for t in cache[0]]
+    cache.compress("alpha", M, 1)                             # n == M < M + 1: nothing may change
+    assert all(torch.equal(a, b) for a, b in zip(before, cache[0]))
+    return int(tie.sum())
+
+
+def test_config3_qwen3_8b_layer_eviction_and_attention():
+    """B=64, 8 KV heads, 32 query heads, M=4096, buffer 128: 512 segments of 4225 rows."""
+    from trimkv_amd import get_attention_interface
+    from trimkv_amd.attn.hip_attn import decode_attention
+    B, H, G, M, n = 64, 8, 4, 4096, 4225
+    cache, k, v, lb, gen = _fill_dense(B, H, n, 3.0, 1.5, seed=3)
+    attn = get_attention_interface("trimkv_hip")
+    q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    K, V, _, _, kw = cache.update(None, None, None, None, 0)
+    out, _, _ = attn(_Mod(), q, K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)
+    # fp32 attention on 16 sampled segments
+    segs = torch.arange(0, B * H, 32)
+    q32 = q.view(B * H, G, 128)[segs].float()
+    k32, v32 = k.view(B * H, n, 128)[segs].float(), v.view(B * H, n, 128)[segs].float()
+    p = torch.softmax(torch.einsum("sgd,snd->sgn", q32, k32) * 128 ** -0.5, -1)
+    want = torch.einsum("sgn,snd->sgd", p, v32)
+    ok, err = attn_close(out.view(B * H, G, 128)[segs], want)
+    assert ok, err
+    # split invariance: any chunking gives the same answer up to bf16 output rounding
+    q2 = q.view(B * H * G, 128)
+    slab = cache._slabs[0]
+    outs = [decode_attention(q2, slab.k, slab.v, B * H, G, slab.seg_len, None, slab.cap, n, 128 ** -0.5, chunk=c)
+            for c in (256, 1024, 8192)]
+    for o in outs:
+        assert (o.float() - out.view(-1, 128).float()).abs().max() < 4e-3
+    # exact linearity in V: doubling V doubles the output bit for bit (powers of two are exact)
+    slab.v.mul_(2)
+    out2 = decode_attention(q2, slab.k, slab.v, B * H, G, slab.seg_len, None, slab.cap, n, 128 ** -0.5)
+    assert torch.equal(out2.float(), out.view(-1, 128).float() * 2)
+    slab.v.div_(2)
+    ties = _check_eviction(cache, k, v, lb, n, M, seen=n)
+    assert ties <= 2
+
+
+def test_config2_qwen3_1p7b_prefill_compression():
+    """B=16, 8 KV heads, G=2: 8192-token prefill compressed to M=2048, then the slab is right-sized."""
+    B, H, M, n = 16, 8, 2048, 8192
+    cache, k, v, lb, _ = _fill_dense(B, H, n, 3.0, 1.0, seed=2)
+    _check_eviction(cache, k, v, lb, n, M, seen=n)
+    kept = [t.clone() for t in cache[0]]
+    cache.compress("alpha", M, 128)                           # no eviction (n == M) but remembers the budget
+    assert cache._slabs[0].cap == n + max(128, n // 8)
+    c2, k2, v2, lb2, _ = _fill_dense(B, H, n, 3.0, 1.0, seed=2)
+    c2.compress("alpha", M, 128)                              # evicts AND shrinks the slab to M + buffer
+    assert c2._slabs[0].cap == M + 128
+    assert all(torch.equal(a, b) for a, b in zip(kept, c2[0]))
+
+
+def test_config5_qwen3_14b_chunk_eviction_gqa5():
+    """8 KV heads, G=5, M=8192, buffer 512: a 4096-token chunk on top of 8192 cached, select 8192 of 12288
+    (batch 2 of the config's 8 to bound memory; the kernel's grid is per segment)."""
+    from trimkv_amd import get_attention_interface
+    B, H, G, M, n = 2, 8, 5, 8192, 12288
+    cache, k, v, lb, gen = _fill_dense(B, H, n, 2.0, 2.0, seed=5)
+    ties = _check_eviction(cache, k, v, lb, n, M, seen=n)
+    assert ties <= 1
+    attn = get_attention_interface("trimkv_hip")
+    q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    K, V, _, _, kw = cache.update(None, None, None, None, 0)
+    out, _, _ = attn(_Mod(), q, K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)
+    p = torch.softmax(torch.einsum("sgd,snd->sgn", q.view(B * H, G, 128).float(), K.reshape(B * H, M, 128).float()) * 128 ** -0.5, -1)
+    want = torch.einsum("sgn,snd->sgd", p, V.reshape(B * H, M, 128).float())
+    ok, err = attn_close(out.view(B * H, G, 128), want)
+    assert ok, err
+
+
+def test_config4_ragged_lognormal_budgets():
+    """B=32, 8 KV heads, G=4; per-head budgets lognormal(median 1024, sigma 1) clipped to [64, 8192],
+    prompt lengths U[512, 16384] per batch element; decode steps with per-head eviction at budget + 128."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, get_attention_interface
+    B, H, G, buf = 32, 8, 4, 128
+    rng = np.random.default_rng(4)
+    budgets = np.clip(np.round(np.exp(rng.normal(np.log(1024), 1.0, size=B * H))), 64, 8192).astype(np.int64)
+    prompt = rng.integers(512, 16385, size=B)
+    start = np.minimum(budgets, np.repeat(prompt, H))         # what each head holds after its prompt
+    S = int(start.max())
+    gen = torch.Generator(device=DEV).manual_seed(4)
+    cache = BatchedDynamicBudgetTrimKVCache()
+    k = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    v = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    lb = torch.nn.functional.logsigmoid(torch.randn(B, H, S, generator=gen, device=DEV) * 1.5 + 3.0)
+    cache.update(k, v, lb, torch.arange(S, device=DEV), 0)
+    cache.set_budgets(start)
+    cache.evict_to_budgets(buffer_size=0)                     # ragged initial state
+    assert cache.head_lens[0].cpu().tolist() == start.tolist()
+    pos0 = cache.segment_positions()[0]
+    sc = lb.float() * (S + 1 - torch.arange(S, device=DEV))
+    for seg in rng.choice(B * H, 24, replace=False):           # kept set = top-start[seg] of the prompt, in order
+        want = torch.sort(torch.topk(sc.view(B * H, S)[seg], int(start[seg])).indices).values.cpu()
+        assert torch.equal(pos0[seg], want)
+    cache.set_budgets(budgets)
+    attn = get_attention_interface("db_attn_flash_batched")
+    lens = start.copy()
+    for t in range(140):
+        kn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        vn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        lbn = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) * 1.5 + 3.0)
+        K, V, _, _, kw = cache.update(kn, vn, lbn, torch.arange(S + t, S + t + 1, device=DEV), 0)
+        lens += 1
+        if t % 35 == 0:
+            q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+            out, _, _ = attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw)
+            slab = cache._slabs[0]
+            for seg in (0, 37, 101, 255):
+                n = int(lens[seg])
+                kk, vv = slab.k[seg, :n].float(), slab.v[seg, :n].float()
+                p = torch.softmax(q.view(B * H, G, 128)[seg].float() @ kk.T * 128 ** -0.5, -1)
+                ok, err = attn_close(out.view(B * H, G, 128)[seg], p @ vv)
+                assert ok, (seg, err)
+        cache.evict_to_budgets(buffer_size=buf)
+        hit = (lens > budgets) & (lens >= budgets + buf)
+        lens = np.where(hit, budgets, lens)
+        assert cache._slabs[0].lens.tolist() == lens.tolist()
+    assert cache.head_lens[0].cpu().tolist() == lens.tolist()
+    assert cache.cu_seqlens_k[0].cpu().tolist() == [0] + np.cumsum(lens).tolist()
+    for seg, p in enumerate(cache.segment_positions()[0]):
+        assert p.numel() == lens[seg] and (p[1:] > p[:-1]).all()
+    assert hit.sum() == 0 and (lens <= budgets + buf).all()

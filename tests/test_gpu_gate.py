@@ -1,0 +1,59 @@
+"""GPU parity of the fused retention gate (trimkv_gate_hidden + trimkv_append_gated) against the
+oracle's `rg` gate.  The fused path accumulates in fp32 and rounds where a bf16 module rounds, but
+in a different summation order than torch's bf16 GEMM, so log beta is compared with a tolerance
+(the selection itself is checked bit-exact elsewhere with injected log beta)."""
+import pytest
+import torch
+
+from oracle.attn_ref import retention_gate_rg
+from tests.gpu_util import DEV, draw_kv
+
+pytestmark = pytest.mark.gpu
+
+
+def _gate(hidden, heads, inter=512, seed=0, std=0.02, bias_init=3.0):
+    from trimkv_amd.gate import RetentionGate
+    torch.manual_seed(seed)
+    g = RetentionGate(hidden, heads, inter, bias_init=bias_init, initializer_range=std)
+    g.linear1.bias.data.normal_(0, 0.1)
+    return g.to(torch.bfloat16).eval()
+
+
+@pytest.mark.parametrize("B,S,hidden,heads", [(64, 1, 4096, 8), (3, 37, 2048, 8), (1, 200, 2560, 4)])
+def test_fused_gate_matches_oracle(B, S, hidden, heads):
+    from trimkv_amd import LazyLogBeta
+    g = _gate(hidden, heads, std=0.05)
+    x = torch.randn(B, S, hidden).to(torch.bfloat16)
+    w1, b1, w2, bias = g.linear1.weight.data, g.linear1.bias.data, g.linear2.weight.data, g.bias.data
+    want32 = retention_gate_rg(x.float(), w1.float(), b1.float(), w2.float(), bias.float())   # fp32 oracle
+    want16 = retention_gate_rg(x, w1, b1, w2, bias).float()                                       # the bf16 module itself
+    lazy = g.to(DEV)(x.to(DEV))
+    assert isinstance(lazy, LazyLogBeta) and lazy.shape == (B, S, heads)
+    got = lazy.materialize().float().cpu()
+    assert got.shape == (B, S, heads) and (got <= 0).all()
+    # bf16 has 8 bits of mantissa: the bf16 module is itself ~1e-2 relative away from fp32
+    tol = 3e-2 * want32.abs() + 2e-3
+    assert ((got - want32).abs() <= tol).all(), float((got - want32).abs().max())
+    assert (got - want16).abs().mean() <= (want16 - want32).abs().mean() * 2 + 1e-4  # no worse than the module's own rounding
+    assert g.training is False and torch.equal(g.to("cpu")(x), retention_gate_rg(x, w1, b1, w2, bias))  # CPU / non-fused path = torch expression
+
+
+def test_append_gated_writes_the_same_log_beta_as_materialize():
+    from trimkv_amd import TrimKVCache
+    B, H, S, hidden = 4, 8, 5, 2048
+    g = _gate(hidden, H, std=0.05).to(DEV)
+    gen = torch.Generator().manual_seed(1)
+    cache_a, cache_b = TrimKVCache(), TrimKVCache()
+    T = 0
+    for S in (5, 1, 1):
+        x = torch.randn(B, S, hidden, generator=gen).to(torch.bfloat16).to(DEV)
+        k, v = draw_kv(gen, B, H, S)
+        pos = torch.arange(T, T + S, device=DEV)
+        lazy = g(x).transpose(1, 2)          # what the attention module does with the gate output
+        cache_a.update(k.to(DEV), v.to(DEV), lazy, pos, 0)
+        cache_b.update(k.to(DEV), v.to(DEV), lazy.materialize(), pos, 0)
+        T += S
+    assert cache_a.retention_weights[0].dtype == torch.bfloat16
+    assert torch.equal(cache_a.retention_weights[0], cache_b.retention_weights[0])
+    assert torch.equal(cache_a.key_cache[0], cache_b.key_cache[0]) and torch.equal(cache_a.kv_positions[0], cache_b.kv_positions[0])
+    assert cache_a.get_cache_length(0) == 7
