@@ -231,7 +231,7 @@ def main():
         avg_s = sum(durs) / len(durs)
         avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
         achieved = avg_bytes / avg_s / 1e9
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}> (+ split-K merge)", "achieved": round(achieved, 1),
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}>" + ("" if B * Hkv >= 128 else " + decode_attn_merge_kernel"), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
                 "algorithmic_bytes_per_launch": int(avg_bytes)}

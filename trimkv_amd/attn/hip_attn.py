@@ -124,7 +124,8 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         q2 = query.reshape(B * Hq, D)  # [B,Hq,1,D]: row seg*G+g is query head h*G+g of batch b
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5)
+        out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5,
+                               chunk=kw.get("chunk", 0))
         return out.view(B, 1, Hq, D), None, None
     # prompt chunks: per-segment torch ops with the bottom-right causal mask of flash-attn's causal=True
     out = torch.zeros(B, Q, Hq, D, dtype=query.dtype, device=query.device)

@@ -513,8 +513,11 @@ class _RaggedCache(_SlabBacked):
             # arange(0, nseg*S+1, S), what the reference builds at cache_utils.py:297, 643
             self.n_seen_tokens[layer_idx] += S
         slab = self._slabs[layer_idx]
+        # split-K chunk for ragged lengths: about 512 workgroups over the rows actually cached
+        # (the library's own default assumes every segment is max_len long)
+        chunk = max(512, ((int(slab.lens.sum()) // 512 + 63) // 64) * 64)
         kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu,
-              "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len}
+              "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len, "chunk": chunk}
         flat = (slab.k.view(-1, slab.D), slab.v.view(-1, slab.D), slab.lb.view(-1, 1), slab.pos.view(-1, 1))
         return flat, kw
 

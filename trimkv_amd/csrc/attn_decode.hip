@@ -6,7 +6,8 @@
 //
 // The op is HBM-bound (about 4 flop per byte of K/V), so the kernel is built around the stream:
 //   * a wavefront reads whole 256-byte rows, 16 lanes x 16 bytes per row, 4 rows per load
-//     instruction (1 KiB contiguous), always with the next tile already in flight;
+//     instruction (1 KiB contiguous), with a ring of register buffers that keeps several tiles of
+//     its K/V stream in flight (the kernel is bound by bytes in flight over latency, not by ALU);
 //   * q.K uses v_dot2_f32_bf16 on the bytes as loaded; the 16-lane partial sums of one tile are
 //     reduced with a transposing DPP butterfly that leaves ONE (row, head) score per lane, so the
 //     softmax costs one exp per lane per tile;
@@ -15,8 +16,12 @@
 //     packed bf16 pairs, and P.V is v_dot2_f32_bf16 over two rows at a time (v_perm_b32
 //     interleaves the rows);
 //   * the four wavefronts of a workgroup own disjoint quarters of the workgroup's rows and merge
-//     (max, sum, accumulator) in LDS; workgroups of one segment merge in a second tiny kernel.
+//     (max, sum, accumulator) in LDS; with 512 segments or more one workgroup covers a whole
+//     segment and writes the output itself, otherwise segments are split and a second, tiny
+//     kernel merges the partials.
 #include "common.hip.h"
+
+#include <type_traits>
 
 namespace trimkv {
 
@@ -31,11 +36,16 @@ constexpr float AT_NEG = -1.0e30f;   // "minus infinity" that stays finite under
 
 template <int G>
 struct AttnCfg {
-    static constexpr int NJ = G <= 2 ? 8 : (G <= 4 ? 4 : 2);  // load instructions (of 4 rows) per tile
+    static constexpr int NJ = G <= 4 ? 4 : 2;                  // load instructions (of 4 rows) per tile
     static constexpr int NV = NJ * G;                          // scores per tile per 16-lane row group (<= 16)
     static constexpr int TILE_ROWS = NJ * 4;
     static constexpr int NT = AT_BLOCK_ROWS / TILE_ROWS;       // tiles per block
     static constexpr int PSTRIDE = NV <= 8 ? 8 : 16;           // bf16 slots per (tile, row group) in LDS
+#ifndef TRIMKV_AT_RING
+    static constexpr int RING = (NJ >= 4 || G >= 6) ? 4 : 8;   // register tile buffers: RING-1 tiles in flight per wavefront
+#else
+    static constexpr int RING = TRIMKV_AT_RING;
+#endif
 };
 
 typedef uint32_t __attribute__((may_alias)) u32_alias;  // LDS words written as bf16 halves, read as pairs
@@ -83,7 +93,7 @@ struct AttnArgs {
 };
 
 template <int G>
-__global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
+__global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2))) void decode_attn_kernel(AttnArgs a) {
     using C = AttnCfg<G>;
     constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
 
@@ -93,7 +103,13 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     __shared__ float sm[AT_WAVES][8];
     __shared__ float sl[AT_WAVES][8];
 
-    const int seg = blockIdx.y, split = blockIdx.x;
+    // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
+    // axis so that consecutive ids are different segments: with the split as the fast axis and 8
+    // splits, every "split 0" workgroup would land on the same XCD, and ragged lengths (most
+    // segments need one or two splits) would leave most of the chip idle.
+    // High splits exist only for the longest segments; they are dispatched first so that the few
+    // long segments do not form the tail of the launch.
+    const int seg = blockIdx.x, split = (int)gridDim.y - 1 - (int)blockIdx.y;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int nsp = (n + a.chunk - 1) / a.chunk;
@@ -115,9 +131,14 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     const uint4* kp = a.k + row0 * 16 + c;  // 16 uint4 per 256-byte row; this lane's 16-byte column
     const uint4* vp = a.v + row0 * 16 + c;
 
+    // q is loaded and waited for before the first K/V prefetch is issued: if its loads were still
+    // outstanding behind the prefetches, the wait for q at the first q.K (static code, executed by
+    // every block) would drain the whole prefetch ring each time.
     uint4 qv[G];
 #pragma unroll
     for (int g = 0; g < G; ++g) qv[g] = a.q[((int64_t)seg * G + g) * 16 + c];
+#pragma unroll
+    for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
 
     // which (row-in-tile, head) this lane owns after the transposing reduction
     const int my_x = ((c & 4) << 1) | ((c & 1) << 2) | (c & 2) | ((c & 8) >> 3);
@@ -134,7 +155,7 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     }
     float l_lane = 0.0f;
 
-    auto load_tile = [&](const uint4* base, int row_begin, uint4 (&dst)[NJ]) {
+    auto load_tile = [&](const uint4* base, int row_begin, uint4 (&dst)[NJ]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < NJ; ++j) {
             const int row = min(row_begin + j * 4 + r, w1 - 1);  // rows past the end re-read the last one (weight 0)
@@ -143,48 +164,46 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     };
 
     if (w0 < w1) {
-        // Two register buffers per operand, indexed by tile parity (the tile loops are fully
-        // unrolled, so the parity is static): while tile t is being consumed, tile t+1 -- or the
-        // first tile of the next phase -- is in flight.  NT is even, so tile 0 always sits in [0].
-        uint4 kb[2][NJ], vb[2][NJ];
-        load_tile(kp, w0, kb[0]);
-#pragma unroll 1
-        for (int blk = w0; blk < w1; blk += AT_BLOCK_ROWS) {
-            const int nrows = min(AT_BLOCK_ROWS, w1 - blk);
-            float s[NT];
-            // ---- scores of up to 128 rows ----
+        // The wavefront consumes one stream of tiles: for every block of up to 128 rows, its K tiles
+        // (slots 0..NT-1) and then its V tiles (slots NT..2NT-1).  A ring of RING register buffers,
+        // indexed by slot % RING (static: the slot loop is fully unrolled and 2*NT is a multiple of
+        // RING), keeps the next RING-1 tiles of that stream in flight while one is consumed -- K and
+        // V alike, across the softmax and across block boundaries.  Bandwidth here is bytes in
+        // flight over latency, and registers are the cheapest place to park them.
+        constexpr int RING = C::RING, PD = RING - 1;
+        uint4 ring[RING][NJ];
+        float s[NT];
+        float m_mine = AT_NEG;
+        u16_alias* pw16 = (u16_alias*)&p_lds[w][0][0][0];
+
+        auto scores_of_tile = [&](int t, int blk, const uint4 (&kt)[NJ]) __attribute__((always_inline)) {
+            float part[16];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                s[t] = AT_NEG;
-                if (t * TILE_ROWS < nrows) {
-                    if (t + 1 < NT && (t + 1) * TILE_ROWS < nrows) load_tile(kp, blk + (t + 1) * TILE_ROWS, kb[(t + 1) & 1]);
-                    else load_tile(vp, blk, vb[0]);
-                    float part[16];
+            for (int x = 0; x < 16; ++x) part[x] = 0.0f;
 #pragma unroll
-                    for (int x = 0; x < 16; ++x) part[x] = 0.0f;
+            for (int j = 0; j < NJ; ++j) {
 #pragma unroll
-                    for (int j = 0; j < NJ; ++j) {
-#pragma unroll
-                        for (int g = 0; g < G; ++g) {
-                            float acc = dot2_bf16(kb[t & 1][j].x, qv[g].x, 0.0f);
-                            acc = dot2_bf16(kb[t & 1][j].y, qv[g].y, acc);
-                            acc = dot2_bf16(kb[t & 1][j].z, qv[g].z, acc);
-                            acc = dot2_bf16(kb[t & 1][j].w, qv[g].w, acc);
-                            part[j * G + g] = acc;
-                        }
-                    }
-                    const float val = reduce16_transposed(part, c);
-                    const int row = blk + t * TILE_ROWS + my_j * 4 + r;
-                    if (my_valid && row < w1) s[t] = val * a.scale_log2;
+                for (int g = 0; g < G; ++g) {
+                    float acc = dot2_bf16(kt[j].x, qv[g].x, 0.0f);
+                    acc = dot2_bf16(kt[j].y, qv[g].y, acc);
+                    acc = dot2_bf16(kt[j].z, qv[g].z, acc);
+                    acc = dot2_bf16(kt[j].w, qv[g].w, acc);
+                    part[j * G + g] = acc;
                 }
             }
-            // ---- running max, probabilities ----
+            const float val = reduce16_transposed(part, c);
+            const int row = blk + t * TILE_ROWS + my_j * 4 + r;
+            return (my_valid && row < w1) ? val * a.scale_log2 : AT_NEG;
+        };
+        // ntiles: tiles of this block that were scored (the rest of s[] is not read)
+        auto softmax_of_block = [&](auto ntb_c, int nrows) __attribute__((always_inline)) {
+            constexpr int NTB = decltype(ntb_c)::value;
             float lmax = AT_NEG;
 #pragma unroll
-            for (int t = 0; t < NT; ++t) lmax = fmaxf(lmax, s[t]);
+            for (int t = 0; t < NTB; ++t) lmax = fmaxf(lmax, s[t]);
             if (lane < 8) smax[w][lane] = float_key(AT_NEG);
             if (my_valid) atomicMax(&smax[w][my_g], float_key(lmax));
-            float alpha_mine = 1.0f, m_mine = AT_NEG;
+            float alpha_mine = 1.0f;
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 const float mb = key_float(smax[w][g]);
@@ -196,43 +215,95 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
                 if (g == my_g) { alpha_mine = alpha; m_mine = m_new; }
             }
             l_lane *= alpha_mine;
-            u16_alias* pw16 = (u16_alias*)&p_lds[w][0][0][0];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
+            for (int t = 0; t < NTB; ++t) {
                 if (t * TILE_ROWS < nrows) {
                     const float p = my_valid ? __builtin_amdgcn_exp2f(s[t] - m_mine) : 0.0f;
                     l_lane += p;
                     if (my_valid) pw16[(t * 4 + r) * PS + my_g * NJ + my_j] = f32_to_bf16_bits(p);
                 }
             }
-            // ---- P.V over the same rows ----
+        };
+        auto accumulate_tile = [&](int t, const uint4 (&vt)[NJ]) __attribute__((always_inline)) {
+            uint32_t pd[NV / 2];
 #pragma unroll
-            for (int t = 0; t < NT; ++t) {
-                if (t * TILE_ROWS < nrows) {
-                    if (t + 1 < NT && (t + 1) * TILE_ROWS < nrows) load_tile(vp, blk + (t + 1) * TILE_ROWS, vb[(t + 1) & 1]);
-                    else if (blk + AT_BLOCK_ROWS < w1) load_tile(kp, blk + AT_BLOCK_ROWS, kb[0]);
-                    uint32_t pd[NV / 2];
+            for (int i = 0; i < NV / 2; ++i) pd[i] = p_lds[w][t][r][i];
 #pragma unroll
-                    for (int i = 0; i < NV / 2; ++i) pd[i] = p_lds[w][t][r][i];
+            for (int u = 0; u < NJ / 2; ++u) {
+                const uint4 ra = vt[2 * u], rb = vt[2 * u + 1];
+                const uint32_t va[4] = {ra.x, ra.y, ra.z, ra.w};
+                const uint32_t vv[4] = {rb.x, rb.y, rb.z, rb.w};
 #pragma unroll
-                    for (int u = 0; u < NJ / 2; ++u) {
-                        const uint4 ra = vb[t & 1][2 * u], rb = vb[t & 1][2 * u + 1];
-                        const uint32_t va[4] = {ra.x, ra.y, ra.z, ra.w};
-                        const uint32_t vv[4] = {rb.x, rb.y, rb.z, rb.w};
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t lo = __builtin_amdgcn_perm(vv[i], va[i], 0x05040100u);  // rows (2u, 2u+1), element 2i
+                    const uint32_t hi = __builtin_amdgcn_perm(vv[i], va[i], 0x07060302u);  // rows (2u, 2u+1), element 2i+1
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const uint32_t lo = __builtin_amdgcn_perm(vv[i], va[i], 0x05040100u);  // rows (2u, 2u+1), element 2i
-                            const uint32_t hi = __builtin_amdgcn_perm(vv[i], va[i], 0x07060302u);  // rows (2u, 2u+1), element 2i+1
-#pragma unroll
-                            for (int g = 0; g < G; ++g) {
-                                const uint32_t pp = pd[(g * NJ) / 2 + u];
-                                o[g][2 * i] = dot2_bf16(lo, pp, o[g][2 * i]);
-                                o[g][2 * i + 1] = dot2_bf16(hi, pp, o[g][2 * i + 1]);
-                            }
-                        }
+                    for (int g = 0; g < G; ++g) {
+                        const uint32_t pp = pd[(g * NJ) / 2 + u];
+                        o[g][2 * i] = dot2_bf16(lo, pp, o[g][2 * i]);
+                        o[g][2 * i + 1] = dot2_bf16(hi, pp, o[g][2 * i + 1]);
                     }
                 }
             }
+        };
+
+        // One block of NTB tiles (NTB*TILE_ROWS rows, `nrows` of them real) as straight-line code:
+        // slots 0..NTB-1 are its K tiles, NTB..2NTB-1 its V tiles.  Loads are never placed under a
+        // branch: the compiler can count outstanding loads exactly (s_waitcnt vmcnt(N), N > 0:
+        // "wait for this tile, leave the prefetched ones in flight") only when every path issues
+        // the same loads.  Rows are clamped to the wavefront's last row, so a load past the end is
+        // legal and re-reads cached bytes; its scores are masked.
+        // CHAINED: the first PD slots are already in flight and the block prefetches the first PD
+        // slots of the block that follows it (the steady-state loop over full blocks).
+        auto run_block = [&](auto ntb_c, auto chained_c, int blk, int nrows) __attribute__((always_inline)) {
+            constexpr int NTB = decltype(ntb_c)::value;
+            constexpr bool CHAINED = decltype(chained_c)::value;
+            constexpr int SL = 2 * NTB;
+            static_assert(!CHAINED || (SL % RING == 0 && PD <= NTB), "chained blocks need ring-aligned slots");
+            auto load_slot = [&](int slot, int base_row, uint4 (&dst)[NJ]) __attribute__((always_inline)) {
+                if (slot < NTB) load_tile(kp, base_row + slot * TILE_ROWS, dst);
+                else load_tile(vp, base_row + (slot - NTB) * TILE_ROWS, dst);
+            };
+            if (!CHAINED) {
+#pragma unroll
+                for (int sl = 0; sl < (PD < SL ? PD : SL); ++sl) load_slot(sl, blk, ring[sl % RING]);
+            }
+#pragma unroll
+            for (int sl = 0; sl < SL; ++sl) {
+                const int ahead = sl + PD;
+                if (ahead < SL) load_slot(ahead, blk, ring[ahead % RING]);
+                else if (CHAINED) load_slot(ahead - SL, blk + NTB * TILE_ROWS, ring[ahead % RING]);
+                // keep the prefetch where it is: left alone, the scheduler sinks these loads past
+                // the arithmetic to shorten live ranges, which empties the pipeline
+                __builtin_amdgcn_sched_barrier(0);
+                if (sl == NTB) softmax_of_block(ntb_c, nrows);
+                if (sl < NTB) {
+                    s[sl] = scores_of_tile(sl, blk, ring[sl % RING]);
+                } else if (CHAINED || (sl - NTB) * TILE_ROWS < nrows) {
+                    accumulate_tile(sl - NTB, ring[sl % RING]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        using std::integral_constant;
+        using std::true_type;
+        using std::false_type;
+
+#pragma unroll
+        for (int sl = 0; sl < PD; ++sl) load_tile(kp, w0 + sl * TILE_ROWS, ring[sl % RING]);
+        int blk = w0;
+#pragma unroll 1
+        for (; blk + AT_BLOCK_ROWS <= w1; blk += AT_BLOCK_ROWS)
+            run_block(integral_constant<int, NT>{}, true_type{}, blk, AT_BLOCK_ROWS);
+        // the tail (< 128 rows): the smallest power-of-two block that covers it, one pipelined pass
+        const int rest = w1 - blk;
+        if (rest > 0) {
+            const int need = (rest + TILE_ROWS - 1) / TILE_ROWS;  // 1 .. NT tiles
+            if (need <= 1) run_block(integral_constant<int, 1>{}, false_type{}, blk, rest);
+            else if (need <= 2) run_block(integral_constant<int, 2>{}, false_type{}, blk, rest);
+            else if (need <= 4) run_block(integral_constant<int, 4>{}, false_type{}, blk, rest);
+            else if (need <= 8) run_block(integral_constant<int, (NT >= 8 ? 8 : NT)>{}, false_type{}, blk, rest);
+            else run_block(integral_constant<int, NT>{}, false_type{}, blk, rest);
         }
     }
 
@@ -284,43 +355,64 @@ __global__ __launch_bounds__(AT_THREADS) void decode_attn_kernel(AttnArgs a) {
     }
 }
 
+// Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
+// splits first (independent loads), then the accumulators.  A separate launch on purpose: the
+// kernel boundary is what makes partials written on one XCD visible on another; doing the same
+// inside one kernel needs device-scope fences (an L2 write-back and invalidate per workgroup on
+// this part), which costs far more than the launch.
 template <int G>
-__global__ __launch_bounds__(AT_D) void decode_attn_merge_kernel(AttnArgs a) {
-    const int seg = blockIdx.x, d = threadIdx.x;
+__global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
+    const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int nsp = (n + a.chunk - 1) / a.chunk;
+    const int64_t slot0 = ((int64_t)seg * a.nsplit) * G + g;
+    float mx = AT_NEG;
+    for (int sp = 0; sp < nsp; ++sp) mx = fmaxf(mx, a.ws_ml[(slot0 + (int64_t)sp * G) * 2]);
+    float acc = 0.0f, lsum = 0.0f;
+    int sp = 0;
+    for (; sp + 4 <= nsp; sp += 4) {
+        float m4[4], l4[4], o4[4];
 #pragma unroll
-    for (int g = 0; g < G; ++g) {
-        float mx = AT_NEG;
-        for (int s = 0; s < nsp; ++s) mx = fmaxf(mx, a.ws_ml[(((int64_t)seg * a.nsplit + s) * G + g) * 2]);
-        float acc = 0.0f, lsum = 0.0f;
-        for (int s = 0; s < nsp; ++s) {
-            const int64_t slot = ((int64_t)seg * a.nsplit + s) * G + g;
-            const float f = __builtin_amdgcn_exp2f(a.ws_ml[slot * 2] - mx);
-            acc += f * a.ws_o[slot * AT_D + d];
-            lsum += f * a.ws_ml[slot * 2 + 1];
+        for (int u = 0; u < 4; ++u) {
+            const int64_t slot = slot0 + (int64_t)(sp + u) * G;
+            m4[u] = a.ws_ml[slot * 2];
+            l4[u] = a.ws_ml[slot * 2 + 1];
+            o4[u] = a.ws_o[slot * AT_D + d];
         }
-        const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-        ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const float f = __builtin_amdgcn_exp2f(m4[u] - mx);
+            acc += f * o4[u];
+            lsum += f * l4[u];
+        }
     }
+    for (; sp < nsp; ++sp) {
+        const int64_t slot = slot0 + (int64_t)sp * G;
+        const float f = __builtin_amdgcn_exp2f(a.ws_ml[slot * 2] - mx);
+        acc += f * a.ws_o[slot * AT_D + d];
+        lsum += f * a.ws_ml[slot * 2 + 1];
+    }
+    const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+    ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
 }
 
 static int pick_chunk(int nseg, int max_len) {
-    // Aim for about 8 workgroups per CU (256 CUs) so the tail of the grid is short, but keep a
-    // workgroup's share at 256 rows or more so the merge traffic stays below 1 % of the K/V bytes.
-    const int64_t rows = (int64_t)nseg * max_len;
-    int64_t chunk = (rows + 2047) / 2048;
-    chunk = ((chunk + 127) / 128) * 128;
-    if (chunk < 256) chunk = 256;
-    if (chunk > 2048) chunk = 2048;
-    return (int)chunk;
+    // One workgroup per segment streams at full rate already with 128 segments (a workgroup keeps
+    // 12 tiles in flight); with fewer, segments are cut so that about 256 workgroups exist, but
+    // not below 512 rows each (one full block per wavefront).
+    const int whole = ((max_len + 63) / 64) * 64;
+    if (nseg >= 128) return whole;
+    const int nsplit = (256 + nseg - 1) / nseg;
+    int chunk = (((max_len + nsplit - 1) / nsplit + 63) / 64) * 64;
+    if (chunk < 512) chunk = 512;
+    return chunk < whole ? chunk : whole;
 }
 
 template <int G>
 static void launch_attn(const AttnArgs& a, hipStream_t st) {
-    hipLaunchKernelGGL(decode_attn_kernel<G>, dim3(a.nsplit, a.nseg), dim3(AT_THREADS), 0, st, a);
-    if (!a.direct) hipLaunchKernelGGL(decode_attn_merge_kernel<G>, dim3(a.nseg), dim3(AT_D), 0, st, a);
+    hipLaunchKernelGGL(decode_attn_kernel<G>, dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
+    if (!a.direct) hipLaunchKernelGGL(decode_attn_merge_kernel<G>, dim3(a.nseg), dim3(G * AT_D), 0, st, a);
 }
 
 }  // namespace trimkv
@@ -345,7 +437,6 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     if (head_dim != AT_D) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be %d (got %d)", fn, AT_D, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
-    if (nseg > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nseg=%d exceeds the grid limit 65535", fn, nseg);
     if (!seg_start && max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
     if (((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_slab | (uintptr_t)v_slab) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: q/out/K/V must be 16-byte aligned", fn);
     if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
@@ -354,12 +445,14 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     a.q = (const uint4*)q; a.out = out; a.k = (const uint4*)k_slab; a.v = (const uint4*)v_slab;
     a.seg_len = seg_len; a.seg_start = seg_start; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
     a.nsplit = (max_len + chunk - 1) / chunk;
+    if (a.nsplit > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: max_len/chunk = %d splits exceeds the grid limit 65535", fn, a.nsplit);
     a.direct = a.nsplit <= 1;
     a.scale_log2 = scale * 1.4426950408889634f;
     a.ws_o = nullptr; a.ws_ml = nullptr;
     if (!a.direct) {
         const size_t need = trimkv_decode_attn_workspace(nseg, group, head_dim, max_len, chunk);
         if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+        if ((uintptr_t)workspace & 15) return fail(TRIMKV_ERR_SHAPE, "%s: workspace must be 16-byte aligned", fn);
         a.ws_o = (float*)workspace;
         a.ws_ml = a.ws_o + (size_t)nseg * a.nsplit * group * AT_D;
     }
