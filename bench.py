@@ -50,6 +50,20 @@ def algorithmic_bytes(c):
     return dict(attn=attn_kv + attn_qo, append=append, evict=evict, step=c["L"] * (attn_kv + attn_qo + append + evict))
 
 
+def measured_traffic_ratio():
+    """HBM bytes per attention launch over algorithmic bytes, as measured with rocprofv3 --pmc
+    FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known size); the summary of those two runs
+    is committed under profiles/ and carries the ratio on a `traffic_over_algorithmic:` line."""
+    path = os.path.join(ROOT, "profiles", "decode_attn_config3_pmc_traffic.md")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_over_algorithmic:"):
+                return float(line.split(":")[1]), os.path.relpath(path, ROOT)
+    except OSError:
+        pass
+    return None, None
+
+
 def cpu_baseline(c, budget_s=20.0):
     """The oracle (the reference's pure-PyTorch CPU path restated) on ONE layer at full shape,
     extrapolated to the full step: t_step = L * (B / b) * (t_append_attend + t_evict / buffer)."""
@@ -140,6 +154,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers (smoke runs only; makes the result invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--event-every", type=int, default=8, help="sample attention launches with HIP events every N steps")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy (a kernel of known traffic) so that rocprofv3 --pmc "
+                         "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: the path shards by batch or KV head without communication, "
@@ -190,6 +207,13 @@ def main():
                         torch.randn(B, Hq, 1, D, generator=gen, device=dev).to(torch.bfloat16)))
         pool.append(per)
     torch.cuda.synchronize()
+    if args.calibrate_copy:  # 2**30 bytes read + 2**30 bytes written by one elementwise kernel
+        src = torch.empty(2 ** 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     T = n0
     events = []
@@ -231,8 +255,10 @@ def main():
         avg_s = sum(durs) / len(durs)
         avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
         achieved = avg_bytes / avg_s / 1e9
+        ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
         roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}>" + ("" if B * Hkv >= 128 else " + decode_attn_merge_kernel"), "achieved": round(achieved, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
                 "algorithmic_bytes_per_launch": int(avg_bytes)}
     parity = parity_gate(cache, c, attn_fn, mod)
