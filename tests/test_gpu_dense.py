@@ -32,7 +32,7 @@ def _same_state(cache, ref, layers):
 
 
 def _run(B, Hkv, G, L, prefill, steps, M, buf, seed, lb_dtype=torch.float32, strategy="alpha", attend_every=1,
-         chunks=None, sigma=1.0):
+         chunks=None, sigma=1.0, snapshots=None):
     from trimkv_amd import TrimKVCache, get_attention_interface
     attn = get_attention_interface("trimkv_hip")
     gen = torch.Generator().manual_seed(seed)
@@ -70,6 +70,8 @@ def _run(B, Hkv, G, L, prefill, steps, M, buf, seed, lb_dtype=torch.float32, str
         if ref.get_cache_length(0) != before:
             evictions += 1
             _same_state(cache, ref, range(L))
+            if snapshots is not None:
+                snapshots.append(cache.kv_positions[0].cpu().numpy())
 
     for S in (chunks or [prefill]):
         step(S, False)
@@ -83,9 +85,16 @@ def _run(B, Hkv, G, L, prefill, steps, M, buf, seed, lb_dtype=torch.float32, str
 def test_parity_config_1_single_layer_qwen3_1p7b_shape():
     """BASELINE config 1: B=1, 8 KV heads, 16 query heads, D=128, M=512, buffer 128, 1024-token prefill,
     4096 decode steps; retained index set checked bit-exact after each of the 1 + 32 evictions."""
-    ev, worst = _run(B=1, Hkv=8, G=2, L=1, prefill=1024, steps=4096, M=512, buf=128, seed=1, attend_every=16)
+    import os
+    snaps = []
+    ev, worst = _run(B=1, Hkv=8, G=2, L=1, prefill=1024, steps=4096, M=512, buf=128, seed=1, attend_every=16, snapshots=snaps)
     assert ev == 33
     assert worst < 2e-2
+    # and against the committed golden vectors (tests/golden/make_golden.py)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "config1_retained_positions.npz"))["positions"]
+    assert gold.shape == (33, 8, 512)
+    for i, got in enumerate(snaps):
+        assert np.array_equal(got[0].astype(np.int64), gold[i].astype(np.int64)), f"eviction {i} differs from the golden vectors"
 
 
 def test_multi_layer_batch_gqa4():

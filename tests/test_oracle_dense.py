@@ -211,3 +211,20 @@ def test_parity_config_matches_numpy_simulation():
     assert len(got) == len(want) == 1 + steps // buf
     for a, b in zip(got, want):
         assert np.array_equal(a, b)
+
+
+def test_oracle_reproduces_the_committed_golden_vectors():
+    """tests/golden/config1_retained_positions.npz: BASELINE config 1 in full (33 evictions)."""
+    import importlib.util
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    spec = importlib.util.spec_from_file_location("make_golden", os.path.join(here, "golden", "make_golden.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    gold = np.load(os.path.join(here, "golden", "config1_retained_positions.npz"))
+    assert gold["meta"].tolist() == [mod.SEED, mod.B, mod.H, mod.M, mod.BUF, mod.PREFILL, mod.STEPS]
+    got = mod.run()
+    assert got.shape == gold["positions"].shape == (33, 8, 512)
+    assert np.array_equal(got, gold["positions"])
+    last = gold["positions"][-1].astype(np.int64)
+    assert (np.diff(last, axis=1) > 0).all() and last.max() < 1024 + 4096
