@@ -207,6 +207,26 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
                        int nseg, int cap, int head_dim, int group, int dtype, float scale,
                        int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * trimkv_prefill_attn -- GQA attention of a block of q_len queries (a prompt or prompt chunk)
+ * over every segment's retained K/V, bottom-right causal: query t sees keys j <= n - q_len + t,
+ * n = seg_len[seg] (the chunk's own tokens are already appended).  A query that sees no key
+ * yields zeros.
+ * Replaces flash_attn_varlen_func with causal=True at Q_LEN > 1 (src/trimkv/attn/flash_attn.py:
+ * 61-71, 135-145) and HF flash_attention_2 on the dense cache during prefill
+ * (src/trimkv/attn/__init__.py:15-26).
+ *
+ * q is [batch][kv_heads*group][q_len][head_dim] with ELEMENT strides q_stride_b/h/t (head_dim
+ * contiguous, strides multiples of 8); out is [batch][q_len][kv_heads*group][head_dim],
+ * contiguous.  Segment batch b, kv head h is attended by query heads h*group .. h*group+group-1
+ * (flash_attn.py:120-125).  K/V rows as in trimkv_decode_attn (seg_start or seg*cap; seg_len may be
+ * NULL for a dense cache of max_len rows).  head_dim must be 128; group in [1, 8]; dtype bf16.
+ */
+int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t, void* out,
+                        const void* k_slab, const void* v_slab, const int32_t* seg_len, const int32_t* seg_start,
+                        int batch, int kv_heads, int group, int q_len, int cap, int head_dim, int dtype, float scale,
+                        int max_len, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -57,6 +57,25 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
     return out
 
 
+def prefill_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, batch: int, kv_heads: int, group: int,
+                      seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
+                      scale: float) -> torch.Tensor:
+    """``query`` [B, Hq, Q, D] (any strides with D contiguous) -> [B, Q, Hq, D], bottom-right causal."""
+    if not query.is_cuda:
+        raise _lib.TrimKVLibraryError("prefill attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
+    lib = _lib.load()
+    B, Hq, Q, D = query.shape
+    if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
+        query = query.contiguous()
+    out = torch.empty(B, Q, Hq, D, dtype=query.dtype, device=query.device)
+    rc = lib.trimkv_prefill_attn(query.data_ptr(), query.stride(0), query.stride(1), query.stride(2), out.data_ptr(),
+                                 k_rows.data_ptr(), v_rows.data_ptr(), _lib.ptr(seg_len), _lib.ptr(seg_start),
+                                 batch, kv_heads, group, Q, cap, D, _lib.dtype_code(query.dtype), float(scale), max_len,
+                                 _lib.current_stream(query.device))
+    _lib.check(rc, "trimkv_prefill_attn")
+    return out
+
+
 def _causal_bottom_right(qlen: int, n: int, device) -> torch.Tensor:
     t = torch.arange(qlen, device=device)[:, None]
     j = torch.arange(n, device=device)[None, :]
@@ -85,7 +104,17 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             seg_len = None
         out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale)
         return out.view(B, 1, Hq, D), None, None
-    # prompt chunks and masked batches: torch ops (bottom-right causal, as flash-attn aligns it)
+    if attention_mask is None and query.dtype == torch.bfloat16 and D == 128:
+        ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
+              and value.stride() == key.stride() and key.stride(1) % D == 0)
+        if not ok:
+            key, value = key.contiguous(), value.contiguous()
+        seg_len = (flash_attn_kwargs or {}).get("seg_len")
+        if seg_len is not None and (seg_len.numel() != B * Hkv or (flash_attn_kwargs or {}).get("max_len") != n):
+            seg_len = None
+        out = prefill_attention(query, key, value, B, Hkv, G, seg_len, None, key.stride(1) // D, n, scale)
+        return out, None, None
+    # masked batches (padding): torch ops
     k = key.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
     v = value.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
     w = torch.matmul(query, k.transpose(2, 3)).float() * scale
@@ -127,22 +156,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5,
                                chunk=kw.get("chunk", 0))
         return out.view(B, 1, Hq, D), None, None
-    # prompt chunks: per-segment torch ops with the bottom-right causal mask of flash-attn's causal=True
-    out = torch.zeros(B, Q, Hq, D, dtype=query.dtype, device=query.device)
-    starts = seg_start.tolist()
-    lens = head_lens.tolist()
-    for seg in range(nseg):
-        b, h = divmod(seg, num_kv_heads)
-        n = lens[seg]
-        if n == 0:
-            continue
-        k = key[starts[seg]:starts[seg] + n].float()
-        v = value[starts[seg]:starts[seg] + n].float()
-        qs = query[b, h * G:(h + 1) * G].float()
-        s = torch.einsum("gqd,nd->gqn", qs, k) * (D ** -0.5)
-        s = s.masked_fill(~_causal_bottom_right(Q, n, query.device), float("-inf"))
-        p = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
-        out[b, :, h * G:(h + 1) * G] = torch.einsum("gqn,nd->qgd", p, v).to(query.dtype)
+    out = prefill_attention(query, key, value, batch_size, num_kv_heads, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5)
     return out, None, None
 
 
