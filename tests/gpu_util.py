@@ -25,7 +25,7 @@ def boundary_ties(log_beta, positions, q_idx, keep):
 
 def attn_close(got, want, atol=2e-2, rtol=1e-2):
     """The north-star tolerance: max-abs 2e-2 and relative 1e-2 against the fp32 reference."""
-    got, want = got.float().cpu(), want.float().cpu()
+    got, want = got.detach().float().cpu(), want.detach().float().cpu()
     err = (got - want).abs()
     ok = bool((err <= atol + rtol * want.abs()).all())
     return ok, float(err.max())
