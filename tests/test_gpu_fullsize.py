@@ -168,3 +168,62 @@ def test_config4_ragged_lognormal_budgets():
     for seg, p in enumerate(cache.segment_positions()[0]):
         assert p.numel() == lens[seg] and (p[1:] > p[:-1]).all()
     assert hit.sum() == 0 and (lens <= budgets + buf).all()
+
+
+def test_config5_long_prompt_streamed_in_chunks_then_decode():
+    """BASELINE config 5 pattern at its real lengths for one layer and one sequence: a 131072-token prompt in
+    32 chunks of 4096 (append -> chunk attention over the retained KV -> evict to M=8192 once 8704 are
+    held), then decode steps.  Every eviction is checked against torch.topk on the device, the chunk
+    attention of sampled queries against fp32."""
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    B, H, G, D, M, buf, S = 1, 8, 5, 128, 8192, 512, 4096
+    gen = torch.Generator(device=DEV).manual_seed(55)
+    cache = TrimKVCache()
+    attn = get_attention_interface("trimkv_hip")
+    T = 0
+    evictions = 0
+    rows = torch.tensor([0, 17, 2048, 4095], device=DEV)
+    for chunk in range(32):
+        k = torch.randn(B, H, S, D, generator=gen, device=DEV).to(torch.bfloat16)
+        v = torch.randn(B, H, S, D, generator=gen, device=DEV).to(torch.bfloat16)
+        lb = torch.nn.functional.logsigmoid(torch.randn(B, H, S, generator=gen, device=DEV) * 2.0 + 2.0)
+        q = torch.randn(B, H * G, S, D, generator=gen, device=DEV).to(torch.bfloat16)
+        K, V, LB, POS, kw = cache.update(k, v, lb, torch.arange(T, T + S, device=DEV), 0)
+        T += S
+        n = K.shape[2]
+        assert n == min(T, M + S) and POS.shape == (B, H, n)
+        out, _, _ = attn(_Mod(), q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+        if chunk in (0, 1, 2, 31):
+            for h in (0, 7):
+                for g in (0, 4):
+                    s = (q[0, h * G + g, rows].float() @ K[0, h].float().T) * D ** -0.5
+                    vis = torch.arange(n, device=DEV)[None, :] <= (n - S + rows)[:, None]
+                    want = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ V[0, h].float()
+                    ok, err = attn_close(out[0, rows, h * G + g], want)
+                    assert ok, (chunk, h, g, err)
+        if n >= M + buf:
+            sc = LB.float() * (T + 1 - POS)
+            top = torch.topk(sc, M + 1, dim=-1).values
+            assert not (top[..., M - 1] == top[..., M]).any()
+            want_pos = torch.gather(POS, -1, torch.sort(torch.topk(sc, M, dim=-1).indices, dim=-1).values)
+            want_k = None
+        cache.compress("alpha", M, buf)
+        if n >= M + buf:
+            evictions += 1
+            assert cache.get_cache_length(0) == M and torch.equal(cache.kv_positions[0], want_pos)
+    assert evictions == 30 and cache.get_seq_length() == 131072      # chunks 1-2 stay below M + buffer
+    assert cache._slabs[0].cap <= 2 * (M + S)                         # the slab never grew past what a chunk needs
+    dec = get_attention_interface("trimkv_hip")
+    for t in range(8):
+        k = torch.randn(B, H, 1, D, generator=gen, device=DEV).to(torch.bfloat16)
+        v = torch.randn(B, H, 1, D, generator=gen, device=DEV).to(torch.bfloat16)
+        lb = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) * 2.0 + 2.0)
+        q = torch.randn(B, H * G, 1, D, generator=gen, device=DEV).to(torch.bfloat16)
+        K, V, _, _, kw = cache.update(k, v, lb, torch.arange(T, T + 1, device=DEV), 0)
+        T += 1
+        out, _, _ = dec(_Mod(), q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+        p = torch.softmax(torch.einsum("hgd,hnd->hgn", q.view(H, G, D).float(), K[0].float()) * D ** -0.5, -1)
+        ok, err = attn_close(out.view(H, G, D), torch.einsum("hgn,hnd->hgd", p, V[0].float()))
+        assert ok, err
+        cache.compress("alpha", M, buf)
+    assert cache.get_cache_length(0) == M + 8

@@ -41,7 +41,7 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     const uint16_t* wp = a.w1 + (int64_t)unit * a.hidden + ks * kspan + kg * 8;
 
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 8
+#pragma unroll 2
     for (int k = 0; k < kspan; k += 32) {
         const bf16x8_t av = *(const bf16x8_t*)(xp + k);
         const bf16x8_t bv = *(const bf16x8_t*)(wp + k);
