@@ -154,6 +154,11 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers (smoke runs only; makes the result invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--event-every", type=int, default=8, help="sample attention launches with HIP events every N steps")
+    ap.add_argument("--gate", action="store_true",
+                    help="produce log beta with the fused `rg` retention gate (MFMA first linear + epilogue inside the append "
+                         "kernel) from a random hidden state per layer instead of appending drawn values; reported as a "
+                         "variant, the BASELINE configs draw beta directly")
+    ap.add_argument("--hidden", type=int, default=4096, help="hidden size for --gate (Qwen3-8B: 4096)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
@@ -194,8 +199,17 @@ def main():
         k = torch.randn(B, Hkv, n0, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
         v = torch.randn(B, Hkv, n0, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
         lb = torch.nn.functional.logsigmoid(torch.randn(B, Hkv, n0, generator=gen, device=dev) * c["sigma"] + c["mu"])
+        if args.gate:
+            lb = lb.to(torch.bfloat16)   # the gate emits log beta in the model dtype
         cache.update(k, v, lb, pos0, l)
         del k, v, lb
+    gates, hidden_pool = [], []
+    if args.gate:
+        from trimkv_amd.gate import RetentionGate
+        torch.manual_seed(0)
+        for l in range(L):
+            gates.append(RetentionGate(args.hidden, Hkv, 512, bias_init=3.0, initializer_range=0.02).to(torch.bfloat16).to(dev).eval())
+            hidden_pool.append(torch.randn(B, 1, args.hidden, generator=gen, device=dev).to(torch.bfloat16))
     POOL = 4
     pool = []
     for l in range(L):
@@ -223,6 +237,8 @@ def main():
         pos = torch.full((1,), T, dtype=torch.int64, device=dev)
         for l in range(L):
             kn, vn, lbn, q = pool[l][t % POOL]
+            if args.gate:
+                lbn = gates[l](hidden_pool[l]).transpose(1, 2)   # LazyLogBeta: finished inside the append kernel
             K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
             if sample:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -277,6 +293,9 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(c)
+    if args.gate:
+        out["config"]["variant"] = (f"log beta from the fused rg gate (hidden {args.hidden}, intermediate 512, bf16) "
+                                    "instead of drawn values: not the BASELINE configuration")
     if args.layers:
         out["config"]["note"] = "layer count overridden: not the BASELINE configuration"
     print(json.dumps(out))

@@ -12,11 +12,11 @@ from torch import nn
 from oracle.attn_ref import eager_attention, ragged_attention
 from oracle.dense_ref import DenseCacheRef
 from oracle.ragged_ref import BatchedRaggedCacheRef
-from tests.gpu_util import DEV, attn_close
+from tests.gpu_util import DEV, attn_close, boundary_ties
 
 pytestmark = pytest.mark.gpu
 
-HID, HQ, HKV, D, LAYERS = 256, 8, 2, 128, 2
+HID, HQ, HKV, D, LAYERS = 512, 8, 2, 128, 2
 
 
 class Block(nn.Module):
@@ -102,6 +102,9 @@ def test_attention_block_call_order(kind):
             assert ok, f"T={T} layer {l}: attention error {err}"
         T += S
         before = ref.get_total_cached_tokens() if kind == "ragged" else ref.get_cache_length(0)
+        ties = None
+        if kind == "dense" and before >= M + buf:  # bf16 log beta: lb*age collides easily, so cuts do tie
+            ties = [boundary_ties(ref.retention_weights[l], ref.kv_positions[l], ref.get_seq_length(l) + 1, M) for l in range(LAYERS)]
         args = dict(strategy=strategy, memory_size=M, buffer_size=buf, floor_budget_ratio=0.0, alpha_threshold=0.0,
                     num_layers=LAYERS, num_key_value_heads=HKV)
         ref.compress(**args)
@@ -109,8 +112,17 @@ def test_attention_block_call_order(kind):
         after = ref.get_total_cached_tokens() if kind == "ragged" else ref.get_cache_length(0)
         evictions += before != after
         if kind == "dense":
-            for l in range(LAYERS):  # bf16 log beta ties at a cut would show here; none with this seed
-                assert torch.equal(cache.kv_positions[l].cpu(), ref.kv_positions[l])
+            for l in range(LAYERS):
+                got = cache.kv_positions[l].cpu()
+                if ties is None or not ties[l].any():
+                    assert torch.equal(got, ref.kv_positions[l])
+                    continue
+                for b in range(B):           # rows with a tie at the cut: equal up to the tied tokens, then re-synchronise
+                    for h in range(HKV):
+                        diff = set(got[b, h].tolist()) ^ set(ref.kv_positions[l][b, h].tolist())
+                        assert (len(diff) == 0) if not ties[l][b, h] else (len(diff) <= 4), (l, b, h, diff)
+                ref.key_cache[l], ref.value_cache[l] = cache.key_cache[l].cpu(), cache.value_cache[l].cpu()
+                ref.retention_weights[l], ref.kv_positions[l] = cache.retention_weights[l].cpu(), got
         else:
             assert cache.get_total_cached_tokens() == ref.get_total_cached_tokens()
             got, want_pos = cache.segment_positions(), ref.segment_positions()

@@ -60,9 +60,23 @@ class LazyLogBeta:
             raise ValueError("LazyLogBeta only supports transpose(1, 2)")
         return LazyLogBeta(self.part, self.bias_f32, self.batch, self.seq, self.heads, self.dtype, not self.transposed)
 
+    def _sum_slices(self) -> torch.Tensor:
+        """Sum over the slice axis in the order the append kernel uses (lanes j, j+64, ... then a
+        64-lane butterfly), so that materialize() and the fused epilogue agree bit for bit."""
+        n = self.part.shape[0]
+        lanes = torch.zeros((64,) + tuple(self.part.shape[1:]), dtype=torch.float32, device=self.part.device)
+        for j0 in range(0, n, 64):
+            chunk = self.part[j0:j0 + 64]
+            lanes[: chunk.shape[0]] = lanes[: chunk.shape[0]] + chunk
+        d = 32
+        while d > 0:
+            lanes = lanes + lanes[torch.arange(64, device=lanes.device) ^ d]
+            d >>= 1
+        return lanes[0]
+
     def materialize(self) -> torch.Tensor:
         """The finished tensor, computed with torch ops (for callers that need the values)."""
-        acc = self.part.sum(dim=0).view(self.batch, self.seq, self.heads)
+        acc = self._sum_slices().view(self.batch, self.seq, self.heads)
         if self.dtype != torch.float32:
             acc = acc.to(self.dtype).float()
             acc = (acc + self.bias_f32).to(self.dtype).float()

@@ -50,21 +50,31 @@ __global__ __launch_bounds__(AP_THREADS) void append_kernel(AppendArgs a) {
             *(uint4*)(a.k_slab + d) = kq;
             *(uint4*)(a.v_slab + d) = vq;
         }
-        for (int s = s_begin + threadIdx.x; s < s_end; s += AP_THREADS) {
-            float lb;
-            if (GATED) {
+        if (GATED) {
+            // one wavefront per new row: lanes fetch the gate's per-slice partial sums in parallel and
+            // add them with a fixed butterfly (the same order every run), lane 0 finishes the gate
+            const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+            const int64_t ntok = (int64_t)(a.nseg / a.kv_heads) * a.s_new;
+            for (int s = s_begin + wave; s < s_end; s += AP_THREADS / 64) {
                 const int64_t tok = (int64_t)b * a.s_new + s;
-                const int64_t ntok = (int64_t)(a.nseg / a.kv_heads) * a.s_new;
                 float acc = 0.0f;
-                for (int j = 0; j < a.gate_nslice; ++j) acc += a.gate_part[((int64_t)j * ntok + tok) * a.kv_heads + h];
-                // a 16-bit module rounds the second linear's output and the biased sum before logsigmoid
-                acc = round_to_dtype(acc, a.lb_dtype);
-                lb = log_sigmoid(round_to_dtype(acc + a.gate_bias[h], a.lb_dtype));
-            } else {
-                lb = load_as_f32(a.lb_new, (int64_t)b * a.lb_sb + (int64_t)h * a.lb_sh + (int64_t)s * a.lb_ss, a.lb_dtype);
+                for (int j = lane; j < a.gate_nslice; j += 64) acc += a.gate_part[((int64_t)j * ntok + tok) * a.kv_heads + h];
+#pragma unroll
+                for (int d = 32; d > 0; d >>= 1) acc += __shfl_xor(acc, d, 64);
+                if (lane == 0) {
+                    // a 16-bit module rounds the second linear's output and the biased sum before logsigmoid
+                    acc = round_to_dtype(acc, a.lb_dtype);
+                    const float lb = log_sigmoid(round_to_dtype(acc + a.gate_bias[h], a.lb_dtype));
+                    store_from_f32(a.lb_slab, dst_row0 + s, a.lb_dtype, lb);
+                    a.pos_slab[dst_row0 + s] = a.pos_new[(int64_t)b * a.pos_sb + (int64_t)h * a.pos_sh + (int64_t)s * a.pos_ss];
+                }
             }
-            store_from_f32(a.lb_slab, dst_row0 + s, a.lb_dtype, lb);
-            a.pos_slab[dst_row0 + s] = a.pos_new[(int64_t)b * a.pos_sb + (int64_t)h * a.pos_sh + (int64_t)s * a.pos_ss];
+        } else {
+            for (int s = s_begin + threadIdx.x; s < s_end; s += AP_THREADS) {
+                const float lb = load_as_f32(a.lb_new, (int64_t)b * a.lb_sb + (int64_t)h * a.lb_sh + (int64_t)s * a.lb_ss, a.lb_dtype);
+                store_from_f32(a.lb_slab, dst_row0 + s, a.lb_dtype, lb);
+                a.pos_slab[dst_row0 + s] = a.pos_new[(int64_t)b * a.pos_sb + (int64_t)h * a.pos_sh + (int64_t)s * a.pos_ss];
+            }
         }
     }
     if (a.bump_in_kernel && threadIdx.x == 0 && fits) {

@@ -3,10 +3,10 @@
 // logsigmoid (:177-179) run inside the append kernel, so log(beta) never makes a round trip through
 // HBM as a tensor of its own.
 //
-// One workgroup = 16 wavefronts = one slice of 16 intermediate units x 64 tokens.  Wavefront
-// (tt, ks) multiplies token tile tt (16 tokens) with the slice over a quarter ks of the hidden
+// One workgroup = 16 wavefronts = one slice of 16 intermediate units x (16 or 64) tokens.
+// Wavefront (tt, ks) multiplies token tile tt (16 tokens) with the slice over part ks of the hidden
 // axis on v_mfma_f32_16x16x32_bf16 (A = x rows, B = W1 rows, both read straight from global in
-// operand layout: lane l holds 8 consecutive k of row l%16 at k-group l/16); the four quarters are
+// operand layout: lane l holds 8 consecutive k of row l%16 at k-group l/16); the parts are
 // summed in LDS, then bias, SiLU and the 16-unit contraction with W2 finish on the VALU.
 // Intermediate values are rounded to bf16 where a bf16 torch module rounds them.
 #include "common.hip.h"
@@ -17,9 +17,8 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int GH_THREADS = 1024;
+constexpr int GH_WAVES = 16;
 constexpr int GH_UNITS = 16;    // intermediate units per slice
-constexpr int GH_TOKENS = 64;   // tokens per workgroup
-constexpr int GH_KSPLIT = 4;
 constexpr int GH_MAX_HEADS = 32;
 
 struct GateArgs {
@@ -27,25 +26,38 @@ struct GateArgs {
     int ntok, hidden, inter, kv_heads;
 };
 
+// TT token tiles of 16 tokens per workgroup, KS = 16 / TT splits of the hidden axis.
+//   TT = 1, KS = 16: decode (a handful of tokens): many small workgroups and short dependent chains;
+//   TT = 4, KS = 4 : prompts: a W1 slice is reused by 64 tokens.
+// STEPS k-steps of 32 are unrolled with all their loads issued before the first MFMA.
+template <int TT, int STEPS>
 __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
-    __shared__ float red[GH_KSPLIT][GH_TOKENS][GH_UNITS + 1];
-    const int slice = blockIdx.x, tok0 = blockIdx.y * GH_TOKENS;
+    constexpr int KS = GH_WAVES / TT, TOKENS = 16 * TT;
+    __shared__ float red[KS][TOKENS][GH_UNITS + 1];
+    const int slice = blockIdx.x, tok0 = blockIdx.y * TOKENS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int tt = wave & 3, ks = wave >> 2;
+    const int tt = wave % TT, ks = wave / TT;
     const int row = lane & 15, kg = lane >> 4;
 
     const int tok = min(tok0 + tt * 16 + row, a.ntok - 1);  // rows past the end re-read the last token
     const int unit = slice * GH_UNITS + row;
-    const int kspan = a.hidden / GH_KSPLIT;
+    const int kspan = a.hidden / KS;
     const uint16_t* xp = a.x + (int64_t)tok * a.hidden + ks * kspan + kg * 8;
     const uint16_t* wp = a.w1 + (int64_t)unit * a.hidden + ks * kspan + kg * 8;
 
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-    for (int k = 0; k < kspan; k += 32) {
-        const bf16x8_t av = *(const bf16x8_t*)(xp + k);
-        const bf16x8_t bv = *(const bf16x8_t*)(wp + k);
-        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc, 0, 0, 0);
+    for (int k0 = 0; k0 < kspan; k0 += 32 * STEPS) {
+        bf16x8_t av[STEPS], bv[STEPS];
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i) {
+            const int k = min(k0 + 32 * i, kspan - 32);   // a short last group re-reads its final step (weight 0 below)
+            av[i] = *(const bf16x8_t*)(xp + k);
+            bv[i] = *(const bf16x8_t*)(wp + k);
+        }
+#pragma unroll
+        for (int i = 0; i < STEPS; ++i) {
+            if (k0 + 32 * i < kspan) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[i], acc, 0, 0, 0);
+        }
     }
     // D[i][j]: lane holds token i = 4*(lane/16) + v, unit j = lane%16
 #pragma unroll
@@ -53,21 +65,25 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     __syncthreads();
 
     // one (token, unit) per thread: bias, SiLU, then the contraction with W2 over the 16 units
-    const int t = tid >> 4, u = tid & 15;
-    float h = red[0][t][u] + red[1][t][u] + red[2][t][u] + red[3][t][u];
-    const int uu = slice * GH_UNITS + u;
-    if (a.b1) h += bf16_bits_to_f32(a.b1[uu]);
-    h = bf16_bits_to_f32(f32_to_bf16_bits(h));            // nn.Linear output in bf16
-    float act = h / (1.0f + __expf(-h));
-    act = bf16_bits_to_f32(f32_to_bf16_bits(act));        // SiLU output in bf16
-    for (int hh = 0; hh < a.kv_heads; ++hh) {
-        float p = act * bf16_bits_to_f32(a.w2[(int64_t)hh * a.inter + uu]);
-        p += __shfl_xor(p, 1, 64);
-        p += __shfl_xor(p, 2, 64);
-        p += __shfl_xor(p, 4, 64);
-        p += __shfl_xor(p, 8, 64);
-        if (u == 0 && tok0 + t < a.ntok)
-            a.part[((int64_t)slice * a.ntok + tok0 + t) * a.kv_heads + hh] = p;
+    if (tid < TOKENS * GH_UNITS) {
+        const int t = tid >> 4, u = tid & 15;
+        float h = 0.0f;
+#pragma unroll
+        for (int i = 0; i < KS; ++i) h += red[i][t][u];
+        const int uu = slice * GH_UNITS + u;
+        if (a.b1) h += bf16_bits_to_f32(a.b1[uu]);
+        h = bf16_bits_to_f32(f32_to_bf16_bits(h));            // nn.Linear output in bf16
+        float act = h / (1.0f + __expf(-h));
+        act = bf16_bits_to_f32(f32_to_bf16_bits(act));        // SiLU output in bf16
+        for (int hh = 0; hh < a.kv_heads; ++hh) {
+            float p = act * bf16_bits_to_f32(a.w2[(int64_t)hh * a.inter + uu]);
+            p += __shfl_xor(p, 1, 64);
+            p += __shfl_xor(p, 2, 64);
+            p += __shfl_xor(p, 4, 64);
+            p += __shfl_xor(p, 8, 64);
+            if (u == 0 && tok0 + t < a.ntok)
+                a.part[((int64_t)slice * a.ntok + tok0 + t) * a.kv_heads + hh] = p;
+        }
     }
 }
 
@@ -84,13 +100,18 @@ extern "C" int trimkv_gate_hidden(const void* x, const void* w1, const void* b1,
     if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 gate weights are supported (dtype=%d)", fn, dtype);
     if (ntok <= 0 || hidden <= 0 || inter <= 0 || kv_heads <= 0 || kv_heads > GH_MAX_HEADS)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes ntok=%d hidden=%d inter=%d kv_heads=%d", fn, ntok, hidden, inter, kv_heads);
-    if (hidden % (32 * GH_KSPLIT) || inter % GH_UNITS)
-        return fail(TRIMKV_ERR_UNSUPPORTED, "%s: hidden must be a multiple of %d and inter of %d (got %d, %d)", fn, 32 * GH_KSPLIT, GH_UNITS, hidden, inter);
+    if (hidden % (32 * GH_WAVES) || inter % GH_UNITS)
+        return fail(TRIMKV_ERR_UNSUPPORTED, "%s: hidden must be a multiple of %d and inter of %d (got %d, %d)", fn, 32 * GH_WAVES, GH_UNITS, hidden, inter);
     if (((uintptr_t)x | (uintptr_t)w1) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: x and w1 must be 16-byte aligned", fn);
     GateArgs a;
     a.x = (const uint16_t*)x; a.w1 = (const uint16_t*)w1; a.b1 = (const uint16_t*)b1; a.w2 = (const uint16_t*)w2; a.part = part;
     a.ntok = ntok; a.hidden = hidden; a.inter = inter; a.kv_heads = kv_heads;
-    dim3 grid(inter / GH_UNITS, (ntok + GH_TOKENS - 1) / GH_TOKENS);
-    hipLaunchKernelGGL(gate_hidden_kernel, grid, dim3(GH_THREADS), 0, (hipStream_t)stream, a);
+    if (ntok <= 256) {  // decode-sized: 16-token tiles, 16-way split of the hidden axis
+        dim3 grid(inter / GH_UNITS, (ntok + 15) / 16);
+        hipLaunchKernelGGL((gate_hidden_kernel<1, 8>), grid, dim3(GH_THREADS), 0, (hipStream_t)stream, a);
+    } else {
+        dim3 grid(inter / GH_UNITS, (ntok + 63) / 64);
+        hipLaunchKernelGGL((gate_hidden_kernel<4, 8>), grid, dim3(GH_THREADS), 0, (hipStream_t)stream, a);
+    }
     return launch_status(fn);
 }

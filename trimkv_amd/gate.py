@@ -46,7 +46,7 @@ class RetentionGate(nn.Module):
     def forward(self, x: torch.Tensor):
         """x [B, S, hidden] -> log beta [B, S, Hkv] (a LazyLogBeta on the fused path)."""
         use_hip = (self.fused and not self.training and x.is_cuda and x.dtype == torch.bfloat16
-                   and self.hidden_act == "silu" and x.shape[-1] % 128 == 0
+                   and self.hidden_act == "silu" and x.shape[-1] % 512 == 0
                    and self.retention_gate_intermediate_size % 16 == 0)
         if not use_hip:
             return self._torch_forward(x)
