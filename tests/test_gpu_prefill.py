@@ -90,6 +90,48 @@ def test_ragged_prefill_matches_fp32_oracle(G):
     assert (out[1, :Q - 7, 0:G] == 0).all()        # segment of 7 keys: the first Q-7 queries see nothing
 
 
+@pytest.mark.parametrize("G", [1, 3, 4, 5, 7])
+def test_ragged_prefill_long_chunk(G):
+    """Chunks of 64 queries and more take the 32-queries-per-wavefront kernel: ragged segments, one empty,
+    one shorter than the chunk, one whose length is not a multiple of the 64-key tile."""
+    from trimkv_amd import get_attention_interface
+    gen = torch.Generator().manual_seed(100 + G)
+    B, H, D, Q = 2, 3, 128, 96
+    lens = [96, 500, 0, 30, 96 + 64, 1001]
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    N = int(cu[-1])
+    k = torch.randn(N, D, generator=gen).to(torch.bfloat16)
+    v = torch.randn(N, D, generator=gen).to(torch.bfloat16)
+    q = torch.randn(B, H * G, Q, D, generator=gen).to(torch.bfloat16)
+    attn = get_attention_interface("db_attn_flash_batched")
+    kw = {"head_lens": torch.tensor(lens, dtype=torch.int32, device=DEV), "cu_seqlens_k": cu.to(DEV), "batch_size": B, "num_kv_heads": H}
+    out, _, _ = attn(_Mod(), q.to(DEV), k.to(DEV), v.to(DEV), None, flash_attn_kwargs=kw)
+    want = ragged_attention(q, k, v, cu, H)
+    ok, err = attn_close(out, want)
+    assert ok, f"max abs err {err}"
+    assert (out[0, :, 2 * G:3 * G] == 0).all()
+    assert (out[1, :Q - 30, 0:G] == 0).all()
+
+
+@pytest.mark.parametrize("Q,n", [(64, 700), (256, 2000)])
+def test_prefill_growing_row_maxima(Q, n):
+    """Scores that keep growing along the key axis (keys scaled by a ramp, queries aligned with them) force the
+    running exponent reference to move many times, small steps and large ones; sharp softmax rows."""
+    from trimkv_amd.attn.hip_attn import prefill_attention
+    gen = torch.Generator().manual_seed(Q + n)
+    B, H, G, D = 1, 2, 4, 128
+    base = torch.randn(D, generator=gen)
+    ramp = torch.linspace(0.05, 3.0, n)[:, None]
+    k = (base[None] * ramp + 0.3 * torch.randn(n, D, generator=gen)).to(torch.bfloat16)
+    k = torch.stack([k, k.flip(0)])                           # second segment: shrinking instead of growing
+    v = torch.randn(B * H, n, D, generator=gen).to(torch.bfloat16)
+    q = (base[None, None, None] * 0.5 + torch.randn(B, H * G, Q, D, generator=gen)).to(torch.bfloat16)
+    out = prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), B, H, G, None, None, n, n, D ** -0.5)
+    want, _ = eager_attention(q.float(), k.float()[None], v.float()[None], G, D ** -0.5, _bottom_right_mask(Q, n))
+    ok, err = attn_close(out, want)
+    assert ok, f"max abs err {err}"
+
+
 def test_prefill_chunk_at_config5_size():
     """Qwen3-14B chunk: 4096 queries on top of 8192 cached keys, G=5 (two segments to bound the run);
     sampled query rows against fp32 on the device."""

@@ -6,18 +6,26 @@
 // prefill (src/trimkv/attn/__init__.py:15-26): query t of the chunk sees every older cached token
 // plus the chunk's own tokens <= t, i.e. keys j <= n - Q_LEN + t.
 //
+// Two kernels share the formulation below.  prefill_attn_kernel (chunks of 64 queries and more) gives
+// a wavefront 32 queries of one head and uses v_mfma_f32_32x32x16_bf16 on 64-key tiles that are
+// double-buffered in LDS, V stored transposed; prefill_small_kernel (short chunks) gives a wavefront
+// 16 queries and uses v_mfma_f32_16x16x32_bf16 on 32-key tiles.
+//
 // A workgroup owns BT consecutive query times of one segment for all G query heads of its KV head,
-// one wavefront per (head, 16 times), so a K/V tile staged in LDS is shared by the whole group.
-// Per 32-key tile a wavefront computes, with v_mfma_f32_16x16x32_bf16,
+// one wavefront per (head, 16 or 32 times), so a K/V tile staged in LDS is shared by the whole group.
+// Per tile a wavefront computes
 //     S^T[key][query] = K . Q^T           (A = K rows from LDS, B = Q rows held in registers)
 //     O^T[d][query]  += V^T . P^T         (A = V columns gathered from LDS, B = P^T)
-// Both products put the query on the MFMA column index, which is the lane index modulo 16: every
+// Both products put the query on the MFMA column index, which is the lane index modulo 16 (32): every
 // per-query quantity (running max, sum, rescale factor) lives in the lane that needs it, and the
-// probabilities a lane holds after the first product (4 keys of each 16-key block) are exactly the
-// 8 keys its B operand of the second product wants -- P never crosses lanes.  V is row-major, so
-// its A operand (8 keys at one d) is gathered as 8 dwords (d, d+1) per lane and split into an
-// even-d and an odd-d operand with v_perm_b32.
+// probabilities a lane holds after the first product are exactly the keys its B operand of the
+// second product wants -- P never crosses lanes.  V is row-major in memory, so its A operand
+// (8 keys at one d) needs a transposition: the large kernel transposes while it stages the tile
+// (key pairs merged with v_perm_b32, written as dwords into a [d][key slot] array whose slot order
+// is the order in which the MFMA output hands a lane its keys); the small kernel gathers 8 dwords
+// (d, d+1) per lane and splits them into an even-d and an odd-d operand.
 #include "common.hip.h"
+#include <type_traits>
 
 namespace trimkv {
 
@@ -25,6 +33,7 @@ typedef __bf16 pf_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float pf_f32x4 __attribute__((ext_vector_type(4)));
 typedef float pf_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int PF_D = 128;
 constexpr int PF_BN = 32;                  // keys per tile
@@ -41,7 +50,7 @@ struct PrefillArgs {
 };
 
 template <int G>
-struct PrefillCfg {
+struct SmallCfg {
     static constexpr int TT = G >= 4 ? 1 : (G == 3 ? 1 : 4 / G);  // 16-query time tiles per workgroup
     static constexpr int WAVES = G * TT;
     static constexpr int THREADS = WAVES * 64;
@@ -56,8 +65,8 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 }
 
 template <int G>
-__global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(PrefillArgs a) {
-    using C = PrefillCfg<G>;
+__global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(PrefillArgs a) {
+    using C = SmallCfg<G>;
     __shared__ __attribute__((aligned(16))) char lds_k[PF_BN * PF_ROW];
     __shared__ __attribute__((aligned(16))) char lds_v[PF_BN * PF_ROW];
 
@@ -95,7 +104,7 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
     const int vis_wave_max = n - Q + min(Q - 1, t_wg0 + tt * 16 + 15);
 
     // cooperative tile load: piece p of 2*32*16 (K rows then V rows), 16 bytes each
-    uint4 stage[C::PIECES];
+    pf_u32x4 stage[C::PIECES];
     auto fetch = [&](int kbase) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < C::PIECES; ++i) {
@@ -104,7 +113,7 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
                 const int isv = p >= PF_BN * 16, q16 = p & 15, key = (p >> 4) & (PF_BN - 1);
                 const int row = min(kbase + key, max(n - 1, 0));
                 const char* src = (isv ? a.v : a.k) + (row0 + row) * (int64_t)(PF_D * 2) + q16 * 16;
-                stage[i] = *(const uint4*)src;
+                stage[i] = *(const pf_u32x4*)src;
             }
         }
     };
@@ -114,7 +123,7 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
             const int p = tid + i * C::THREADS;
             if (p < 2 * PF_BN * 16) {
                 const int isv = p >= PF_BN * 16, q16 = p & 15, key = (p >> 4) & (PF_BN - 1);
-                *(uint4*)((isv ? lds_v : lds_k) + key * PF_ROW + q16 * 16) = stage[i];
+                *(pf_u32x4*)((isv ? lds_v : lds_k) + key * PF_ROW + q16 * 16) = stage[i];
             }
         }
     };
@@ -212,11 +221,260 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Large-chunk kernel: 32 queries per wavefront, 64-key tiles, v_mfma_f32_32x32x16_bf16.
+//
+// MFMA 32x32x16 register layout (lane l, half hl = l / 32):
+//   A (32 x 16): row l % 32, k = 8 * hl + 0..7          B (16 x 32): column l % 32, k = 8 * hl + 0..7
+//   C (32 x 32): column l % 32, register v holds row 8 * (v / 4) + 4 * hl + v % 4
+// S^T = K . Q^T per 32-key block: after it a lane holds, for its query, keys 8c + 4hl + i (c, i in 0..3).
+// The second product consumes 16 keys per MFMA; step st takes from lane half hl the keys of c = 2st and
+// 2st + 1, i.e. registers v = 8st .. 8st + 7 in order.  The V^T tile is stored so that exactly those
+// 8 keys are 16 contiguous bytes: slot(key) = 16 * (key / 16) + 8 * hl(key) + e(key).
+// ---------------------------------------------------------------------------------------------
+typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int PF2_BN = 64;                          // keys per tile (two 32-key blocks)
+constexpr int PF2_KROW = 272;                       // bytes per staged K row
+constexpr int PF2_KBYTES = PF2_BN * PF2_KROW;       // 17408
+constexpr int PF2_VROW = PF2_BN * 2;                // bytes per V^T row (one d, 64 key slots), swizzled in 16-byte groups
+constexpr int PF2_VBYTES = PF_D * PF2_VROW;         // 16384
+constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
+constexpr int PF2_LDS = 2 * PF2_BUF;                // double buffer
+constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a row maximum grows by more than 2^6
+
 template <int G>
-static void launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
+struct PrefillCfg {
+    static constexpr int TT = G >= 5 ? 1 : (G >= 3 ? 2 : 8 / G);   // 32-query time tiles per workgroup
+    static constexpr int WAVES = G * TT;
+    static constexpr int THREADS = WAVES * 64;
+    static constexpr int BT = 32 * TT;
+    static constexpr int KPIECES = (PF2_BN * 16 + THREADS - 1) / THREADS;        // 16-byte pieces of K per thread
+    static constexpr int VPIECES = ((PF2_BN / 2) * 16 + THREADS - 1) / THREADS;  // (key pair, 8 d) pieces of V per thread
+};
+
+// key (0..63) of the tile that sits in V^T slot `slot`
+__device__ __forceinline__ int pf2_key_of_slot(int slot) {
+    const int kb = slot >> 5, st = (slot >> 4) & 1, hl = (slot >> 3) & 1, e = slot & 7;
+    return kb * 32 + st * 16 + hl * 4 + (e & 3) + ((e >> 2) << 3);
+}
+// 16-byte column group swizzle of V^T row d: reads (8 consecutive d per pass) and writes both spread over the banks
+__device__ __forceinline__ int pf2_swz(int d) { return (d & 7) ^ (((d >> 3) & 1) << 2); }
+
+template <int G>
+__global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(PrefillArgs a) {
     using C = PrefillCfg<G>;
+    extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
+
+    const int seg = blockIdx.y;
+    const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;  // later times see more keys: dispatch them first
+    const int b = seg / a.kv_heads, h = seg - b * a.kv_heads;
+    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
+    n = max(0, min(n, a.max_len));
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int g = w % G, tt = w / G;
+    const int j = lane & 31, hl = lane >> 5;    // MFMA column (query) and lane half
+    const int Q = a.q_len;
+    const int t_wg0 = tile * C::BT;
+    const int t_w0 = t_wg0 + tt * 32;
+    const int t_q = t_w0 + j;                   // this lane's query time
+    const bool q_ok = t_q < Q;
+    const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
+
+    // Q fragments (B operand of S^T): 8 d of step ks at d = ks * 16 + hl * 8
+    pf_bf16x8 qf[8];
+    {
+        const uint16_t* qrow = a.q + (int64_t)b * a.q_sb + (int64_t)(h * G + g) * a.q_sh + (int64_t)min(t_q, Q - 1) * a.q_st;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const pf_bf16x8*)(qrow + ks * 16 + hl * 8);
+    }
+
+    pf_f32x16 o[4];   // O^T: o[db][v] = d (db * 32 + 8 * (v / 4) + 4 * hl + v % 4) of query j
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
+    float m_ref = PF_NEG, l_run = 0.0f;   // exponent reference (scaled log2 units) and this lane's share of the row sum
+
+    const int t_last = min(Q - 1, t_wg0 + C::BT - 1);
+    const int k_end = max(0, min(n, n - Q + t_last + 1));     // keys the workgroup visits
+    const int vis_j = n - Q + t_q;                            // last key this lane's query sees
+    const int vis_lo = n - Q + t_w0;                          // ... the wavefront's first query
+    const int vis_hi = n - Q + min(Q - 1, t_w0 + 31);         // ... its last real query
+    const int last_row = max(n - 1, 0);
+
+    // ---- staging: global -> registers -> LDS (K row-major, V transposed) ----
+    pf_u32x4 kst[C::KPIECES], vst[C::VPIECES][2];
+    auto fetch = [&](int kbase) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < C::KPIECES; ++i) {
+            const int p = min(tid + i * C::THREADS, PF2_BN * 16 - 1);
+            const int row = min(kbase + (p >> 4), last_row);
+            kst[i] = *(const pf_u32x4*)(a.k + (row0 + row) * (int64_t)(PF_D * 2) + (p & 15) * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < C::VPIECES; ++i) {
+            const int p = min(tid + i * C::THREADS, (PF2_BN / 2) * 16 - 1);
+            const int key = pf2_key_of_slot((p >> 4) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
+            const int r0 = min(kbase + key, last_row), r1 = min(kbase + key + 1, last_row);
+            vst[i][0] = *(const pf_u32x4*)(a.v + (row0 + r0) * (int64_t)(PF_D * 2) + (p & 15) * 16);
+            vst[i][1] = *(const pf_u32x4*)(a.v + (row0 + r1) * (int64_t)(PF_D * 2) + (p & 15) * 16);
+        }
+    };
+    auto publish = [&](char* buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < C::KPIECES; ++i) {
+            const int p = tid + i * C::THREADS;
+            if (p < PF2_BN * 16) *(pf_u32x4*)(buf + (p >> 4) * PF2_KROW + (p & 15) * 16) = kst[i];
+        }
+#pragma unroll
+        for (int i = 0; i < C::VPIECES; ++i) {
+            const int p = tid + i * C::THREADS;
+            if (p < (PF2_BN / 2) * 16) {
+                const int sp = p >> 4, dchunk = p & 15;
+                const pf_u32x4 lo = vst[i][0], hi = vst[i][1];
+                char* vt = buf + PF2_KBYTES;
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    const int d0 = dchunk * 8 + 2 * x;
+                    const uint32_t ev = __builtin_amdgcn_perm(hi[x], lo[x], 0x05040100u);   // (key, key + 1) at d0
+                    const uint32_t od = __builtin_amdgcn_perm(hi[x], lo[x], 0x07060302u);   // ... at d0 + 1
+                    *(uint32_t*)(vt + d0 * PF2_VROW + ((((sp >> 2) ^ pf2_swz(d0)) << 2) + (sp & 3)) * 4) = ev;
+                    *(uint32_t*)(vt + (d0 + 1) * PF2_VROW + ((((sp >> 2) ^ pf2_swz(d0 + 1)) << 2) + (sp & 3)) * 4) = od;
+                }
+            }
+        }
+    };
+
+    // per-lane LDS read offsets
+    const int k_off = j * PF2_KROW + hl * 16;
+    const int v_sw = hl ^ pf2_swz(j);            // swizzle of rows d = db * 32 + j depends on j only
+    const int v_off = PF2_KBYTES + j * PF2_VROW;
+
+    auto compute = [&](const char* buf, int kbase, auto masked_tag) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        // ---- S^T = K . Q^T for the two 32-key blocks ----
+        pf_f32x16 s[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) {
+                const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
+                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
+            }
+        }
+        // ---- row maximum of the tile (this lane's 32 keys) ----
+        float tmax = PF_NEG;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float x = s[kb][v];
+                if (MASKED) {
+                    const int key = kbase + kb * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
+                    x = (key <= vis_j) ? x * a.scale_log2 : PF_NEG;
+                    s[kb][v] = x;
+                }
+                tmax = fmaxf(tmax, x);
+            }
+        }
+        if (!MASKED) tmax *= a.scale_log2;
+        // lazy rescale: keep the exponent reference until some row outgrows it by 2^PF2_LAZY
+        if (__builtin_amdgcn_ballot_w64(tmax > m_ref + PF2_LAZY) != 0) {
+            const float t2 = fmaxf(tmax, __shfl_xor(tmax, 32, 64));   // both halves of a query agree on the reference
+            const float m_new = fmaxf(m_ref, t2);
+            const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+            m_ref = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        }
+        // ---- P = exp2(S - ref), O^T += V^T . P^T ----
+        float psum = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+            float p[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                if (MASKED) p[v] = s[kb][v] > 0.5f * PF_NEG ? __builtin_amdgcn_exp2f(s[kb][v] - m_ref) : 0.0f;
+                else p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v], a.scale_log2, -m_ref));
+                psum += p[v];
+            }
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                const uint4 pw = make_uint4(pack_bf16(p[8 * st + 0], p[8 * st + 1]), pack_bf16(p[8 * st + 2], p[8 * st + 3]),
+                                            pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7]));
+                const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pw);
+                const int grp = ((kb * 4 + st * 2) ^ v_sw) * 16;   // column group (kb, st, hl) of row d, swizzled
+#pragma unroll
+                for (int db = 0; db < 4; ++db) {
+                    const pf_bf16x8 vf = *(const pf_bf16x8*)(buf + v_off + db * 32 * PF2_VROW + grp);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pfrag, o[db], 0, 0, 0);
+                }
+            }
+        }
+        l_run += psum;
+    };
+
+    const int ntiles = (k_end + PF2_BN - 1) / PF2_BN;
+    if (ntiles > 0) {
+        fetch(0);
+        publish(pf2_lds);
+        __syncthreads();
+    }
+    for (int it = 0; it < ntiles; ++it) {
+        const int kbase = it * PF2_BN;
+        char* cur = pf2_lds + (it & 1) * PF2_BUF;
+        char* nxt = pf2_lds + ((it + 1) & 1) * PF2_BUF;
+        fetch(kbase + PF2_BN);          // unconditional (rows clamped): the next tile is in flight during the arithmetic
+        if (kbase <= vis_hi) {          // wave-uniform: some query of this wavefront sees part of the tile
+            if (kbase + PF2_BN - 1 <= vis_lo) compute(cur, kbase, std::false_type{});
+            else compute(cur, kbase, std::true_type{});
+        }
+        publish(nxt);                   // free since the barrier that ended the previous iteration
+        __syncthreads();
+    }
+
+    // the two halves of a query hold disjoint keys: add their sums, then normalise and store
+    l_run += __shfl_xor(l_run, 32, 64);
+    if (q_ok) {
+        const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+        char* orow = (char*)(a.out + (((int64_t)b * Q + t_q) * (a.kv_heads * G) + (h * G + g)) * PF_D);
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint2 pk = make_uint2(pack_bf16(o[db][4 * c] * inv, o[db][4 * c + 1] * inv),
+                                            pack_bf16(o[db][4 * c + 2] * inv, o[db][4 * c + 3] * inv));
+                *(uint2*)(orow + (db * 32 + 8 * c + 4 * hl) * 2) = pk;
+            }
+        }
+    }
+}
+
+template <int G>
+static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
+    if (a.q_len < 64) {   // short chunks: 16 queries per wavefront waste fewer MFMA columns
+        using C = SmallCfg<G>;
+        const int tiles = (a.q_len + C::BT - 1) / C::BT;
+        hipLaunchKernelGGL(prefill_small_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
+        return 0;
+    }
+    using C = PrefillCfg<G>;
+    static bool lds_opted_in = false;   // > 64 KB of dynamic LDS needs the attribute once per kernel
+    if (!lds_opted_in) {
+        hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
+        if (e != hipSuccess) return (int)e;
+        lds_opted_in = true;
+    }
     const int tiles = (a.q_len + C::BT - 1) / C::BT;
-    hipLaunchKernelGGL(prefill_attn_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
+    hipLaunchKernelGGL(prefill_attn_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), PF2_LDS, st, a);
+    return 0;
 }
 
 }  // namespace trimkv
@@ -244,15 +502,17 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
     a.k = (const char*)k_slab; a.v = (const char*)v_slab; a.seg_len = seg_len; a.seg_start = seg_start;
     a.kv_heads = kv_heads; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
+    int rc = 0;
     switch (group) {
-        case 1: launch_prefill<1>(a, (int)nseg, st); break;
-        case 2: launch_prefill<2>(a, (int)nseg, st); break;
-        case 3: launch_prefill<3>(a, (int)nseg, st); break;
-        case 4: launch_prefill<4>(a, (int)nseg, st); break;
-        case 5: launch_prefill<5>(a, (int)nseg, st); break;
-        case 6: launch_prefill<6>(a, (int)nseg, st); break;
-        case 7: launch_prefill<7>(a, (int)nseg, st); break;
-        default: launch_prefill<8>(a, (int)nseg, st); break;
+        case 1: rc = launch_prefill<1>(a, (int)nseg, st); break;
+        case 2: rc = launch_prefill<2>(a, (int)nseg, st); break;
+        case 3: rc = launch_prefill<3>(a, (int)nseg, st); break;
+        case 4: rc = launch_prefill<4>(a, (int)nseg, st); break;
+        case 5: rc = launch_prefill<5>(a, (int)nseg, st); break;
+        case 6: rc = launch_prefill<6>(a, (int)nseg, st); break;
+        case 7: rc = launch_prefill<7>(a, (int)nseg, st); break;
+        default: rc = launch_prefill<8>(a, (int)nseg, st); break;
     }
+    if (rc) return fail(rc, "%s: hipFuncSetAttribute failed (%d)", fn, rc);
     return launch_status(fn);
 }
