@@ -45,7 +45,7 @@ struct PrefillArgs {
     uint16_t* out;                                  // [B][Q][Hq][D] contiguous
     const char* k; const char* v;
     const int32_t* seg_len; const int32_t* seg_start;
-    int kv_heads, q_len, cap, max_len;
+    int kv_heads, group, q_len, cap, max_len;
     float scale_log2;
 };
 
@@ -244,15 +244,15 @@ constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
 constexpr int PF2_LDS = 2 * PF2_BUF;                // double buffer
 constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a row maximum grows by more than 2^6
 
-template <int G>
-struct PrefillCfg {
-    static constexpr int TT = G >= 5 ? 1 : (G >= 3 ? 2 : 8 / G);   // 32-query time tiles per workgroup
-    static constexpr int WAVES = G * TT;
-    static constexpr int THREADS = WAVES * 64;
-    static constexpr int BT = 32 * TT;
-    static constexpr int KPIECES = (PF2_BN * 16 + THREADS - 1) / THREADS;        // 16-byte pieces of K per thread
-    static constexpr int VPIECES = ((PF2_BN / 2) * 16 + THREADS - 1) / THREADS;  // (key pair, 8 d) pieces of V per thread
-};
+// A workgroup is always 8 wavefronts (two per SIMD, 256 registers each) and owns 256 / G consecutive query times
+// for all G heads: MFMA column c of wavefront w is row r = 32w + c of the workgroup, time r / G, head r % G.
+// Every per-query quantity is per lane, so a wavefront may mix heads freely; time-major rows keep the
+// spread of a wavefront's causal limits small.
+constexpr int PF2_WAVES = 8;
+constexpr int PF2_THREADS = PF2_WAVES * 64;
+constexpr int PF2_KPIECES = PF2_BN * 16 / PF2_THREADS;          // 16-byte pieces of K per thread (2)
+constexpr int PF2_VPIECES = (PF2_BN / 2) * 16 / PF2_THREADS;    // (key pair, 8 d) pieces of V per thread (1)
+static_assert(PF2_KPIECES * PF2_THREADS == PF2_BN * 16 && PF2_VPIECES * PF2_THREADS == (PF2_BN / 2) * 16, "tile must divide over the workgroup");
 
 // key (0..63) of the tile that sits in V^T slot `slot`
 __device__ __forceinline__ int pf2_key_of_slot(int slot) {
@@ -262,9 +262,7 @@ __device__ __forceinline__ int pf2_key_of_slot(int slot) {
 // 16-byte column group swizzle of V^T row d: reads (8 consecutive d per pass) and writes both spread over the banks
 __device__ __forceinline__ int pf2_swz(int d) { return (d & 7) ^ (((d >> 3) & 1) << 2); }
 
-template <int G>
-__global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(PrefillArgs a) {
-    using C = PrefillCfg<G>;
+__global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
 
     const int seg = blockIdx.y;
@@ -273,13 +271,16 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-    const int g = w % G, tt = w / G;
     const int j = lane & 31, hl = lane >> 5;    // MFMA column (query) and lane half
-    const int Q = a.q_len;
-    const int t_wg0 = tile * C::BT;
-    const int t_w0 = t_wg0 + tt * 32;
-    const int t_q = t_w0 + j;                   // this lane's query time
-    const bool q_ok = t_q < Q;
+    const int G = a.group, Q = a.q_len;
+    const int BT = (PF2_WAVES * 32) / G;        // query times per workgroup; rows BT * G .. 255 are padding
+    const int t_wg0 = tile * BT;
+    const int r = w * 32 + j;
+    const int g = r % G;
+    const int t_q = t_wg0 + r / G;              // this lane's query time
+    const bool q_ok = r < BT * G && t_q < Q;
+    const int t_w_first = t_wg0 + (w * 32) / G;
+    const int t_w_last = t_wg0 + min(w * 32 + 31, BT * G - 1) / G;
     const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
 
     // Q fragments (B operand of S^T): 8 d of step ks at d = ks * 16 + hl * 8
@@ -297,25 +298,25 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
         for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
     float m_ref = PF_NEG, l_run = 0.0f;   // exponent reference (scaled log2 units) and this lane's share of the row sum
 
-    const int t_last = min(Q - 1, t_wg0 + C::BT - 1);
+    const int t_last = min(Q - 1, t_wg0 + BT - 1);
     const int k_end = max(0, min(n, n - Q + t_last + 1));     // keys the workgroup visits
     const int vis_j = n - Q + t_q;                            // last key this lane's query sees
-    const int vis_lo = n - Q + t_w0;                          // ... the wavefront's first query
-    const int vis_hi = n - Q + min(Q - 1, t_w0 + 31);         // ... its last real query
+    const int vis_lo = n - Q + t_w_first;                     // ... the wavefront's first query
+    const int vis_hi = t_w_first < Q ? n - Q + min(Q - 1, t_w_last) : -1;   // ... its last real query (none: skip every tile)
     const int last_row = max(n - 1, 0);
 
     // ---- staging: global -> registers -> LDS (K row-major, V transposed) ----
-    pf_u32x4 kst[C::KPIECES], vst[C::VPIECES][2];
+    pf_u32x4 kst[PF2_KPIECES], vst[PF2_VPIECES][2];
     auto fetch = [&](int kbase) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < C::KPIECES; ++i) {
-            const int p = min(tid + i * C::THREADS, PF2_BN * 16 - 1);
+        for (int i = 0; i < PF2_KPIECES; ++i) {
+            const int p = tid + i * PF2_THREADS;
             const int row = min(kbase + (p >> 4), last_row);
             kst[i] = *(const pf_u32x4*)(a.k + (row0 + row) * (int64_t)(PF_D * 2) + (p & 15) * 16);
         }
 #pragma unroll
-        for (int i = 0; i < C::VPIECES; ++i) {
-            const int p = min(tid + i * C::THREADS, (PF2_BN / 2) * 16 - 1);
+        for (int i = 0; i < PF2_VPIECES; ++i) {
+            const int p = tid + i * PF2_THREADS;
             const int key = pf2_key_of_slot((p >> 4) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
             const int r0 = min(kbase + key, last_row), r1 = min(kbase + key + 1, last_row);
             vst[i][0] = *(const pf_u32x4*)(a.v + (row0 + r0) * (int64_t)(PF_D * 2) + (p & 15) * 16);
@@ -324,14 +325,14 @@ __global__ __launch_bounds__(PrefillCfg<G>::THREADS) void prefill_attn_kernel(Pr
     };
     auto publish = [&](char* buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < C::KPIECES; ++i) {
-            const int p = tid + i * C::THREADS;
-            if (p < PF2_BN * 16) *(pf_u32x4*)(buf + (p >> 4) * PF2_KROW + (p & 15) * 16) = kst[i];
+        for (int i = 0; i < PF2_KPIECES; ++i) {
+            const int p = tid + i * PF2_THREADS;
+            *(pf_u32x4*)(buf + (p >> 4) * PF2_KROW + (p & 15) * 16) = kst[i];
         }
 #pragma unroll
-        for (int i = 0; i < C::VPIECES; ++i) {
-            const int p = tid + i * C::THREADS;
-            if (p < (PF2_BN / 2) * 16) {
+        for (int i = 0; i < PF2_VPIECES; ++i) {
+            const int p = tid + i * PF2_THREADS;
+            {
                 const int sp = p >> 4, dchunk = p & 15;
                 const pf_u32x4 lo = vst[i][0], hi = vst[i][1];
                 char* vt = buf + PF2_KBYTES;
@@ -465,15 +466,14 @@ static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
         hipLaunchKernelGGL(prefill_small_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
         return 0;
     }
-    using C = PrefillCfg<G>;
-    static bool lds_opted_in = false;   // > 64 KB of dynamic LDS needs the attribute once per kernel
+    static bool lds_opted_in = false;   // > 64 KB of dynamic LDS needs the attribute once
     if (!lds_opted_in) {
-        hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel<G>, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
+        hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
         if (e != hipSuccess) return (int)e;
         lds_opted_in = true;
     }
-    const int tiles = (a.q_len + C::BT - 1) / C::BT;
-    hipLaunchKernelGGL(prefill_attn_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), PF2_LDS, st, a);
+    const int bt = (PF2_WAVES * 32) / G;
+    hipLaunchKernelGGL(prefill_attn_kernel, dim3((a.q_len + bt - 1) / bt, nseg), dim3(PF2_THREADS), PF2_LDS, st, a);
     return 0;
 }
 
@@ -500,7 +500,7 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
     PrefillArgs a;
     a.q = (const uint16_t*)q; a.q_sb = q_stride_b; a.q_sh = q_stride_h; a.q_st = q_stride_t; a.out = (uint16_t*)out;
     a.k = (const char*)k_slab; a.v = (const char*)v_slab; a.seg_len = seg_len; a.seg_start = seg_start;
-    a.kv_heads = kv_heads; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.scale_log2 = scale * 1.4426950408889634f;
+    a.kv_heads = kv_heads; a.group = group; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
     int rc = 0;
     switch (group) {
