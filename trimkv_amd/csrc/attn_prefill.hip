@@ -238,7 +238,7 @@ typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
 constexpr int PF2_BN = 64;                          // keys per tile (two 32-key blocks)
 constexpr int PF2_KROW = 272;                       // bytes per staged K row
 constexpr int PF2_KBYTES = PF2_BN * PF2_KROW;       // 17408
-constexpr int PF2_VROW = PF2_BN * 2;                // bytes per V^T row (one d, 64 key slots), swizzled in 16-byte groups
+constexpr int PF2_VROW = PF2_BN * 2 + 16;           // bytes per V^T row (one d, 64 key slots): 9 x 16 bytes, so 16 consecutive rows cover all banks
 constexpr int PF2_VBYTES = PF_D * PF2_VROW;         // 16384
 constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
 constexpr int PF2_LDS = 2 * PF2_BUF;                // double buffer
@@ -254,13 +254,15 @@ constexpr int PF2_KPIECES = PF2_BN * 16 / PF2_THREADS;          // 16-byte piece
 constexpr int PF2_VPIECES = (PF2_BN / 2) * 16 / PF2_THREADS;    // (key pair, 8 d) pieces of V per thread (1)
 static_assert(PF2_KPIECES * PF2_THREADS == PF2_BN * 16 && PF2_VPIECES * PF2_THREADS == (PF2_BN / 2) * 16, "tile must divide over the workgroup");
 
+// V staging piece p of a tile -> (key-slot pair, 16-byte chunk of d).  A wavefront takes 16 slot pairs x 4 chunks:
+// its dword writes into V^T (row stride 36 words) then fall on 32 different banks, and its loads are 64-byte runs.
+__device__ __forceinline__ int pf2_vpiece_sp(int p) { return (p & 15) + 16 * ((p >> 6) & 1); }
+__device__ __forceinline__ int pf2_vpiece_dchunk(int p) { return ((p >> 4) & 3) + 4 * (p >> 7); }
 // key (0..63) of the tile that sits in V^T slot `slot`
 __device__ __forceinline__ int pf2_key_of_slot(int slot) {
     const int kb = slot >> 5, st = (slot >> 4) & 1, hl = (slot >> 3) & 1, e = slot & 7;
     return kb * 32 + st * 16 + hl * 4 + (e & 3) + ((e >> 2) << 3);
 }
-// 16-byte column group swizzle of V^T row d: reads (8 consecutive d per pass) and writes both spread over the banks
-__device__ __forceinline__ int pf2_swz(int d) { return (d & 7) ^ (((d >> 3) & 1) << 2); }
 
 __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
@@ -317,10 +319,10 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 #pragma unroll
         for (int i = 0; i < PF2_VPIECES; ++i) {
             const int p = tid + i * PF2_THREADS;
-            const int key = pf2_key_of_slot((p >> 4) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
+            const int key = pf2_key_of_slot(pf2_vpiece_sp(p) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
             const int r0 = min(kbase + key, last_row), r1 = min(kbase + key + 1, last_row);
-            vst[i][0] = *(const pf_u32x4*)(a.v + (row0 + r0) * (int64_t)(PF_D * 2) + (p & 15) * 16);
-            vst[i][1] = *(const pf_u32x4*)(a.v + (row0 + r1) * (int64_t)(PF_D * 2) + (p & 15) * 16);
+            vst[i][0] = *(const pf_u32x4*)(a.v + (row0 + r0) * (int64_t)(PF_D * 2) + pf2_vpiece_dchunk(p) * 16);
+            vst[i][1] = *(const pf_u32x4*)(a.v + (row0 + r1) * (int64_t)(PF_D * 2) + pf2_vpiece_dchunk(p) * 16);
         }
     };
     auto publish = [&](char* buf) __attribute__((always_inline)) {
@@ -333,7 +335,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         for (int i = 0; i < PF2_VPIECES; ++i) {
             const int p = tid + i * PF2_THREADS;
             {
-                const int sp = p >> 4, dchunk = p & 15;
+                const int sp = pf2_vpiece_sp(p), dchunk = pf2_vpiece_dchunk(p);
                 const pf_u32x4 lo = vst[i][0], hi = vst[i][1];
                 char* vt = buf + PF2_KBYTES;
 #pragma unroll
@@ -341,8 +343,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
                     const int d0 = dchunk * 8 + 2 * x;
                     const uint32_t ev = __builtin_amdgcn_perm(hi[x], lo[x], 0x05040100u);   // (key, key + 1) at d0
                     const uint32_t od = __builtin_amdgcn_perm(hi[x], lo[x], 0x07060302u);   // ... at d0 + 1
-                    *(uint32_t*)(vt + d0 * PF2_VROW + ((((sp >> 2) ^ pf2_swz(d0)) << 2) + (sp & 3)) * 4) = ev;
-                    *(uint32_t*)(vt + (d0 + 1) * PF2_VROW + ((((sp >> 2) ^ pf2_swz(d0 + 1)) << 2) + (sp & 3)) * 4) = od;
+                    *(uint32_t*)(vt + d0 * PF2_VROW + sp * 4) = ev;
+                    *(uint32_t*)(vt + (d0 + 1) * PF2_VROW + sp * 4) = od;
                 }
             }
         }
@@ -350,8 +352,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 
     // per-lane LDS read offsets
     const int k_off = j * PF2_KROW + hl * 16;
-    const int v_sw = hl ^ pf2_swz(j);            // swizzle of rows d = db * 32 + j depends on j only
-    const int v_off = PF2_KBYTES + j * PF2_VROW;
+    const int v_off = PF2_KBYTES + j * PF2_VROW + hl * 16;
 
     auto compute = [&](const char* buf, int kbase, auto masked_tag) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_tag)::value;
@@ -411,7 +412,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
                 const uint4 pw = make_uint4(pack_bf16(p[8 * st + 0], p[8 * st + 1]), pack_bf16(p[8 * st + 2], p[8 * st + 3]),
                                             pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7]));
                 const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pw);
-                const int grp = ((kb * 4 + st * 2) ^ v_sw) * 16;   // column group (kb, st, hl) of row d, swizzled
+                const int grp = (kb * 4 + st * 2) * 16;   // column group (kb, st, hl) of row d
 #pragma unroll
                 for (int db = 0; db < 4; ++db) {
                     const pf_bf16x8 vf = *(const pf_bf16x8*)(buf + v_off + db * 32 * PF2_VROW + grp);
