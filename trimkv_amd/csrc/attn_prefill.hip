@@ -241,7 +241,7 @@ constexpr int PF2_KBYTES = PF2_BN * PF2_KROW;       // 17408
 constexpr int PF2_VROW = PF2_BN * 2 + 16;           // bytes per V^T row (one d, 64 key slots): 9 x 16 bytes, so 16 consecutive rows cover all banks
 constexpr int PF2_VBYTES = PF_D * PF2_VROW;         // 16384
 constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
-constexpr int PF2_LDS = 2 * PF2_BUF;                // double buffer
+constexpr int PF2_LDS = 3 * PF2_BUF;                // three tiles in rotation
 constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a row maximum grows by more than 2^6
 
 // A workgroup is always 8 wavefronts (two per SIMD, 256 registers each) and owns 256 / G consecutive query times
@@ -298,11 +298,14 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
-    float m_ref = PF_NEG, l_run = 0.0f;   // exponent reference (scaled log2 units) and this lane's share of the row sum
+    // exponent reference (scaled log2 units) and this lane's share of the row sum.  A query that sees no key at all
+    // (segment shorter than the chunk) keeps reference 0: its masked scores give exp2(-huge) = 0, never exp2(0).
+    float m_ref = PF_NEG, l_run = 0.0f;
 
     const int t_last = min(Q - 1, t_wg0 + BT - 1);
     const int k_end = max(0, min(n, n - Q + t_last + 1));     // keys the workgroup visits
     const int vis_j = n - Q + t_q;                            // last key this lane's query sees
+    if (vis_j < 0) m_ref = 0.0f;
     const int vis_lo = n - Q + t_w_first;                     // ... the wavefront's first query
     const int vis_hi = t_w_first < Q ? n - Q + min(Q - 1, t_w_last) : -1;   // ... its last real query (none: skip every tile)
     const int last_row = max(n - 1, 0);
@@ -354,37 +357,32 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int k_off = j * PF2_KROW + hl * 16;
     const int v_off = PF2_KBYTES + j * PF2_VROW + hl * 16;
 
-    auto compute = [&](const char* buf, int kbase, auto masked_tag) __attribute__((always_inline)) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
-        // ---- S^T = K . Q^T for the two 32-key blocks ----
-        pf_f32x16 s[2];
+    // S^T = K . Q^T of one 32-key block (raw, unscaled scores)
+    auto qk = [&](const char* buf, int kb) __attribute__((always_inline)) {
+        pf_f32x16 s;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int v = 0; v < 16; ++v) s[v] = 0.0f;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) s[kb][v] = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
-                s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s[kb], 0, 0, 0);
-            }
+        for (int ks = 0; ks < 8; ++ks) {
+            const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
+            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
         }
-        // ---- row maximum of the tile (this lane's 32 keys) ----
-        float tmax = PF_NEG;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        return s;
+    };
+    // Mask (diagonal blocks only), row maximum, and the lazy move of the exponent reference: O and l are
+    // rescaled only when some row of the wavefront outgrows its reference by 2^PF2_LAZY.
+    auto prepare = [&](pf_f32x16& s, int blk) __attribute__((always_inline)) {
+        if (blk * 32 + 31 > vis_lo) {   // wave-uniform: some query of the wavefront does not see the whole block
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                float x = s[kb][v];
-                if (MASKED) {
-                    const int key = kbase + kb * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
-                    x = (key <= vis_j) ? x * a.scale_log2 : PF_NEG;
-                    s[kb][v] = x;
-                }
-                tmax = fmaxf(tmax, x);
+                const int key = blk * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
+                s[v] = key <= vis_j ? s[v] : PF_NEG;
             }
         }
-        if (!MASKED) tmax *= a.scale_log2;
-        // lazy rescale: keep the exponent reference until some row outgrows it by 2^PF2_LAZY
+        float tmax = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) tmax = fmaxf(tmax, s[v]);
+        tmax *= a.scale_log2;
         if (__builtin_amdgcn_ballot_w64(tmax > m_ref + PF2_LAZY) != 0) {
             const float t2 = fmaxf(tmax, __shfl_xor(tmax, 32, 64));   // both halves of a query agree on the reference
             const float m_new = fmaxf(m_ref, t2);
@@ -396,50 +394,103 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 #pragma unroll
                 for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
         }
-        // ---- P = exp2(S - ref), O^T += V^T . P^T ----
-        float psum = 0.0f;
+    };
+    // P = exp2(S * scale - ref) as bf16 (two scores -> one dword) and the row sum of the rounded P
+    auto p_pair = [&](const pf_f32x16& s, int x) __attribute__((always_inline)) {
+        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x], a.scale_log2, -m_ref));
+        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x + 1], a.scale_log2, -m_ref));
+        const uint32_t pw = pack_bf16(p0, p1);
+        l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pf_bf16x2, pw), __builtin_bit_cast(pf_bf16x2, 0x3F803F80u), l_run, false);
+        return pw;
+    };
+    auto v_frag = [&](const char* buf, int kb, int st, int db) __attribute__((always_inline)) {
+        return *(const pf_bf16x8*)(buf + v_off + db * 32 * PF2_VROW + (kb * 4 + st * 2) * 16);
+    };
+    // One pipeline step, in issue order (the fences keep the compiler from regrouping it): the 8 MFMAs of the next
+    // block's scores, each followed by one eighth of this block's exponentials; then the 8 MFMAs of P.V.  Operand
+    // reads from LDS are issued well ahead of the MFMA that consumes them.
+    //   HAS_NEXT = false: last block of the wavefront, no scores to compute.
+    auto step = [&](pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
+                    __attribute__((always_inline)) {
+        constexpr bool HAS_NEXT = decltype(has_next)::value;
+        pf_bf16x8 kf[8], vf[8];
+        uint32_t pw[8];
+        if (HAS_NEXT) {
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            float p[16];
+            for (int ks = 0; ks < 8; ++ks) kf[ks] = *(const pf_bf16x8*)(kbuf + k_off + kkb * 32 * PF2_KROW + ks * 32);
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                if (MASKED) p[v] = s[kb][v] > 0.5f * PF_NEG ? __builtin_amdgcn_exp2f(s[kb][v] - m_ref) : 0.0f;
-                else p[v] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kb][v], a.scale_log2, -m_ref));
-                psum += p[v];
-            }
-#pragma unroll
-            for (int st = 0; st < 2; ++st) {
-                const uint4 pw = make_uint4(pack_bf16(p[8 * st + 0], p[8 * st + 1]), pack_bf16(p[8 * st + 2], p[8 * st + 3]),
-                                            pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7]));
-                const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pw);
-                const int grp = (kb * 4 + st * 2) * 16;   // column group (kb, st, hl) of row d
-#pragma unroll
-                for (int db = 0; db < 4; ++db) {
-                    const pf_bf16x8 vf = *(const pf_bf16x8*)(buf + v_off + db * 32 * PF2_VROW + grp);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pfrag, o[db], 0, 0, 0);
-                }
-            }
+            for (int v = 0; v < 16; ++v) s_nxt[v] = 0.0f;
         }
-        l_run += psum;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            pw[ks] = p_pair(s_cur, ks);
+            if (ks == 2) {
+#pragma unroll
+                for (int db = 0; db < 4; ++db) vf[db] = v_frag(vbuf, vkb, 0, db);
+            }
+            if (ks == 5) {
+#pragma unroll
+                for (int db = 0; db < 4; ++db) vf[4 + db] = v_frag(vbuf, vkb, 1, db);
+            }
+            if (HAS_NEXT) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s_nxt, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+            const pf_u32x4 pq = {pw[4 * st], pw[4 * st + 1], pw[4 * st + 2], pw[4 * st + 3]};
+            const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pq);
+#pragma unroll
+            for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * st + db], pfrag, o[db], 0, 0, 0);
+        }
     };
 
+    // Pipeline over 32-key blocks: while the exponentials of block b run on the VALU, the MFMA unit computes the scores
+    // of block b + 1 and then P.V of block b.  Tiles (two blocks) rotate through three LDS buffers: tile t + 1 is
+    // written at the top of iteration t into the buffer tile t - 2 used (every wavefront left it before the barrier of
+    // iteration t - 1) and becomes visible at the barrier in the middle of iteration t, in time for the scores of its
+    // first block.
     const int ntiles = (k_end + PF2_BN - 1) / PF2_BN;
+    const int nb_w = vis_hi >= 0 ? min(vis_hi / 32 + 1, 2 * ntiles) : 0;   // blocks this wavefront visits
     if (ntiles > 0) {
+        pf_f32x16 s_cur;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_cur[v] = 0.0f;
         fetch(0);
         publish(pf2_lds);
+        fetch(PF2_BN);
         __syncthreads();
-    }
-    for (int it = 0; it < ntiles; ++it) {
-        const int kbase = it * PF2_BN;
-        char* cur = pf2_lds + (it & 1) * PF2_BUF;
-        char* nxt = pf2_lds + ((it + 1) & 1) * PF2_BUF;
-        fetch(kbase + PF2_BN);          // unconditional (rows clamped): the next tile is in flight during the arithmetic
-        if (kbase <= vis_hi) {          // wave-uniform: some query of this wavefront sees part of the tile
-            if (kbase + PF2_BN - 1 <= vis_lo) compute(cur, kbase, std::false_type{});
-            else compute(cur, kbase, std::true_type{});
+        if (nb_w > 0) {
+            s_cur = qk(pf2_lds, 0);
+            prepare(s_cur, 0);
         }
-        publish(nxt);                   // free since the barrier that ended the previous iteration
-        __syncthreads();
+        int i0 = 0, i1 = 1;   // buffer index of tile t and of tile t + 1
+        for (int t = 0; t < ntiles; ++t) {
+            const char* b0 = pf2_lds + i0 * PF2_BUF;
+            char* b1 = pf2_lds + i1 * PF2_BUF;
+            publish(b1);
+            fetch((t + 2) * PF2_BN);          // unconditional (rows clamped)
+            int blk = 2 * t;
+            pf_f32x16 s_nxt;
+            if (blk + 1 < nb_w) {
+                step(s_cur, s_nxt, b0, 1, b0, 0, std::true_type{});
+                prepare(s_nxt, blk + 1);
+                s_cur = s_nxt;
+            } else if (blk < nb_w) {
+                step(s_cur, s_nxt, b0, 1, b0, 0, std::false_type{});
+            }
+            __syncthreads();
+            blk = 2 * t + 1;
+            if (blk + 1 < nb_w) {
+                step(s_cur, s_nxt, b1, 0, b0, 1, std::true_type{});
+                prepare(s_nxt, blk + 1);
+                s_cur = s_nxt;
+            } else if (blk < nb_w) {
+                step(s_cur, s_nxt, b1, 0, b0, 1, std::false_type{});
+            }
+            i0 = i1;
+            i1 = i1 == 2 ? 0 : i1 + 1;
+        }
     }
 
     // the two halves of a query hold disjoint keys: add their sums, then normalise and store
