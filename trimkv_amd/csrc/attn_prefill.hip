@@ -311,21 +311,37 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int last_row = max(n - 1, 0);
 
     // ---- staging: global -> registers -> LDS (K row-major, V transposed) ----
+    // Per-thread pieces are fixed; only the tile base moves.  Rows are addressed as 32-bit byte offsets from the
+    // segment's (wave-uniform) base and clamped to the last row, so every load is unconditional.
     pf_u32x4 kst[PF2_KPIECES], vst[PF2_VPIECES][2];
+    const char* kseg = a.k + row0 * (int64_t)(PF_D * 2);
+    const char* vseg = a.v + row0 * (int64_t)(PF_D * 2);
+    int k_row[PF2_KPIECES], v_row[PF2_VPIECES];
+    uint32_t k_col[PF2_KPIECES], v_col[PF2_VPIECES];
+#pragma unroll
+    for (int i = 0; i < PF2_KPIECES; ++i) {
+        const int p = tid + i * PF2_THREADS;
+        k_row[i] = p >> 4;
+        k_col[i] = (p & 15) * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < PF2_VPIECES; ++i) {
+        const int p = tid + i * PF2_THREADS;
+        v_row[i] = pf2_key_of_slot(pf2_vpiece_sp(p) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
+        v_col[i] = pf2_vpiece_dchunk(p) * 16;
+    }
     auto fetch = [&](int kbase) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < PF2_KPIECES; ++i) {
-            const int p = tid + i * PF2_THREADS;
-            const int row = min(kbase + (p >> 4), last_row);
-            kst[i] = *(const pf_u32x4*)(a.k + (row0 + row) * (int64_t)(PF_D * 2) + (p & 15) * 16);
+            const uint32_t off = (uint32_t)min(kbase + k_row[i], last_row) * (uint32_t)(PF_D * 2) + k_col[i];
+            kst[i] = *(const pf_u32x4*)(kseg + off);
         }
 #pragma unroll
         for (int i = 0; i < PF2_VPIECES; ++i) {
-            const int p = tid + i * PF2_THREADS;
-            const int key = pf2_key_of_slot(pf2_vpiece_sp(p) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
-            const int r0 = min(kbase + key, last_row), r1 = min(kbase + key + 1, last_row);
-            vst[i][0] = *(const pf_u32x4*)(a.v + (row0 + r0) * (int64_t)(PF_D * 2) + pf2_vpiece_dchunk(p) * 16);
-            vst[i][1] = *(const pf_u32x4*)(a.v + (row0 + r1) * (int64_t)(PF_D * 2) + pf2_vpiece_dchunk(p) * 16);
+            const uint32_t o0 = (uint32_t)min(kbase + v_row[i], last_row) * (uint32_t)(PF_D * 2) + v_col[i];
+            const uint32_t o1 = (uint32_t)min(kbase + v_row[i] + 1, last_row) * (uint32_t)(PF_D * 2) + v_col[i];
+            vst[i][0] = *(const pf_u32x4*)(vseg + o0);
+            vst[i][1] = *(const pf_u32x4*)(vseg + o1);
         }
     };
     auto publish = [&](char* buf) __attribute__((always_inline)) {
