@@ -144,6 +144,85 @@ def parity_gate(cache, c, attn_fn, mod):
     return result
 
 
+def prefill_main(args):
+    """Secondary workload (--prefill): chunked prompt processing at BASELINE config 5's shape.  One step = one
+    chunk of 4096 tokens through every layer: append 4096 rows per segment, chunk attention (bottom-right causal,
+    4096 queries x 5 heads per segment over 8192 retained + 4096 new keys) and the eviction back to 8192.
+    The roofline prices the attention kernel against the dense bf16 MFMA peak with its causal flops."""
+    import torch
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    c = dict(CONFIGS[5])
+    if args.layers:
+        c["L"] = args.layers
+    L, B, Hkv, Hq, M, buf = c["L"], c["B"], c["Hkv"], c["Hq"], c["M"], c["buf"]
+    G, S = Hq // Hkv, 4096
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(0)
+
+    class Mod:
+        training = False
+        num_key_value_groups = G
+
+    attn_fn = get_attention_interface("trimkv_hip")
+    cache = TrimKVCache()
+    draw_lb = lambda *shape: torch.nn.functional.logsigmoid(torch.randn(*shape, generator=gen, device=dev) * c["sigma"] + c["mu"])
+    for l in range(L):   # steady state of the chunk loop: M retained tokens per head
+        k = torch.randn(B, Hkv, M, D, generator=gen, device=dev).to(torch.bfloat16)
+        v = torch.randn(B, Hkv, M, D, generator=gen, device=dev).to(torch.bfloat16)
+        cache.update(k, v, draw_lb(B, Hkv, M), torch.arange(M, device=dev), l)
+        del k, v
+    POOL = 2
+    pool = [(torch.randn(B, Hkv, S, D, generator=gen, device=dev).to(torch.bfloat16),
+             torch.randn(B, Hkv, S, D, generator=gen, device=dev).to(torch.bfloat16),
+             draw_lb(B, Hkv, S),
+             torch.randn(B, S, Hq, D, generator=gen, device=dev).to(torch.bfloat16).transpose(1, 2)) for _ in range(POOL)]
+    T = M
+    events = []
+
+    def step(t, sample):
+        nonlocal T
+        pos = torch.arange(T, T + S, device=dev)
+        for l in range(L):
+            kn, vn, lbn, q = pool[(t + l) % POOL]
+            K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            if sample:
+                e0.record()
+            attn_fn(Mod(), q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+            if sample:
+                e1.record()
+                events.append((e0, e1))
+        T += S
+        cache.compress("alpha", M, buf)
+
+    for t in range(args.warmup):
+        step(t, False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for t in range(args.steps):
+        step(args.warmup + t, True)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    n = M + S
+    flops = 4.0 * D * G * B * Hkv * S * (n - S + (S + 1) / 2)     # causal (visible) query-key pairs, two products
+    avg_s = sum(e0.elapsed_time(e1) for e0, e1 in events) * 1e-3 / len(events)
+    out = {
+        "metric": "chunked-prefill tokens/s (append + chunk attention + evict), Qwen3-14B shape", "value": round(B * S * args.steps / seconds, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3 / args.steps, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"BASELINE config 5 ({c['name']} shape) prompt phase: {L} layers, batch {B}, {Hkv} KV heads, {Hq} query heads, "
+                               f"head_dim {D}, chunks of {S} tokens on {M} retained tokens per head, eviction {n} -> {M} after every chunk",
+                   "note": "secondary workload; the headline metric is the default run"},
+        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel", "achieved": round(flops / avg_s / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": round(flops / avg_s / 1e12 / 2500.0, 4), "traffic": None, "avg_launch_us": round(avg_s * 1e6, 1),
+                     "launches_sampled": len(events), "algorithmic_flops_per_launch": int(flops)},
+    }
+    if args.layers:
+        out["config"]["note"] = "layer count overridden: not the BASELINE configuration"
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -162,11 +241,19 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
+    ap.add_argument("--prefill", action="store_true",
+                    help="secondary workload: chunked prompt processing at config 5's shape (4096-token chunks); "
+                         "with it --steps/--warmup count chunks (defaults 6/2)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: the path shards by batch or KV head without communication, "
               "so a multi-GPU figure is N independent copies of this run; --gpus must be 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.prefill:
+        if args.steps == 1024 and args.warmup == 128:
+            args.steps, args.warmup = 6, 2
+        return prefill_main(args)
 
     import torch
     from trimkv_amd import TrimKVCache, get_attention_interface
