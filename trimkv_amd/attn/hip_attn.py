@@ -10,8 +10,9 @@ Three callables with the reference's attention-interface signature
   are a ragged cache's slabs) in ``flash_attn_kwargs``; segment ``b*Hkv+h`` is attended by query
   heads ``h*G .. h*G+G-1`` of batch element ``b`` (flash_attn.py:120-125, 147-149).
 
-Q_LEN == 1 runs ``trimkv_decode_attn``.  Longer query blocks (prompt chunks) are computed with
-torch ops on the same device until the chunk-prefill kernel exists.  As in the reference the
+Q_LEN == 1 runs ``trimkv_decode_attn``; longer query blocks (prompt chunks) run the MFMA kernel
+``trimkv_prefill_attn`` (the dense entry point falls back to torch ops only when an explicit
+``attention_mask`` comes with Q_LEN > 1).  As in the reference the
 ragged entry points ignore ``attention_mask`` and ``scaling`` (flash_attn.py:15, 85; the scale is
 ``D**-0.5``) and apply a bottom-right causal mask when Q_LEN > 1.
 """

@@ -1,0 +1,227 @@
+"""A thin TrimKV Qwen3 decoder on PyTorch-ROCm: the caller either side of the cache hot path.
+
+It exists to run the reference's call order end to end through this package's cache, fused gate and
+attention kernels: per layer ``retention_gate(hidden) -> RoPE -> cache.update -> attention``
+(src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:315-388) and, after the final norm,
+``cache.compress(...)`` when ``config.compress_memory`` (:751-760); a missing cache is created as a
+``TrimKVCache`` (:648-652).  Parameter names follow the reference (``model.layers.N.self_attn.q_proj``,
+``...retention_gate.linear1`` ...), so a local Qwen3 state dict plus ``trimkv_weights.pth`` loads with
+``load_state_dict``; nothing here downloads anything.  The dense projections, norms and RoPE are plain
+torch ops (rocBLAS/hipBLASLt GEMMs); training, the rg2/rg3 gates and generation utilities beyond greedy
+decoding are out of scope.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from types import SimpleNamespace
+from typing import Optional
+
+import torch
+from torch import nn
+import torch.nn.functional as F
+
+from .attn import get_attention_interface
+from .cache_utils import TrimKVCache
+from .gate import RetentionGate
+
+
+@dataclass
+class TrimKVQwen3Config:
+    """The fields of the reference's config that the inference path reads
+    (src/trimkv/models/qwen3/configuration_trimkv_qwen3.py:10-47 on top of HF's Qwen3Config)."""
+    vocab_size: int = 151936
+    hidden_size: int = 4096
+    intermediate_size: int = 12288
+    num_hidden_layers: int = 36
+    num_attention_heads: int = 32
+    num_key_value_heads: int = 8
+    head_dim: int = 128
+    hidden_act: str = "silu"
+    rms_norm_eps: float = 1e-6
+    rope_theta: float = 1_000_000.0
+    attention_bias: bool = False
+    tie_word_embeddings: bool = False
+    initializer_range: float = 0.02
+    retention_gate: Optional[str] = "rg"
+    retention_gate_bias_init: float = 10.0
+    retention_gate_intermediate_size: int = 512
+    memory_size: int = 1024
+    buffer_size: int = 128
+    compress_memory: bool = True
+    compress_strategy: str = "alpha"
+    floor_budget_ratio: float = 0.0
+    alpha_threshold: float = 0.0
+    max_seq_len: int = 131072
+    _attn_implementation: str = "trimkv_hip"
+
+
+class RMSNorm(nn.Module):
+    def __init__(self, dim: int, eps: float):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.variance_epsilon = eps
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        h = x.float()
+        h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * h.to(x.dtype)
+
+
+class MLP(nn.Module):
+    def __init__(self, config: TrimKVQwen3Config):
+        super().__init__()
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype):
+    """cos, sin [B, S, head_dim] of the default RoPE (frequencies theta^(-2i/d), halves concatenated)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=position_ids.device, dtype=torch.float32) / head_dim))
+    ang = position_ids[..., None].float() * inv_freq
+    emb = torch.cat([ang, ang], dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """x [B, H, S, D]; cos/sin [B, S, D]."""
+    half = x.shape[-1] // 2
+    rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
+    return x * cos[:, None] + rot * sin[:, None]
+
+
+class TrimKVQwen3Attention(nn.Module):
+    def __init__(self, config: TrimKVQwen3Config, layer_idx: int):
+        super().__init__()
+        self.config, self.layer_idx = config, layer_idx
+        self.head_dim = config.head_dim
+        self.num_key_value_groups = config.num_attention_heads // config.num_key_value_heads
+        self.scaling = self.head_dim ** -0.5
+        hs, d = config.hidden_size, config.head_dim
+        self.q_proj = nn.Linear(hs, config.num_attention_heads * d, bias=config.attention_bias)
+        self.k_proj = nn.Linear(hs, config.num_key_value_heads * d, bias=config.attention_bias)
+        self.v_proj = nn.Linear(hs, config.num_key_value_heads * d, bias=config.attention_bias)
+        self.o_proj = nn.Linear(config.num_attention_heads * d, hs, bias=config.attention_bias)
+        self.q_norm = RMSNorm(d, config.rms_norm_eps)
+        self.k_norm = RMSNorm(d, config.rms_norm_eps)
+        if config.retention_gate == "rg":
+            self.retention_gate = RetentionGate(hs, config.num_key_value_heads, config.retention_gate_intermediate_size,
+                                                config.retention_gate_bias_init, config.initializer_range, config.hidden_act)
+        elif config.retention_gate is None:
+            self.retention_gate = None
+        else:
+            raise NotImplementedError(f"retention gate {config.retention_gate!r}: only 'rg' is built")
+
+    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
+        B, S, _ = hidden_states.shape
+        shape = (B, S, -1, self.head_dim)
+        q = self.q_norm(self.q_proj(hidden_states).view(shape)).transpose(1, 2)
+        k = self.k_norm(self.k_proj(hidden_states).view(shape)).transpose(1, 2)
+        v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
+        # the gate sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
+        retention = self.retention_gate(hidden_states).transpose(1, 2) if self.retention_gate is not None else None
+        cos, sin = position_embeddings
+        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        offset = past_key_values.get_seq_length(self.layer_idx)
+        k, v, retention, kv_positions, fa_kwargs = past_key_values.update(
+            k, v, retention, cache_position, self.layer_idx,
+            {"sin": sin, "cos": cos, "cache_position": cache_position, "attention_mask": attention_mask})
+        attend = get_attention_interface(self.config._attn_implementation)
+        out, _, _ = attend(self, q, k, v, attention_mask=attention_mask, retention_weights=retention, kv_positions=kv_positions,
+                           offset=offset, dropout=0.0, scaling=self.scaling, sliding_window=None, is_causal=True,
+                           flash_attn_kwargs=fa_kwargs)
+        return self.o_proj(out.reshape(B, S, -1).contiguous())
+
+
+class TrimKVQwen3DecoderLayer(nn.Module):
+    def __init__(self, config: TrimKVQwen3Config, layer_idx: int):
+        super().__init__()
+        self.self_attn = TrimKVQwen3Attention(config, layer_idx)
+        self.mlp = MLP(config)
+        self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
+        hidden_states = hidden_states + self.self_attn(self.input_layernorm(hidden_states), position_embeddings, attention_mask,
+                                                       past_key_values, cache_position)
+        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+
+
+class TrimKVQwen3Model(nn.Module):
+    def __init__(self, config: TrimKVQwen3Config):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList([TrimKVQwen3DecoderLayer(config, i) for i in range(config.num_hidden_layers)])
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, input_ids=None, past_key_values=None, inputs_embeds=None, cache_position=None, position_ids=None,
+                attention_mask=None):
+        if (input_ids is None) == (inputs_embeds is None):
+            raise ValueError("You must specify exactly one of input_ids or inputs_embeds")
+        if inputs_embeds is None:
+            inputs_embeds = self.embed_tokens(input_ids)
+        if past_key_values is None:   # qwen3:648-652
+            past_key_values = TrimKVCache(max_seq_len=self.config.max_seq_len, device=inputs_embeds.device)
+        if cache_position is None:
+            seen = past_key_values.get_seq_length()
+            cache_position = torch.arange(seen, seen + inputs_embeds.shape[1], device=inputs_embeds.device)
+        if position_ids is None:
+            position_ids = cache_position.unsqueeze(0)
+        position_embeddings = rotary_tables(position_ids, self.config.head_dim, self.config.rope_theta, inputs_embeds.dtype)
+        hidden_states = inputs_embeds
+        for layer in self.layers:
+            hidden_states = layer(hidden_states, position_embeddings, attention_mask, past_key_values, cache_position)
+        hidden_states = self.norm(hidden_states)
+        c = self.config
+        if c.compress_memory:   # qwen3:751-760: after every forward, prompt or decode step
+            past_key_values.compress(strategy=c.compress_strategy, memory_size=c.memory_size, buffer_size=c.buffer_size,
+                                     floor_budget_ratio=c.floor_budget_ratio, alpha_threshold=c.alpha_threshold,
+                                     num_layers=c.num_hidden_layers, num_key_value_heads=c.num_key_value_heads)
+        return SimpleNamespace(last_hidden_state=hidden_states, past_key_values=past_key_values)
+
+
+class TrimKVQwen3ForCausalLM(nn.Module):
+    def __init__(self, config: TrimKVQwen3Config):
+        super().__init__()
+        self.config = config
+        self.model = TrimKVQwen3Model(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+        if config.tie_word_embeddings:
+            self.lm_head.weight = self.model.embed_tokens.weight
+        for m in self.modules():   # random init (no checkpoint is fetched): N(0, initializer_range), zero biases
+            if isinstance(m, (nn.Linear, nn.Embedding)):
+                m.weight.data.normal_(mean=0.0, std=config.initializer_range)
+                if getattr(m, "bias", None) is not None:
+                    m.bias.data.zero_()
+        for m in self.modules():
+            if isinstance(m, RetentionGate):
+                m.reset_parameters()
+
+    def forward(self, input_ids=None, past_key_values=None, inputs_embeds=None, cache_position=None, position_ids=None,
+                attention_mask=None, logits_to_keep: int = 0):
+        out = self.model(input_ids, past_key_values, inputs_embeds, cache_position, position_ids, attention_mask)
+        h = out.last_hidden_state
+        if logits_to_keep:
+            h = h[:, -logits_to_keep:]
+        return SimpleNamespace(logits=self.lm_head(h), past_key_values=out.past_key_values)
+
+    @torch.no_grad()
+    def generate(self, input_ids: torch.Tensor, max_new_tokens: int, past_key_values=None, prefill_chunk: int = 0):
+        """Greedy decoding.  ``prefill_chunk`` > 0 streams the prompt in chunks of that many tokens, evicting after
+        each (the long-prompt mode of the reference's examples); returns prompt + new tokens."""
+        chunk = prefill_chunk or input_ids.shape[1]
+        out = None
+        for s in range(0, input_ids.shape[1], chunk):
+            out = self(input_ids[:, s:s + chunk], past_key_values=past_key_values, logits_to_keep=1)
+            past_key_values = out.past_key_values
+        tokens = [input_ids]
+        for i in range(max_new_tokens):
+            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+            tokens.append(nxt)
+            if i + 1 < max_new_tokens:
+                out = self(nxt, past_key_values=past_key_values, logits_to_keep=1)
+        return torch.cat(tokens, dim=1)
