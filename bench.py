@@ -363,7 +363,10 @@ def main():
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
-                "algorithmic_bytes_per_launch": int(avg_bytes)}
+                "algorithmic_bytes_per_launch": int(avg_bytes),
+                "mfma_utilisation": 0.0,
+                "mfma_note": f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
+                             "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
     parity = parity_gate(cache, c, attn_fn, mod)
     out = {
         "metric": METRIC, "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,

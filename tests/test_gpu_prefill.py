@@ -132,6 +132,21 @@ def test_prefill_growing_row_maxima(Q, n):
     assert ok, f"max abs err {err}"
 
 
+def test_prefill_non_positive_scale_long_chunk():
+    """A negative softmax scale (legal for the entry point) turns row maxima into minima: long chunks must still be right."""
+    from trimkv_amd.attn.hip_attn import prefill_attention
+    gen = torch.Generator().manual_seed(77)
+    B, H, G, D, Q, n = 1, 2, 2, 128, 80, 200
+    q = torch.randn(B, H * G, Q, D, generator=gen).to(torch.bfloat16)
+    k = torch.randn(B * H, n, D, generator=gen).to(torch.bfloat16)
+    v = torch.randn(B * H, n, D, generator=gen).to(torch.bfloat16)
+    for scale in (-0.08, 0.0):
+        out = prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), B, H, G, None, None, n, n, scale)
+        want, _ = eager_attention(q.float(), k.float()[None], v.float()[None], G, scale, _bottom_right_mask(Q, n))
+        ok, err = attn_close(out, want)
+        assert ok, (scale, err)
+
+
 def test_prefill_chunk_at_config5_size():
     """Qwen3-14B chunk: 4096 queries on top of 8192 cached keys, G=5 (two segments to bound the run);
     sampled query rows against fp32 on the device."""

@@ -1,0 +1,55 @@
+"""CPU checks of the thin Qwen3 caller: parameter names are the reference's (so its checkpoints load with
+load_state_dict: src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:148-158, 281-312, 405-411, 593-599, 800-803),
+and running it without a GPU fails loudly instead of falling back to a CPU path."""
+import pytest
+import torch
+
+from trimkv_amd.qwen3 import TrimKVQwen3Config, TrimKVQwen3ForCausalLM, apply_rope, rotary_tables
+
+
+def _tiny():
+    return TrimKVQwen3Config(vocab_size=64, hidden_size=512, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
+                             num_key_value_heads=2, head_dim=128, retention_gate_intermediate_size=32)
+
+
+def test_parameter_names_follow_the_reference():
+    keys = set(TrimKVQwen3ForCausalLM(_tiny()).state_dict())
+    per_layer = ["self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight", "self_attn.o_proj.weight",
+                 "self_attn.q_norm.weight", "self_attn.k_norm.weight",
+                 "self_attn.retention_gate.linear1.weight", "self_attn.retention_gate.linear1.bias",
+                 "self_attn.retention_gate.linear2.weight", "self_attn.retention_gate.bias",
+                 "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight",
+                 "input_layernorm.weight", "post_attention_layernorm.weight"]
+    want = {"model.embed_tokens.weight", "model.norm.weight", "lm_head.weight"}
+    want |= {f"model.layers.{l}.{k}" for l in range(2) for k in per_layer}
+    assert keys == want
+
+
+def test_gate_init_matches_reference_reset():
+    m = TrimKVQwen3ForCausalLM(_tiny())
+    g = m.model.layers[0].self_attn.retention_gate
+    assert torch.all(g.bias == 10.0) and torch.all(g.linear1.bias == 0) and g.linear2.bias is None
+    assert 0.01 < g.linear1.weight.std().item() < 0.03
+
+
+def test_rope_is_a_rotation_and_relative():
+    pos = torch.arange(7)[None]
+    cos, sin = rotary_tables(pos, 128, 10000.0, torch.float32)
+    x = torch.randn(1, 2, 7, 128, generator=torch.Generator().manual_seed(0))
+    y = apply_rope(x, cos, sin)
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-4)          # rotations keep the norm
+    assert torch.allclose(y[:, :, 0], x[:, :, 0])                            # position 0 is the identity
+    q = torch.randn(128, generator=torch.Generator().manual_seed(1)); k = torch.randn(128, generator=torch.Generator().manual_seed(2))
+    def dot(i, j):
+        c, s = rotary_tables(torch.tensor([[i, j]]), 128, 10000.0, torch.float64)
+        qq = apply_rope(q.double()[None, None, None].expand(1, 1, 2, 128), c, s)[0, 0, 0]
+        kk = apply_rope(k.double()[None, None, None].expand(1, 1, 2, 128), c, s)[0, 0, 1]
+        return float(qq @ kk)
+    assert abs(dot(3, 1) - dot(10, 8)) < 1e-5                                 # scores depend on the distance only
+
+
+def test_no_cpu_fallback():
+    from trimkv_amd._lib import TrimKVLibraryError
+    m = TrimKVQwen3ForCausalLM(_tiny()).eval()
+    with pytest.raises((TrimKVLibraryError, RuntimeError)):
+        m(torch.zeros(1, 3, dtype=torch.long))

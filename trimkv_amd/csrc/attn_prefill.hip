@@ -528,7 +528,9 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 
 template <int G>
 static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
-    if (a.q_len < 64) {   // short chunks: 16 queries per wavefront waste fewer MFMA columns
+    // short chunks: 16 queries per wavefront waste fewer MFMA columns; a non-positive scale: the large kernel takes
+    // row maxima before scaling, which needs scale > 0
+    if (a.q_len < 64 || !(a.scale_log2 > 0.0f)) {
         using C = SmallCfg<G>;
         const int tiles = (a.q_len + C::BT - 1) / C::BT;
         hipLaunchKernelGGL(prefill_small_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
