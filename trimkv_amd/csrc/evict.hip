@@ -151,6 +151,16 @@ __device__ __forceinline__ void land(int64_t& v) { asm volatile("" : "+v"(v)); }
 // idx[r] (ascending, idx[r] >= r) is the source row of destination row r.  Tile t's destinations
 // [t*R, (t+1)*R) can only overlap sources of tiles <= t, so each tile is loaded whole, the
 // workgroup meets at a barrier with its loads complete, and only then is the tile stored.
+typedef uint32_t ev_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_stream(const char* p) {
+    const ev_u32x4 t = __builtin_nontemporal_load((const ev_u32x4*)p);
+    return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void store_stream(char* p, const uint4& v) {
+    const ev_u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (ev_u32x4*)p);
+}
+
 __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg, int64_t* posseg, const uint32_t* idx,
                                              int kept, int first_moved, int row_bytes, int lpr_shift, int lb_bytes) {
     const int lpr = 1 << lpr_shift;
@@ -171,8 +181,8 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
                 if (src != r) {
                     mv[p] = true;
                     const int64_t o = (int64_t)src * row_bytes + (piece << 4);
-                    kk[p] = *(const uint4*)(kseg + o);
-                    vv[p] = *(const uint4*)(vseg + o);
+                    kk[p] = load_stream(kseg + o);   // rows move once and are next read a whole decode step later:
+                    vv[p] = load_stream(vseg + o);   // streaming (non-temporal) loads and stores
                 }
             }
         }
@@ -184,8 +194,8 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
             if (mv[p]) {
                 const int r = base + p * rpp + rl;
                 const int64_t o = (int64_t)r * row_bytes + (piece << 4);
-                *(uint4*)(kseg + o) = kk[p];
-                *(uint4*)(vseg + o) = vv[p];
+                store_stream(kseg + o, kk[p]);
+                store_stream(vseg + o, vv[p]);
             }
         }
     }
