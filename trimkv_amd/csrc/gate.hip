@@ -45,6 +45,20 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     const uint16_t* xp = a.x + (int64_t)tok * a.hidden + ks * kspan + kg * 8;
     const uint16_t* wp = a.w1 + (int64_t)unit * a.hidden + ks * kspan + kg * 8;
 
+    // Epilogue operands do not depend on the products: request them first so that their latency hides under the main loop.
+    constexpr int HB = 8;                       // heads per epilogue pass
+    const bool epi = tid < TOKENS * GH_UNITS;
+    const int eu = slice * GH_UNITS + (tid & 15);
+    float b1v = 0.0f, w2v[HB];
+#pragma unroll
+    for (int i = 0; i < HB; ++i) w2v[i] = 0.0f;
+    if (epi) {
+        if (a.b1) b1v = bf16_bits_to_f32(a.b1[eu]);
+#pragma unroll
+        for (int i = 0; i < HB; ++i)
+            if (i < a.kv_heads) w2v[i] = bf16_bits_to_f32(a.w2[(int64_t)i * a.inter + eu]);
+    }
+
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < kspan; k0 += 32 * STEPS) {
         bf16x8_t av[STEPS], bv[STEPS];
@@ -65,24 +79,35 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     __syncthreads();
 
     // one (token, unit) per thread: bias, SiLU, then the contraction with W2 over the 16 units
-    if (tid < TOKENS * GH_UNITS) {
+    if (epi) {
         const int t = tid >> 4, u = tid & 15;
         float h = 0.0f;
 #pragma unroll
         for (int i = 0; i < KS; ++i) h += red[i][t][u];
-        const int uu = slice * GH_UNITS + u;
-        if (a.b1) h += bf16_bits_to_f32(a.b1[uu]);
+        h += b1v;
         h = bf16_bits_to_f32(f32_to_bf16_bits(h));            // nn.Linear output in bf16
         float act = h / (1.0f + __expf(-h));
         act = bf16_bits_to_f32(f32_to_bf16_bits(act));        // SiLU output in bf16
-        for (int hh = 0; hh < a.kv_heads; ++hh) {
-            float p = act * bf16_bits_to_f32(a.w2[(int64_t)hh * a.inter + uu]);
-            p += __shfl_xor(p, 1, 64);
-            p += __shfl_xor(p, 2, 64);
-            p += __shfl_xor(p, 4, 64);
-            p += __shfl_xor(p, 8, 64);
-            if (u == 0 && tok0 + t < a.ntok)
-                a.part[((int64_t)slice * a.ntok + tok0 + t) * a.kv_heads + hh] = p;
+        for (int h0 = 0; h0 < a.kv_heads; h0 += HB) {
+            if (h0 > 0) {                                      // more than HB heads: fetch the next batch of W2
+#pragma unroll
+                for (int i = 0; i < HB; ++i)
+                    w2v[i] = h0 + i < a.kv_heads ? bf16_bits_to_f32(a.w2[(int64_t)(h0 + i) * a.inter + eu]) : 0.0f;
+            }
+            float p[HB];
+#pragma unroll
+            for (int i = 0; i < HB; ++i) {
+                p[i] = act * w2v[i];
+                p[i] += __shfl_xor(p[i], 1, 64);
+                p[i] += __shfl_xor(p[i], 2, 64);
+                p[i] += __shfl_xor(p[i], 4, 64);
+                p[i] += __shfl_xor(p[i], 8, 64);
+            }
+            if (u == 0 && tok0 + t < a.ntok) {
+#pragma unroll
+                for (int i = 0; i < HB; ++i)
+                    if (h0 + i < a.kv_heads) a.part[((int64_t)slice * a.ntok + tok0 + t) * a.kv_heads + h0 + i] = p[i];
+            }
         }
     }
 }
