@@ -195,8 +195,11 @@ int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlen
  * or, when seg_start is NULL, at seg*cap.  seg_len may be NULL: every segment then holds max_len
  * rows (a dense cache).  max_len is the caller's upper bound on seg_len (longer segments are
  * truncated to it).  A segment of length 0 yields zeros.
- * Split-K: every segment is cut into chunks of `chunk` rows (0 = chosen from nseg/max_len; one
- * chunk per segment when there are 512 segments or more).  Partial (max, sum, accumulator)
+ * Split-K: every segment is cut into chunks of `chunk` rows (a multiple of 64).  0 lets the library
+ * choose from nseg and max_len alone -- one chunk per segment from 128 segments on, which is right
+ * for near-equal lengths; a caller that knows its lengths are very uneven should pass about
+ * total_rows / 512 (at least 512) so that a few long segments do not run on one workgroup each
+ * (the Python ragged caches do).  Partial (max, sum, accumulator)
  * triples go through `workspace` (trimkv_decode_attn_workspace bytes, 0 when nothing is split) and
  * are merged by a second, tiny kernel.  Calls that share a workspace must be ordered (same stream).
  * head_dim must be 128; group in [1, 8]; dtype bf16.
