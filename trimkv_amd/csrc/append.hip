@@ -83,6 +83,60 @@ __global__ __launch_bounds__(AP_THREADS) void append_kernel(AppendArgs a) {
     }
 }
 
+// Decode-sized appends (all new 16-byte pieces of a segment fit one wavefront): one wavefront per segment.  Every
+// load -- the old length, the new K/V pieces, log(beta) or the gate partials, the position -- is issued before
+// anything waits, so the kernel costs one memory round trip instead of two; no barrier is needed because a single
+// wavefront reads the length before its lane 0 rewrites it (program order).
+template <bool GATED>
+__global__ __launch_bounds__(64) void append_small_kernel(AppendArgs a) {
+    const int seg = blockIdx.x, lane = threadIdx.x;
+    const int b = seg / a.kv_heads, h = seg - b * a.kv_heads;
+    const int lpr = a.row_bytes >> 4;
+    const int pieces = a.s_new * lpr;
+    const int n0 = a.seg_len[seg];
+    const int s = lane / lpr, piece = lane - s * lpr;
+    uint4 kq = make_uint4(0, 0, 0, 0), vq = kq;
+    if (lane < pieces) {
+        const int64_t so = (int64_t)b * a.kv_sb + (int64_t)h * a.kv_sh + (int64_t)s * a.kv_ss + ((int64_t)piece << 4);
+        kq = *(const uint4*)(a.k_new + so);
+        vq = *(const uint4*)(a.v_new + so);
+    }
+    float lb = 0.0f;
+    int64_t pos = 0;
+    if (lane < a.s_new) {
+        if (!GATED) lb = load_as_f32(a.lb_new, (int64_t)b * a.lb_sb + (int64_t)h * a.lb_sh + (int64_t)lane * a.lb_ss, a.lb_dtype);
+        pos = a.pos_new[(int64_t)b * a.pos_sb + (int64_t)h * a.pos_sh + (int64_t)lane * a.pos_ss];
+    }
+    if (GATED) {   // same summation order as the large kernel: lane-strided partial sums, then a fixed butterfly
+        const int64_t ntok = (int64_t)(a.nseg / a.kv_heads) * a.s_new;
+        for (int r = 0; r < a.s_new; ++r) {
+            const int64_t tok = (int64_t)b * a.s_new + r;
+            float acc = 0.0f;
+            for (int j = lane; j < a.gate_nslice; j += 64) acc += a.gate_part[((int64_t)j * ntok + tok) * a.kv_heads + h];
+#pragma unroll
+            for (int d = 32; d > 0; d >>= 1) acc += __shfl_xor(acc, d, 64);
+            acc = round_to_dtype(acc, a.lb_dtype);
+            const float v = log_sigmoid(round_to_dtype(acc + a.gate_bias[h], a.lb_dtype));
+            if (lane == r) lb = v;
+        }
+    }
+    if (n0 < 0 || n0 + a.s_new > a.cap) return;   // never write past the slab
+    const int64_t dst_row0 = (int64_t)seg * a.cap + n0;
+    if (lane < pieces) {
+        const int64_t d = (dst_row0 + s) * a.row_bytes + ((int64_t)piece << 4);
+        *(uint4*)(a.k_slab + d) = kq;
+        *(uint4*)(a.v_slab + d) = vq;
+    }
+    if (lane < a.s_new) {
+        store_from_f32(a.lb_slab, dst_row0 + lane, a.lb_dtype, lb);
+        a.pos_slab[dst_row0 + lane] = pos;
+    }
+    if (lane == 0) {
+        a.seg_len[seg] = n0 + a.s_new;
+        if (a.cu) a.cu[seg + 1] += (seg + 1) * a.s_new;
+    }
+}
+
 // Used when one segment's new rows are spread over several workgroups: lengths advance only
 // after every copy of the append launch has read the old ones (stream order).
 __global__ void bump_len_kernel(int32_t* seg_len, int32_t* cu, int nseg, int cap, int s_new) {
@@ -129,6 +183,12 @@ static int append_common(bool gated, void* k_slab, void* v_slab, void* lb_slab, 
     const int ny = (s_new + AP_ROWS_PER_BLOCK - 1) / AP_ROWS_PER_BLOCK;
     a.bump_in_kernel = (ny == 1);
     hipStream_t st = (hipStream_t)stream;
+    if (s_new * (row_bytes >> 4) <= 64) {   // decode: one wavefront per segment
+        a.bump_in_kernel = 1;
+        if (gated) hipLaunchKernelGGL(append_small_kernel<true>, dim3(nseg), dim3(64), 0, st, a);
+        else hipLaunchKernelGGL(append_small_kernel<false>, dim3(nseg), dim3(64), 0, st, a);
+        return launch_status(fn);
+    }
     dim3 grid(nseg, ny);
     if (gated) hipLaunchKernelGGL(append_kernel<true>, grid, dim3(AP_THREADS), 0, st, a);
     else hipLaunchKernelGGL(append_kernel<false>, grid, dim3(AP_THREADS), 0, st, a);
