@@ -89,5 +89,10 @@ def ptr(t) -> int:
 
 
 def current_stream(device) -> int:
+    """Raw hipStream_t of torch's current stream on ``device`` (the fast C accessor when torch has it)."""
     import torch
+    raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+    if raw is not None:
+        idx = device.index if isinstance(device, torch.device) else torch.device(device).index
+        return raw(torch.cuda.current_device() if idx is None else idx)
     return torch.cuda.current_stream(device).cuda_stream

@@ -92,16 +92,16 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     G = Hq // Hkv
     scale = D ** -0.5 if scaling is None else scaling
     if Q == 1 and attention_mask is None:
-        ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
-              and value.stride() == key.stride() and key.stride(1) % D == 0)
-        if not ok:
+        ks = key.stride()
+        if not (ks[3] == 1 and ks[2] == D and ks[0] == Hkv * ks[1] and value.stride() == ks and ks[1] % D == 0):
             key, value = key.contiguous(), value.contiguous()
-        cap = key.stride(1) // D
+            ks = key.stride()
+        cap = ks[1] // D
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        seg_len = (flash_attn_kwargs or {}).get("seg_len")
-        if seg_len is not None and (seg_len.numel() != B * Hkv or (flash_attn_kwargs or {}).get("max_len") != n):
+        seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
+        if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
         out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale)
         return out.view(B, 1, Hq, D), None, None

@@ -89,7 +89,7 @@ class LazyLogBeta:
 class _Slab:
     """Device storage of one layer."""
 
-    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len")
+    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -102,6 +102,16 @@ class _Slab:
         self.cu = torch.zeros(nseg + 1, dtype=torch.int32, device=device) if ragged else None
         self.lens = np.zeros(nseg, dtype=np.int64)  # exact host mirror of seg_len
         self.max_len = 0
+        self._refresh_views()
+
+    def _refresh_views(self) -> None:
+        """[B,Hkv,cap,...] views of the slabs and their addresses, rebuilt only when storage changes: the per-step
+        views handed to callers are one narrow() of these."""
+        B, H, cap, D = self.B, self.H, self.cap, self.D
+        self.k4, self.v4 = self.k.view(B, H, cap, D), self.v.view(B, H, cap, D)
+        self.lb3, self.pos3 = self.lb.view(B, H, cap), self.pos.view(B, H, cap)
+        self.ptrs = (self.k.data_ptr(), self.v.data_ptr(), self.lb.data_ptr(), self.pos.data_ptr(), self.seg_len.data_ptr(),
+                     None if self.cu is None else self.cu.data_ptr())
 
     @property
     def nseg(self) -> int:
@@ -117,6 +127,7 @@ class _Slab:
                 new[:, :keep] = old[:, :keep]
             setattr(self, name, new)
         self.cap = new_cap
+        self._refresh_views()
 
 
 def _require_cuda(t: torch.Tensor, what: str) -> None:
@@ -182,7 +193,8 @@ class _SlabBacked(_CacheBase):
                 slab.regrow(self._new_capacity(slab, slab.max_len + S, S))
         if v.shape != k.shape or v.dtype != k.dtype:
             raise ValueError("value_states must match key_states in shape and dtype")
-        if k.stride(3) != 1 or (k.stride(0) * 2) % 16 or (k.stride(1) * 2) % 16 or (k.stride(2) * 2) % 16 or k.data_ptr() % 16:
+        ks = k.stride()
+        if ks[3] != 1 or (ks[0] | ks[1] | ks[2]) % 8 or k.data_ptr() % 16:
             k = k.contiguous()
         if v.stride() != k.stride() or v.data_ptr() % 16:
             v = v.contiguous()
@@ -200,9 +212,9 @@ class _SlabBacked(_CacheBase):
             ps = pos.stride()
         lib = _lib.load()
         st = _lib.current_stream(k.device)
-        common = (slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
-                  _lib.ptr(slab.cu), slab.nseg, H, slab.cap, D, _lib.dtype_code(k.dtype), _lib.dtype_code(slab.lb.dtype),
-                  k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2))
+        ks = k.stride()
+        common = (*slab.ptrs, slab.nseg, H, slab.cap, D, _lib.dtype_code(k.dtype), _lib.dtype_code(slab.lb.dtype),
+                  k.data_ptr(), v.data_ptr(), ks[0], ks[1], ks[2])
         if lazy:
             if not lb.transposed or lb.shape != (B, H, S):
                 raise ValueError("a lazy log-beta must be the [B,Hkv,S] transpose of the gate output")
@@ -249,6 +261,8 @@ class _SlabBacked(_CacheBase):
 class _DenseViews:
     """List-like ``cache.key_cache`` etc.: item ``l`` is the live ``[B,Hkv,n,...]`` view of layer l."""
 
+    _BASE = {"k": "k4", "v": "v4", "lb": "lb3", "pos": "pos3"}
+
     def __init__(self, cache: "TrimKVCache", which: str):
         self._c, self._w = cache, which
 
@@ -263,11 +277,7 @@ class _DenseViews:
         s = self._c._slabs[layer]
         if s is None:
             return _EMPTY()
-        n = s.max_len
-        t = getattr(s, self._w)
-        if self._w in ("k", "v"):
-            return t.view(s.B, s.H, s.cap, s.D)[:, :, :n]
-        return t.view(s.B, s.H, s.cap)[:, :, :n]
+        return getattr(s, self._BASE[self._w]).narrow(2, 0, s.max_len)
 
     def __iter__(self):
         return (self[i] for i in range(len(self)))
@@ -300,7 +310,11 @@ class TrimKVCache(_SlabBacked):
         return _DenseViews(self, "pos")
 
     def _layer_tuple(self, layer: int):
-        return (self.key_cache[layer], self.value_cache[layer], self.retention_weights[layer], self.kv_positions[layer])
+        s = self._slabs[layer]
+        if s is None:
+            return (self.key_cache[layer], self.value_cache[layer], self.retention_weights[layer], self.kv_positions[layer])
+        n = s.max_len
+        return (s.k4.narrow(2, 0, n), s.v4.narrow(2, 0, n), s.lb3.narrow(2, 0, n), s.pos3.narrow(2, 0, n))
 
     def __getitem__(self, layer_idx: int):
         if layer_idx < len(self):
@@ -403,6 +417,7 @@ class TrimKVCache(_SlabBacked):
             slab.seg_len = slab.seg_len.view(slab.B, slab.H)[idx].reshape(-1).contiguous()
             slab.lens = slab.lens.reshape(slab.B, slab.H)[idx.cpu().numpy()].reshape(-1).copy()
             slab.B = nb
+            slab._refresh_views()
 
     def batch_split(self, full_batch_size: int, split_size: int) -> List["TrimKVCache"]:
         out = []
@@ -421,6 +436,7 @@ class TrimKVCache(_SlabBacked):
                 new.k, new.v, new.lb, new.pos = slab.k[lo:hi], slab.v[lo:hi], slab.lb[lo:hi], slab.pos[lo:hi]
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
                 new.lens, new.max_len = slab.lens[lo:hi].copy(), slab.max_len
+                new._refresh_views()
                 part._slabs.append(new)
             out.append(part)
         return out
@@ -452,6 +468,7 @@ class TrimKVCache(_SlabBacked):
             c.k, c.v, c.lb, c.pos = (t.to(device, copy=True) for t in (slab.k, slab.v, slab.lb, slab.pos))
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
             c.lens, c.max_len = slab.lens.copy(), slab.max_len
+            c._refresh_views()
             new._slabs.append(c)
         return new
 
