@@ -94,8 +94,11 @@ struct AttnArgs {
     float* ws_o; float* ws_ml;
 };
 
+// Attention of the G query heads of segment `seg` over its rows [t0, t1): the body shared by both kernels.
+// `direct`: normalise and write the output; otherwise the unnormalised accumulator and (max, sum) go to partial
+// slot `slot` of the workspace.  All 256 threads of the workgroup must call it together (it uses barriers).
 template <int G>
-__global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2))) void decode_attn_kernel(AttnArgs a) {
+__device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base) {
     using C = AttnCfg<G>;
     constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
 
@@ -105,27 +108,8 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
     __shared__ float sm[AT_WAVES][8];
     __shared__ float sl[AT_WAVES][8];
 
-    // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
-    // axis so that consecutive ids are different segments: with the split as the fast axis and 8
-    // splits, every "split 0" workgroup would land on the same XCD, and ragged lengths (most
-    // segments need one or two splits) would leave most of the chip idle.
-    // High splits exist only for the longest segments; they are dispatched first so that the few
-    // long segments do not form the tail of the launch.
-    const int seg = blockIdx.x, split = (int)gridDim.y - 1 - (int)blockIdx.y;
-    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
-    n = max(0, min(n, a.max_len));
-    const int nsp = (n + a.chunk - 1) / a.chunk;
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int c = lane & 15, r = lane >> 4;
-
-    if (split >= nsp) {
-        if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
-            for (int i = tid; i < G * AT_D; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * AT_D + i] = 0;
-        }
-        return;
-    }
-    const int rps = (n + nsp - 1) / nsp;
-    const int t0 = split * rps, t1 = min(n, t0 + rps);
     const int pw = (t1 - t0 + AT_WAVES - 1) / AT_WAVES;
     const int w0 = t0 + w * pw, w1 = min(t1, w0 + pw);
 
@@ -349,15 +333,38 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
             acc += f * so[ww][g][d];
             lsum += f * sl[ww][g];
         }
-        if (a.direct) {
+        if (direct) {
             const float y = lsum > 0.0f ? acc / lsum : 0.0f;
             ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
         } else {
-            const int64_t slot = ((int64_t)seg * a.nsplit + split) * G + g;
+            const int64_t slot = slot_base * G + g;
             a.ws_o[slot * AT_D + d] = acc;
             if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
         }
     }
+}
+
+template <int G>
+__global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2))) void decode_attn_kernel(AttnArgs a) {
+    // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
+    // axis so that consecutive ids are different segments: with the split as the fast axis and 8
+    // splits, every "split 0" workgroup would land on the same XCD, and ragged lengths (most
+    // segments need one or two splits) would leave most of the chip idle.
+    // High splits exist only for the longest segments; they are dispatched first so that the few
+    // long segments do not form the tail of the launch.
+    const int seg = blockIdx.x, split = (int)gridDim.y - 1 - (int)blockIdx.y;
+    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
+    n = max(0, min(n, a.max_len));
+    const int nsp = (n + a.chunk - 1) / a.chunk;
+    if (split >= nsp) {
+        if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
+            for (int i = threadIdx.x; i < G * AT_D; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * AT_D + i] = 0;
+        }
+        return;
+    }
+    const int rps = (n + nsp - 1) / nsp;
+    const int t0 = split * rps, t1 = min(n, t0 + rps);
+    attend_rows<G>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split);
 }
 
 // Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
