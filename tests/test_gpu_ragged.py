@@ -301,3 +301,27 @@ def test_empty_segments_yield_zeros_and_q_len_gt_1_is_causal_bottom_right():
     out3, _, _ = attn(_Mod(), q3.to(DEV), k.to(DEV), v.to(DEV), None, flash_attn_kwargs=kw)
     want3 = ragged_attention(q3, k, v, cu, H)
     assert out3.shape == (B, 3, H * G, D) and attn_close(out3, want3)[0]
+
+
+def test_decode_attention_dispatch_order_changes_nothing_but_scheduling():
+    """seg_order (longest first) permutes which workgroup handles which segment; results are bit-identical, with and
+    without split-K, and out-of-range entries are clamped instead of read."""
+    from trimkv_amd.attn.hip_attn import decode_attention
+    gen = torch.Generator().manual_seed(11)
+    nseg, G, D, cap = 40, 4, 128, 1500
+    rng = np.random.default_rng(11)
+    lens = rng.integers(0, cap, size=nseg).astype(np.int32)
+    k = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    v = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    q = torch.randn(nseg * G, D, generator=gen).to(torch.bfloat16).to(DEV)
+    L = torch.from_numpy(lens).to(DEV)
+    order = torch.from_numpy(np.argsort(-lens, kind="stable").astype(np.int32)).to(DEV)
+    for chunk in (0, 512):
+        base = decode_attention(q, k, v, nseg, G, L, None, cap, cap, D ** -0.5, chunk=chunk)
+        perm = decode_attention(q, k, v, nseg, G, L, None, cap, cap, D ** -0.5, chunk=chunk, seg_order=order)
+        assert torch.equal(base, perm)
+    wild = order.clone()
+    wild[0], wild[1] = -5, 10_000          # clamped to segments 0 and nseg-1: no fault, the other segments unaffected
+    got = decode_attention(q, k, v, nseg, G, L, None, cap, cap, D ** -0.5, chunk=512, seg_order=wild)
+    untouched = [s for s in range(1, nseg - 1) if s not in (int(order[0]), int(order[1]))]
+    assert torch.equal(got.view(nseg, G, D)[untouched], base.view(nseg, G, D)[untouched])

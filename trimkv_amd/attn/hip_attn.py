@@ -41,8 +41,9 @@ def _workspace(device, nbytes: int) -> Optional[torch.Tensor]:
 
 def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, nseg: int, group: int,
                      seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
-                     scale: float, chunk: int = 0) -> torch.Tensor:
-    """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``."""
+                     scale: float, chunk: int = 0, seg_order: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``.
+    ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only)."""
     if not query.is_cuda:
         raise _lib.TrimKVLibraryError("decode attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
     lib = _lib.load()
@@ -51,7 +52,7 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
     ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, max_len, chunk)
     ws = _workspace(query.device, ws_bytes)
     rc = lib.trimkv_decode_attn(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(),
-                                _lib.ptr(seg_len), _lib.ptr(seg_start), nseg, cap, d, group, _lib.dtype_code(query.dtype),
+                                _lib.ptr(seg_len), _lib.ptr(seg_start), _lib.ptr(seg_order), nseg, cap, d, group, _lib.dtype_code(query.dtype),
                                 float(scale), max_len, chunk, _lib.ptr(ws), 0 if ws is None else ws.numel(),
                                 _lib.current_stream(query.device))
     _lib.check(rc, "trimkv_decode_attn")
@@ -155,7 +156,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         if not q2.is_contiguous():
             q2 = q2.contiguous()
         out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5,
-                               chunk=kw.get("chunk", 0))
+                               chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"))
         return out.view(B, 1, Hq, D), None, None
     out = prefill_attention(query, key, value, batch_size, num_kv_heads, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5)
     return out, None, None

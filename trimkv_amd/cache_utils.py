@@ -89,7 +89,7 @@ class LazyLogBeta:
 class _Slab:
     """Device storage of one layer."""
 
-    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs")
+    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -102,6 +102,7 @@ class _Slab:
         self.cu = torch.zeros(nseg + 1, dtype=torch.int32, device=device) if ragged else None
         self.lens = np.zeros(nseg, dtype=np.int64)  # exact host mirror of seg_len
         self.max_len = 0
+        self.order = None  # ragged caches: segments by decreasing length/budget (dispatch order of the attention launch)
         self._refresh_views()
 
     def _refresh_views(self) -> None:
@@ -435,7 +436,7 @@ class TrimKVCache(_SlabBacked):
                 lo, hi = i * slab.H, (i + nb) * slab.H
                 new.k, new.v, new.lb, new.pos = slab.k[lo:hi], slab.v[lo:hi], slab.lb[lo:hi], slab.pos[lo:hi]
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
-                new.lens, new.max_len = slab.lens[lo:hi].copy(), slab.max_len
+                new.lens, new.max_len, new.order = slab.lens[lo:hi].copy(), slab.max_len, None
                 new._refresh_views()
                 part._slabs.append(new)
             out.append(part)
@@ -467,7 +468,7 @@ class TrimKVCache(_SlabBacked):
             c.B, c.H, c.D, c.cap = slab.B, slab.H, slab.D, slab.cap
             c.k, c.v, c.lb, c.pos = (t.to(device, copy=True) for t in (slab.k, slab.v, slab.lb, slab.pos))
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
-            c.lens, c.max_len = slab.lens.copy(), slab.max_len
+            c.lens, c.max_len, c.order = slab.lens.copy(), slab.max_len, None
             c._refresh_views()
             new._slabs.append(c)
         return new
@@ -548,7 +549,8 @@ class _RaggedCache(_SlabBacked):
         # (the library's own default assumes every segment is max_len long)
         chunk = max(512, ((int(slab.lens.sum()) // 512 + 63) // 64) * 64)
         kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu,
-              "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len, "chunk": chunk}
+              "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len, "chunk": chunk,
+              "seg_order": slab.order}
         flat = (slab.k.view(-1, slab.D), slab.v.view(-1, slab.D), slab.lb.view(-1, 1), slab.pos.view(-1, 1))
         return flat, kw
 
@@ -640,6 +642,18 @@ class _RaggedCache(_SlabBacked):
             for i, l in enumerate(layers):
                 self._slabs[l].lens = lens[i].copy()
                 self._slabs[l].max_len = int(lens[i].max())
+                if getattr(self, "_budgets_host", None) is None:
+                    self._set_dispatch_order(self._slabs[l], lens[i])
+
+    @staticmethod
+    def _set_dispatch_order(slab: _Slab, key) -> None:
+        """Very uneven segments: hand the attention launch the segments longest first (``key`` = lengths or budgets),
+        so that the long ones are not dispatched last.  Near-equal lengths need no order."""
+        key = np.asarray(key, dtype=np.int64)
+        if key.size < 16 or int(key.max()) * key.size <= 1.5 * max(1, int(key.sum())):
+            slab.order = None
+        else:
+            slab.order = torch.from_numpy(np.argsort(-key, kind="stable").astype(np.int32)).to(slab.k.device)
 
     def set_budgets(self, budgets) -> None:
         """Give every segment its own token budget: ``budgets`` is ``[nseg]`` (all layers alike) or
@@ -647,6 +661,9 @@ class _RaggedCache(_SlabBacked):
         arr = np.asarray(budgets.cpu() if torch.is_tensor(budgets) else budgets, dtype=np.int64)
         self._budgets_host = arr
         self._budgets_dev: Dict[Any, torch.Tensor] = {}
+        for l, slab in enumerate(self._slabs):
+            if slab is not None:
+                self._set_dispatch_order(slab, arr if arr.ndim == 1 else arr[l])
 
     def evict_to_budgets(self, buffer_size: int = 0, strategy: str = "alpha", layers: Optional[List[int]] = None) -> None:
         """Per-head budgets: segment ``seg`` of every listed layer is cut to its ``budget[seg]`` best

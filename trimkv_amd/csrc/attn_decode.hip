@@ -88,7 +88,7 @@ __device__ __forceinline__ float reduce16_transposed(float (&v)[16], int c) {
 
 struct AttnArgs {
     const uint4* q; void* out; const uint4* k; const uint4* v;
-    const int32_t* seg_len; const int32_t* seg_start;
+    const int32_t* seg_len; const int32_t* seg_start; const int32_t* seg_order;
     int nseg, cap, max_len, chunk, nsplit, direct;
     float scale_log2;
     float* ws_o; float* ws_ml;
@@ -352,7 +352,11 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
     // segments need one or two splits) would leave most of the chip idle.
     // High splits exist only for the longest segments; they are dispatched first so that the few
     // long segments do not form the tail of the launch.
-    const int seg = blockIdx.x, split = (int)gridDim.y - 1 - (int)blockIdx.y;
+    // seg_order (optional): the segment each grid column works on, longest first, so that with very uneven lengths
+    // the long segments are dispatched first instead of forming the tail of the launch.
+    int seg = blockIdx.x;
+    if (a.seg_order) seg = min(max(a.seg_order[seg], 0), a.nseg - 1);
+    const int split = (int)gridDim.y - 1 - (int)blockIdx.y;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
     const int nsp = (n + a.chunk - 1) / a.chunk;
@@ -440,7 +444,7 @@ extern "C" size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim
 }
 
 extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
-                                  const int32_t* seg_len, const int32_t* seg_start,
+                                  const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
                                   int nseg, int cap, int head_dim, int group, int dtype, float scale,
                                   int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_decode_attn";
@@ -455,7 +459,7 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     if (chunk % 64) return fail(TRIMKV_ERR_SHAPE, "%s: chunk must be a multiple of 64 (got %d)", fn, chunk);
     AttnArgs a;
     a.q = (const uint4*)q; a.out = out; a.k = (const uint4*)k_slab; a.v = (const uint4*)v_slab;
-    a.seg_len = seg_len; a.seg_start = seg_start; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
+    a.seg_len = seg_len; a.seg_start = seg_start; a.seg_order = seg_order; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
     a.nsplit = (max_len + chunk - 1) / chunk;
     if (a.nsplit > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: max_len/chunk = %d splits exceeds the grid limit 65535", fn, a.nsplit);
     a.direct = a.nsplit <= 1;
