@@ -227,3 +227,30 @@ def test_config5_long_prompt_streamed_in_chunks_then_decode():
         assert ok, err
         cache.compress("alpha", M, buf)
     assert cache.get_cache_length(0) == M + 8
+
+
+def test_uncompressed_long_context_decode_and_chunk():
+    """A cache that is never evicted (compress_memory off) at a 100k-token context: decode attention splits each of
+    the 8 segments 32 ways; a 512-token chunk on top of it runs the MFMA kernel.  Checked against fp32 on the device."""
+    from trimkv_amd.attn.hip_attn import decode_attention, prefill_attention
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    B, H, G, D, n = 1, 8, 2, 128, 100_003
+    k = torch.randn(B * H, n, D, generator=gen, device=DEV).to(torch.bfloat16)
+    v = torch.randn(B * H, n, D, generator=gen, device=DEV).to(torch.bfloat16)
+    q = torch.randn(B * H * G, D, generator=gen, device=DEV).to(torch.bfloat16)
+    out = decode_attention(q, k, v, B * H, G, None, None, n, n, D ** -0.5)
+    p = torch.softmax(torch.einsum("sgd,snd->sgn", q.view(B * H, G, D).float(), k.float()) * D ** -0.5, -1)
+    want = torch.einsum("sgn,snd->sgd", p, v.float())
+    ok, err = attn_close(out.view(B * H, G, D), want)
+    assert ok, err
+    Q = 512
+    qc = torch.randn(B, H * G, Q, D, generator=gen, device=DEV).to(torch.bfloat16)
+    outc = prefill_attention(qc, k, v, B, H, G, None, None, n, n, D ** -0.5)
+    rows = torch.tensor([0, 63, 64, 255, 511], device=DEV)
+    for seg in (0, 5):
+        for g in range(G):
+            s = (qc[0, seg * G + g, rows].float() @ k[seg].float().T) * D ** -0.5
+            vis = torch.arange(n, device=DEV)[None, :] <= (n - Q + rows)[:, None]
+            want = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ v[seg].float()
+            ok, err = attn_close(outc[0, rows, seg * G + g], want)
+            assert ok, (seg, g, err)
