@@ -21,25 +21,32 @@ TRIMKV_ATTENTION_IMPLEMENTATIONS = {
 }
 
 
-def get_trimkv_wrapper(attn_impl: str):
+_TRIMKV_ONLY_KWARGS = frozenset(("retention_weights", "kv_positions", "rg_dropout", "flash_attn_kwargs"))
+
+
+def _adapt_hf_attention(name: str):
+    """HF's attention function ``name`` behind the TrimKV calling convention: the TrimKV-only keyword arguments are
+    removed before the call and a third ``None`` is appended to its ``(output, weights)`` result."""
     from transformers.modeling_utils import ALL_ATTENTION_FUNCTIONS
 
-    attn_fn = ALL_ATTENTION_FUNCTIONS[attn_impl]
+    hf_attention = ALL_ATTENTION_FUNCTIONS[name]
 
-    def attn_wrapper(*args, **kwargs):
-        for name in ("retention_weights", "kv_positions", "rg_dropout", "flash_attn_kwargs"):
-            kwargs.pop(name, None)
-        attn_output, attn_weights = attn_fn(*args, **kwargs)
-        return attn_output, attn_weights, None
+    def adapted(module, query, key, value, attention_mask=None, **kwargs):
+        passed_on = {k: v for k, v in kwargs.items() if k not in _TRIMKV_ONLY_KWARGS}
+        output, weights = hf_attention(module, query, key, value, attention_mask, **passed_on)
+        return output, weights, None
 
-    return attn_wrapper
+    return adapted
 
 
-def get_attention_interface(attn_impl: str, compile=False):
-    if attn_impl in TRIMKV_ATTENTION_IMPLEMENTATIONS:
-        attention_inference = TRIMKV_ATTENTION_IMPLEMENTATIONS[attn_impl]
-    else:
-        attention_inference = get_trimkv_wrapper(attn_impl)
-    if compile:
-        attention_inference = torch.compile(attention_inference)
-    return attention_inference
+get_trimkv_wrapper = _adapt_hf_attention   # the reference's name for the same adapter
+
+
+def get_attention_interface(attn_impl: str, compile: bool = False):
+    """Name -> callable.  ``compile`` wraps an HF fallback in ``torch.compile`` as the reference does; the entries backed
+    by libtrimkv_hip.so are ctypes launches of hand-written kernels and are returned as they are."""
+    native = TRIMKV_ATTENTION_IMPLEMENTATIONS.get(attn_impl)
+    if native is not None:
+        return native
+    adapted = _adapt_hf_attention(attn_impl)
+    return torch.compile(adapted) if compile else adapted
