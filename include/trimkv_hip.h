@@ -164,6 +164,24 @@ int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* po
                            void* stream);
 
 /*
+ * trimkv_group_threshold_wide -- the same selection with the same outputs, spread over one
+ * workgroup per (layer, segment) instead of one per group: four histogram launches (one per key
+ * byte), a count launch and a scan launch.  For large groups -- one sequence's budget over all
+ * layers and heads is about 10^6 scores (cache_utils.py:418-472) -- this takes tens of
+ * microseconds where a single workgroup takes milliseconds; for small groups (one layer of one
+ * batch element) trimkv_group_threshold is the cheaper call.  workspace:
+ * trimkv_group_threshold_workspace bytes, 4-byte aligned.
+ */
+size_t trimkv_group_threshold_workspace(int nlayers, int nseg, int segs_per_group);
+int trimkv_group_threshold_wide(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+                                const void* const* k_slabs, const int32_t* const* seg_lens,
+                                int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
+                                int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
+                                int64_t q_idx, int strategy, int rounding,
+                                uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * trimkv_compact_threshold -- in-place compaction of one layer against group thresholds:
  * keeps token i of segment seg iff key_i > thr_key[g] or (key_i == thr_key[g] and its rank
  * among equal keys, tie_base[seg] + rank inside the segment, is < tie_take[g]); g =
@@ -176,6 +194,48 @@ int trimkv_compact_threshold(void* k_slab, void* v_slab, void* lb_slab, int64_t*
                              const uint32_t* thr_key, const int32_t* tie_take, const int32_t* tie_base,
                              int64_t q_idx, int strategy, int rounding, int max_len,
                              void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * One layer's slabs, for the entry points that work on several layers in one launch.  The table
+ * (nlayers entries) lives in device memory.
+ */
+typedef struct trimkv_layer_slabs {
+    void* k_slab;        /* [nseg][cap][head_dim] */
+    void* v_slab;
+    void* lb_slab;       /* [nseg][cap] log beta */
+    int64_t* pos_slab;   /* [nseg][cap] */
+    int32_t* seg_len;    /* [nseg], updated */
+    int64_t q_idx;       /* tokens seen by this layer + 1 (cache_utils.py:173) */
+    int32_t cap;         /* rows per segment in this layer's slabs */
+    int32_t reserved;
+} trimkv_layer_slabs;
+
+/*
+ * trimkv_evict_layers -- trimkv_evict for nlayers layers in ONE launch: the loop over layers of
+ * TrimKVCache.compress (src/trimkv/cache_utils.py:152-158) and of the per-head selections
+ * (:508-521).  With a handful of segments per layer (small batches) one launch per layer leaves
+ * the chip idle; here the grid is nseg x nlayers workgroups.  keep_per_seg (optional) is [nseg]
+ * (keep_layer_stride = 0: the same budgets for every layer) or [nlayers][nseg]
+ * (keep_layer_stride = nseg).  max_len bounds every layer's segment lengths and must not exceed any
+ * layer's cap; workspace: nlayers * trimkv_evict_workspace(nseg, max_len) bytes.
+ */
+int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                        int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                        int strategy, int rounding, int sliding_window, int max_len,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * trimkv_compact_threshold_layers -- trimkv_compact_threshold for nlayers layers in one launch
+ * (the per-layer rebuild loops at cache_utils.py:466-482, 912-943).  thr_key / tie_take are
+ * [ngroups] shared by all layers (thr_layer_stride = 0: one budget across layers) or
+ * [nlayers][ngroups] (thr_layer_stride = ngroups: layer-wise budgets); tie_base is [nlayers][nseg]
+ * as trimkv_group_threshold writes it.
+ */
+int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int segs_per_group, int head_dim,
+                                    int kv_dtype, int lb_dtype,
+                                    const uint32_t* thr_key, const int32_t* tie_take, int thr_layer_stride,
+                                    const int32_t* tie_base, int strategy, int rounding, int max_len,
+                                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * trimkv_build_cu_seqlens -- cu[0] = 0, cu[i+1] = cu[i] + seg_len[i] (int32), the offsets the

@@ -325,3 +325,43 @@ def test_decode_attention_dispatch_order_changes_nothing_but_scheduling():
     got = decode_attention(q, k, v, nseg, G, L, None, cap, cap, D ** -0.5, chunk=512, seg_order=wild)
     untouched = [s for s in range(1, nseg - 1) if s not in (int(order[0]), int(order[1]))]
     assert torch.equal(got.view(nseg, G, D)[untouched], base.view(nseg, G, D)[untouched])
+
+
+@pytest.mark.parametrize("nlayers,B,H,budget,threshold", [(3, 2, 4, 500, None), (40, 1, 8, 3000, None), (40, 1, 8, 10 ** 9, None),
+                                                          (5, 3, 2, 0, None), (6, 2, 4, 0, -0.7), (2, 1, 2, 77, None)])
+def test_wide_group_threshold_equals_the_single_workgroup_selection(nlayers, B, H, budget, threshold):
+    """trimkv_group_threshold_wide must return exactly what trimkv_group_threshold returns: cut key, tie quota, per-segment
+    kept counts and tie bases -- with heavy ties (log beta on a coarse grid), ragged and empty segments, more than 256
+    (layer, segment) pairs per group, budgets of zero and beyond the token count, and the threshold mode."""
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(nlayers * 100 + B)
+    nseg, cap, D = B * H, 96, 128
+    lens = rng.integers(0, cap + 1, size=(nlayers, nseg)).astype(np.int32)
+    lens[0, 0] = 0
+    lb = [torch.from_numpy(-(rng.integers(1, 6, size=(nseg, cap)) / 8.0).astype(np.float32)).to(DEV) for _ in range(nlayers)]
+    pos = [torch.from_numpy(np.tile(np.arange(cap, dtype=np.int64), (nseg, 1))).to(DEV) for _ in range(nlayers)]
+    ln = [torch.from_numpy(lens[l].copy()).to(DEV) for l in range(nlayers)]
+    table = lambda ts: torch.tensor([t.data_ptr() for t in ts], dtype=torch.int64, device=DEV)
+    lb_t, pos_t, len_t = table(lb), table(pos), table(ln)
+    st = L.current_stream(torch.device(DEV))
+
+    def run(wide):
+        thr = torch.zeros(B, dtype=torch.int32, device=DEV); take = torch.zeros(B, dtype=torch.int32, device=DEV)
+        tb = torch.full((nlayers, nseg), -1, dtype=torch.int32, device=DEV); nl = torch.full((nlayers, nseg), -1, dtype=torch.int32, device=DEV)
+        args = (lb_t.data_ptr(), pos_t.data_ptr(), None, len_t.data_ptr(), nlayers, nseg, H, cap, D, L.BF16, L.F32, budget,
+                0 if threshold is None else 1, 0.0 if threshold is None else threshold, cap + 5, 0, 1,
+                thr.data_ptr(), take.data_ptr(), tb.data_ptr(), nl.data_ptr())
+        if wide:
+            ws = torch.empty(lib.trimkv_group_threshold_workspace(nlayers, nseg, H), dtype=torch.uint8, device=DEV)
+            L.check(lib.trimkv_group_threshold_wide(*args, ws.data_ptr(), ws.numel(), st), "wide")
+        else:
+            L.check(lib.trimkv_group_threshold(*args, st), "single")
+        return [t.cpu() for t in (thr, take, tb, nl)]
+
+    for a, b in zip(run(False), run(True)):
+        assert torch.equal(a, b)
+    nl = run(True)[3].numpy()
+    if threshold is None:
+        want = np.minimum(budget, lens.reshape(nlayers, B, H).sum(axis=(0, 2)))
+        assert (nl.reshape(nlayers, B, H).sum(axis=(0, 2)) == want).all()      # every group keeps exactly its budget

@@ -235,6 +235,43 @@ class _SlabBacked(_CacheBase):
         slab.max_len += S
         return slab
 
+    # ---- several layers in one launch ----------------------------------------------------------
+    _LAYER_DT = np.dtype([("k", "<u8"), ("v", "<u8"), ("lb", "<u8"), ("pos", "<u8"), ("len", "<u8"),
+                          ("q", "<i8"), ("cap", "<i4"), ("res", "<i4")])   # struct trimkv_layer_slabs
+
+    def _layers_alike(self, layers: List[int]) -> bool:
+        s0 = self._slabs[layers[0]]
+        return all((s.nseg, s.D, s.k.dtype, s.lb.dtype, s.k.device) == (s0.nseg, s0.D, s0.k.dtype, s0.lb.dtype, s0.k.device)
+                   for s in (self._slabs[l] for l in layers))
+
+    def _layer_table(self, layers: List[int], q_idx) -> torch.Tensor:
+        """Device table of ``trimkv_layer_slabs`` for ``layers``; ``q_idx`` maps a layer to its tokens seen + 1."""
+        arr = np.zeros(len(layers), dtype=self._LAYER_DT)
+        for i, l in enumerate(layers):
+            s = self._slabs[l]
+            arr[i] = (s.ptrs[0], s.ptrs[1], s.ptrs[2], s.ptrs[3], s.ptrs[4], int(q_idx(l)), s.cap, 0)
+        return torch.from_numpy(arr.view(np.uint8)).to(self._slabs[layers[0]].k.device)
+
+    def _evict_layers(self, layers: List[int], keep: int, keep_per_seg: Optional[np.ndarray], slack: int, strategy_code: int,
+                      rounding: int, sliding_window: int, q_idx) -> None:
+        """``trimkv_evict_layers`` over ``layers`` (all of one shape): one launch of nseg x len(layers) workgroups."""
+        s0 = self._slabs[layers[0]]
+        dev = s0.k.device
+        max_len = max(self._slabs[l].max_len for l in layers)
+        table = self._layer_table(layers, q_idx)
+        kdev, stride = None, 0
+        if keep_per_seg is not None:
+            kp = np.ascontiguousarray(keep_per_seg, dtype=np.int32)
+            stride = 0 if kp.ndim == 1 else s0.nseg
+            kdev = torch.from_numpy(kp.reshape(-1)).to(dev)
+        lib = _lib.load()
+        ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
+        rc = lib.trimkv_evict_layers(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                     int(keep), _lib.ptr(kdev), stride, int(slack), strategy_code, rounding, int(sliding_window), max_len,
+                                     _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
+        _lib.check(rc, "trimkv_evict_layers")
+        self._keepalive_layers = (table, kdev)   # read asynchronously by the launch
+
     def _ensure_layer(self, layer: int) -> None:
         while len(self._slabs) <= layer:
             self._slabs.append(None)
@@ -369,23 +406,34 @@ class TrimKVCache(_SlabBacked):
         num_key_value_heads = heads if num_key_value_heads is None else num_key_value_heads
         assert num_key_value_heads == heads, "Key and value caches must have the same number of heads"
         self._budget_hint = memory_size + buffer_size
-        for layer_idx in range(skip_layers, num_layers):
-            if memory_size + buffer_size <= self.get_cache_length(layer_idx):
-                self.compress_layer(layer_idx, memory_size, strategy, self.sliding_window_size)
-                slab = self._slabs[layer_idx]
-                if slab.cap > 2 * self._budget_hint:  # a long prefill left a slab far larger than steady state needs
-                    slab.regrow(self._budget_hint)
+        todo = [l for l in range(skip_layers, num_layers) if memory_size + buffer_size <= self.get_cache_length(l)]
+        if len(todo) > 1 and self._layers_alike(todo):   # the usual case: every layer is due at the same step -> one launch
+            self._evict_layers(todo, memory_size, None, 0, self._dense_strategy_code(strategy), _lib.ROUND_UPCAST,
+                               self.sliding_window_size, lambda l: self.get_seq_length(l) + 1)
+            for l in todo:
+                self._slabs[l].lens[:] = memory_size
+                self._slabs[l].max_len = memory_size
+        else:
+            for l in todo:
+                self.compress_layer(l, memory_size, strategy, self.sliding_window_size)
+        for l in todo:
+            slab = self._slabs[l]
+            if slab.cap > 2 * self._budget_hint:  # a long prefill left a slab far larger than steady state needs
+                slab.regrow(self._budget_hint)
+
+    @staticmethod
+    def _dense_strategy_code(strategy: str) -> int:
+        if strategy == "alpha":
+            return _lib.SCORE_ALPHA
+        if strategy == "knorm_alpha":
+            return _lib.SCORE_KNORM_ALPHA
+        raise ValueError(f"Unknown compression strategy: {strategy}")
 
     def compress_layer(self, layer_idx: int, memory_size: int, comrpess_strategy: str = "alpha", sliding_window_size: int = 0,
                        return_indices: bool = False):
         """Keep, per (batch, head), the ``memory_size`` tokens with the largest
         ``fp32(log beta) * (seen + 1 - position)`` in temporal order (cache_utils.py:160-198)."""
-        if comrpess_strategy == "alpha":
-            strat = _lib.SCORE_ALPHA
-        elif comrpess_strategy == "knorm_alpha":
-            strat = _lib.SCORE_KNORM_ALPHA
-        else:
-            raise ValueError(f"Unknown compression strategy: {comrpess_strategy}")
+        strat = self._dense_strategy_code(comrpess_strategy)
         slab = self._slabs[layer_idx]
         n = slab.max_len
         if memory_size > n:
@@ -596,13 +644,18 @@ class _RaggedCache(_SlabBacked):
         k_t = self._ptr_table([s.k for s in slabs], dev)
         len_t = self._ptr_table([s.seg_len for s in slabs], dev)
         lib = _lib.load()
-        rc = lib.trimkv_group_threshold(lb_t.data_ptr(), pos_t.data_ptr(), k_t.data_ptr(), len_t.data_ptr(),
-                                        L, s0.nseg, segs_per_group, s0.cap, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
-                                        int(budget), 0 if threshold is None else 1, 0.0 if threshold is None else float(threshold),
-                                        self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE,
-                                        thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(),
-                                        _lib.current_stream(dev))
-        _lib.check(rc, "trimkv_group_threshold")
+        args = (lb_t.data_ptr(), pos_t.data_ptr(), k_t.data_ptr(), len_t.data_ptr(),
+                L, s0.nseg, segs_per_group, s0.cap, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                int(budget), 0 if threshold is None else 1, 0.0 if threshold is None else float(threshold),
+                self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE,
+                thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr())
+        if L * segs_per_group >= 16:   # a large group (a budget shared by all layers): one workgroup per (layer, segment)
+            ws = self._workspace(lib.trimkv_group_threshold_workspace(L, s0.nseg, segs_per_group), dev)
+            rc = lib.trimkv_group_threshold_wide(*args, ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
+            _lib.check(rc, "trimkv_group_threshold_wide")
+        else:
+            rc = lib.trimkv_group_threshold(*args, _lib.current_stream(dev))
+            _lib.check(rc, "trimkv_group_threshold")
         self._keepalive = (lb_t, pos_t, k_t, len_t)  # the launch reads these tables asynchronously
         return thr, take, tie_base, new_len
 
@@ -616,6 +669,27 @@ class _RaggedCache(_SlabBacked):
                                           self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE, slab.max_len,
                                           _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(slab.k.device))
         _lib.check(rc, "trimkv_compact_threshold")
+
+    def _compact_layers(self, layers: List[int], segs_per_group: int, thr, take, tie_base, strategy: str) -> None:
+        """One budget across ``layers``: every layer compacted against the same group thresholds, in one launch."""
+        if len(layers) == 1 or not self._layers_alike(layers):
+            for i, l in enumerate(layers):
+                self._compact(l, segs_per_group, thr, take, tie_base[i], strategy)
+            return
+        s0 = self._slabs[layers[0]]
+        dev = s0.k.device
+        max_len = max(self._slabs[l].max_len for l in layers)
+        q = self.get_seq_length() + 1
+        table = self._layer_table(layers, lambda l: q)
+        lib = _lib.load()
+        ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
+        rc = lib.trimkv_compact_threshold_layers(table.data_ptr(), len(layers), s0.nseg, segs_per_group, s0.D,
+                                                 _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                                 thr.data_ptr(), take.data_ptr(), 0, tie_base.data_ptr(),
+                                                 self._strategy_code(strategy), _lib.ROUND_NATIVE, max_len,
+                                                 _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
+        _lib.check(rc, "trimkv_compact_threshold_layers")
+        self._keepalive_layers = (table, None)
 
     def _evict_per_segment(self, layer: int, keep: np.ndarray, strategy: str) -> None:
         slab = self._slabs[layer]
@@ -768,8 +842,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             if "threshold" in strategy:
                 threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
             thr, take, tie_base, _ = self._group_select(layers, H, num_layers * H * memory_size, strategy, threshold)
-            for i, l in enumerate(layers):
-                self._compact(l, H, thr, take, tie_base[i], strategy)
+            self._compact_layers(layers, H, thr, take, tie_base, strategy)
             self._refresh(layers)
 
     def log(self):
@@ -823,8 +896,7 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             if "threshold" in strategy:
                 threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
             thr, take, tie_base, _ = self._group_select(layers, H, total_budget, strategy, threshold)
-            for i, l in enumerate(layers):
-                self._compact(l, H, thr, take, tie_base[i], strategy)
+            self._compact_layers(layers, H, thr, take, tie_base, strategy)
             self._refresh(layers)
             return
         assert "threshold" not in strategy, "Thresholding strategy is not compatible with floor_budget_ratio > 0"
@@ -842,8 +914,13 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
         credited -= moved
         credited[:-1] += moved[1:]
         head_cnt = credited + int(memory_size * floor_budget_ratio)
-        for i, l in enumerate(layers):
-            self._evict_per_segment(l, head_cnt[i * H:(i + 1) * H], strategy)  # k >= len keeps all (:514-516)
+        if len(layers) > 1 and self._layers_alike(layers):   # k >= len keeps all (:514-516)
+            q = self.get_seq_length() + 1
+            self._evict_layers(layers, 0, head_cnt.reshape(len(layers), H), 0, self._strategy_code(strategy), _lib.ROUND_NATIVE, 0,
+                               lambda l: q)
+        else:
+            for i, l in enumerate(layers):
+                self._evict_per_segment(l, head_cnt[i * H:(i + 1) * H], strategy)
         self._refresh(layers)
 
     def _first_token_selected(self, layers, thr, take, tie_base, strategy) -> np.ndarray:

@@ -244,7 +244,23 @@ struct EvictArgs {
     uint32_t* ws_keys; int ws_stride;  // used when the keys do not fit in LDS
     // threshold mode (trimkv_compact_threshold)
     const uint32_t* thr_key; const int32_t* tie_take; const int32_t* tie_base; int segs_per_group;
+    // several layers in one launch (blockIdx.y = layer): per-layer slabs come from this device table
+    const trimkv_layer_slabs* layers; int keep_layer_stride, thr_layer_stride;
 };
+
+// blockIdx.y selects a layer: its slab addresses, capacity and query index replace the scalar fields, and the
+// per-layer parts of the other arrays are stepped to.
+__device__ __forceinline__ void select_layer(EvictArgs& a) {
+    if (!a.layers) return;
+    const int layer = blockIdx.y;
+    const trimkv_layer_slabs L = a.layers[layer];
+    a.k_slab = (char*)L.k_slab; a.v_slab = (char*)L.v_slab; a.lb_slab = (char*)L.lb_slab; a.pos_slab = L.pos_slab; a.seg_len = L.seg_len;
+    a.q_idx = L.q_idx; a.cap = L.cap;
+    if (a.keep_per_seg) a.keep_per_seg += (int64_t)layer * a.keep_layer_stride;
+    if (a.tie_base) a.tie_base += (int64_t)layer * a.nseg;
+    if (a.thr_key) { a.thr_key += (int64_t)layer * a.thr_layer_stride; a.tie_take += (int64_t)layer * a.thr_layer_stride; }
+    if (a.ws_keys) a.ws_keys += (int64_t)layer * a.nseg * a.ws_stride;
+}
 
 // SELECT = true: find the cut inside the segment (trimkv_evict).
 // SELECT = false: the cut comes from thr_key/tie_take/tie_base (trimkv_compact_threshold).
@@ -255,6 +271,7 @@ __global__ __launch_bounds__(EV_THREADS) void evict_kernel(EvictArgs a) {
     __shared__ uint32_t scratch[EV_THREADS / 64 + 4];
     __shared__ int first_evicted;
 
+    select_layer(a);
     const int seg = blockIdx.x;
     const int n = a.seg_len[seg];
     if (n <= 0 || n > a.cap) return;  // nothing cached, or a corrupt length: touch nothing
@@ -415,6 +432,182 @@ __global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a
     }
 }
 
+// ---- the same selection spread over many workgroups (large groups: one sequence over all layers, ...) -----------
+// One workgroup per (layer, segment).  Four histogram launches (one per key byte, most significant first) add into a
+// per-group global histogram; every workgroup re-derives the digits chosen so far from the earlier histograms (a
+// 256-bin walk, cheap) before it bins its own segment.  A count launch then classifies every segment's tokens against
+// the cut, and a scan launch (one workgroup per group) turns the per-segment counts into new_len / tie_base in
+// (layer, segment) order.  Kernel boundaries are the only synchronisation.
+constexpr int GW_THREADS = 256;
+struct WideArgs {
+    GroupArgs g;
+    uint32_t* hist;   // [ngroups][4][256]
+    uint32_t* cnt;    // [nlayers][nseg][2]: tokens above the cut, tokens equal to it
+};
+
+// digit and remaining rank chosen in a pass, from that pass's 256-bin histogram (in LDS), largest bin first
+__device__ __forceinline__ void walk_bins(const uint32_t* h, uint64_t remaining, uint32_t& digit, uint64_t& left) {
+    uint64_t acc = 0;
+    int b = 255;
+    for (; b > 0; --b) {
+        if (acc + h[b] >= remaining) break;
+        acc += h[b];
+    }
+    digit = (uint32_t)b;
+    left = remaining - acc;
+}
+
+// prefix (digits of passes 0..npass-1) and remaining rank for group g; *total = tokens in the group.  All threads call.
+__device__ __forceinline__ void wide_prefix(const WideArgs& w, int g, int npass, uint32_t* lh, uint32_t* sh_digit,
+                                            unsigned long long* sh_left, uint32_t& prefix, uint64_t& remaining, uint64_t& total) {
+    prefix = 0;
+    remaining = (uint64_t)max((int64_t)0, w.g.budget);
+    total = 0;
+    for (int q = 0; q < npass; ++q) {
+        __syncthreads();
+        lh[threadIdx.x] = w.hist[((int64_t)g * 4 + q) * 256 + threadIdx.x];
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            if (q == 0) {
+                uint64_t t = 0;
+                for (int b = 0; b < 256; ++b) t += lh[b];
+                sh_left[1] = t;
+            }
+            uint32_t d;
+            uint64_t left;
+            walk_bins(lh, remaining, d, left);
+            *sh_digit = d;
+            sh_left[0] = left;
+        }
+        __syncthreads();
+        prefix |= *sh_digit << (24 - 8 * q);
+        remaining = sh_left[0];
+        if (q == 0) total = sh_left[1];
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(GW_THREADS) void group_hist_kernel(WideArgs w, int pass) {
+    __shared__ uint32_t lh[256];
+    __shared__ uint32_t sh_digit;
+    __shared__ unsigned long long sh_left[2];
+    const GroupArgs& a = w.g;
+    const int s = blockIdx.x, l = blockIdx.y, g = blockIdx.z;
+    const int seg = g * a.segs_per_group + s;
+    uint32_t prefix;
+    uint64_t remaining, total;
+    wide_prefix(w, g, pass, lh, &sh_digit, sh_left, prefix, remaining, total);
+    const int shift = 24 - 8 * pass;
+    const uint32_t hi_mask = pass == 0 ? 0u : (0xffffffffu << (shift + 8));
+    lh[threadIdx.x] = 0;
+    __syncthreads();
+    const int n = max(0, min(a.seg_lens[l][seg], a.cap));
+    const ScoreArgs sa = group_segment(a, l, seg);
+    for (int i = threadIdx.x; i < n; i += GW_THREADS) {
+        const uint32_t key = score_key(sa, i, n);
+        if ((key & hi_mask) == prefix) atomicAdd(&lh[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (lh[threadIdx.x]) atomicAdd(&w.hist[((int64_t)g * 4 + pass) * 256 + threadIdx.x], lh[threadIdx.x]);
+}
+
+// cut of group g: from the threshold, or from the four histograms (with the keep-all / keep-nothing cases)
+__device__ __forceinline__ void wide_cut(const WideArgs& w, int g, uint32_t* lh, uint32_t* sh_digit, unsigned long long* sh_left,
+                                         uint32_t& thr, int64_t& take) {
+    const GroupArgs& a = w.g;
+    if (a.use_threshold) {
+        thr = float_key(a.threshold_score);
+        take = INT32_MAX;
+        return;
+    }
+    uint32_t prefix;
+    uint64_t remaining, total;
+    wide_prefix(w, g, 4, lh, sh_digit, sh_left, prefix, remaining, total);
+    const uint64_t budget = (uint64_t)max((int64_t)0, a.budget);
+    if (budget >= total) { thr = 0u; take = INT32_MAX; }
+    else if (budget == 0) { thr = 0xffffffffu; take = 0; }
+    else { thr = prefix; take = (int64_t)remaining; }
+}
+
+__global__ __launch_bounds__(GW_THREADS) void group_count_kernel(WideArgs w) {
+    __shared__ uint32_t lh[256];
+    __shared__ uint32_t sh_digit;
+    __shared__ unsigned long long sh_left[2];
+    __shared__ uint64_t red[GW_THREADS / 64];
+    const GroupArgs& a = w.g;
+    const int s = blockIdx.x, l = blockIdx.y, g = blockIdx.z;
+    const int seg = g * a.segs_per_group + s;
+    uint32_t thr;
+    int64_t take;
+    wide_cut(w, g, lh, &sh_digit, sh_left, thr, take);
+    const int n = max(0, min(a.seg_lens[l][seg], a.cap));
+    const ScoreArgs sa = group_segment(a, l, seg);
+    uint64_t cnt = 0;  // low 32 bits: greater, high 32 bits: equal
+    for (int i = threadIdx.x; i < n; i += GW_THREADS) {
+        const uint32_t key = score_key(sa, i, n);
+        cnt += (key > thr ? 1ull : 0ull) + (key == thr ? (1ull << 32) : 0ull);
+    }
+    for (int d = 32; d > 0; d >>= 1) cnt += __shfl_down(cnt, d, 64);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = cnt;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint64_t t = 0;
+        for (int i = 0; i < GW_THREADS / 64; ++i) t += red[i];
+        const int64_t e = ((int64_t)l * a.nseg + seg) * 2;
+        w.cnt[e] = (uint32_t)(t & 0xffffffffull);
+        w.cnt[e + 1] = (uint32_t)(t >> 32);
+        if (s == 0 && l == 0) {
+            a.thr_key[g] = thr;
+            a.tie_take[g] = (int32_t)min(take, (int64_t)INT32_MAX);
+        }
+    }
+}
+
+__global__ __launch_bounds__(GW_THREADS) void group_scan_kernel(WideArgs w) {
+    __shared__ uint32_t gt_l[GW_THREADS], eq_l[GW_THREADS];
+    __shared__ int32_t len_l[GW_THREADS], base_l[GW_THREADS];
+    __shared__ long long carry;
+    const GroupArgs& a = w.g;
+    const int g = blockIdx.x;
+    const int64_t take = a.tie_take[g];   // written by the count launch
+    const int entries = a.nlayers * a.segs_per_group;   // (layer, segment) pairs of the group, in tie order
+    if (threadIdx.x == 0) carry = 0;
+    for (int e0 = 0; e0 < entries; e0 += GW_THREADS) {
+        __syncthreads();
+        const int e = e0 + threadIdx.x;
+        int64_t idx = 0;
+        if (e < entries) {
+            const int l = e / a.segs_per_group, s = e - l * a.segs_per_group;
+            idx = (int64_t)l * a.nseg + g * a.segs_per_group + s;
+            gt_l[threadIdx.x] = w.cnt[idx * 2];
+            eq_l[threadIdx.x] = w.cnt[idx * 2 + 1];
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            long long eq_seen = carry;
+            const int m = min(GW_THREADS, entries - e0);
+            for (int i = 0; i < m; ++i) {
+                const long long eq = eq_l[i];
+                const long long eq_kept = max(0ll, min(eq, (long long)take - eq_seen));
+                len_l[i] = (int32_t)((long long)gt_l[i] + eq_kept);
+                base_l[i] = (int32_t)min(eq_seen, (long long)INT32_MAX);
+                eq_seen += eq;
+            }
+            carry = eq_seen;
+        }
+        __syncthreads();
+        if (e < entries) {
+            a.new_len[idx] = len_l[threadIdx.x];
+            a.tie_base[idx] = base_l[threadIdx.x];
+        }
+    }
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = v;
+}
+
 __global__ void cu_seqlens_kernel(const int32_t* seg_len, int nseg, int32_t* cu) {
     __shared__ uint32_t scratch[1024 / 64 + 1];
     int32_t running = 0;
@@ -438,7 +631,7 @@ static int lpr_shift_of(int row_bytes) {
 }
 
 template <bool SELECT>
-static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st) {
+static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st, int nlayers = 1) {
     const size_t key_bytes = (size_t)max_len * 4;
     if (key_bytes <= (size_t)EV_LDS_KEY_BYTES) {
         static bool attr_set = false;
@@ -447,14 +640,14 @@ static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspa
             if (e != hipSuccess) return fail((int)e, "%s: hipFuncSetAttribute: %s", fn, hipGetErrorString(e));
             attr_set = true;
         }
-        hipLaunchKernelGGL((evict_kernel<true, SELECT>), dim3(a.nseg), dim3(EV_THREADS), key_bytes, st, a);
+        hipLaunchKernelGGL((evict_kernel<true, SELECT>), dim3(a.nseg, nlayers), dim3(EV_THREADS), key_bytes, st, a);
     } else {
-        const size_t need = (size_t)a.nseg * max_len * 4;
+        const size_t need = (size_t)nlayers * a.nseg * max_len * 4;
         if (!workspace || workspace_bytes < need)
             return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed for max_len=%d, got %zu", fn, need, max_len, workspace_bytes);
         a.ws_keys = (uint32_t*)workspace;
         a.ws_stride = max_len;
-        hipLaunchKernelGGL((evict_kernel<false, SELECT>), dim3(a.nseg), dim3(EV_THREADS), 0, st, a);
+        hipLaunchKernelGGL((evict_kernel<false, SELECT>), dim3(a.nseg, nlayers), dim3(EV_THREADS), 0, st, a);
     }
     return launch_status(fn);
 }
@@ -525,6 +718,62 @@ extern "C" int trimkv_compact_threshold(void* k_slab, void* v_slab, void* lb_sla
     return launch_evict<false>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
+static int check_layer_args(const char* fn, const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype,
+                            int lb_dtype, int max_len, int* lpr_shift) {
+    if (!layers) return fail(TRIMKV_ERR_NULL, "%s: null layer table", fn);
+    if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0)
+        return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
+    if (nlayers <= 0 || nlayers > 65535 || nseg <= 0 || head_dim <= 0 || max_len <= 0)
+        return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d head_dim=%d max_len=%d", fn, nlayers, nseg, head_dim, max_len);
+    *lpr_shift = lpr_shift_of(head_dim * 2);
+    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be 16 * a power of two <= 1024 (head_dim=%d)", fn, head_dim);
+    return TRIMKV_OK;
+}
+
+extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                                   int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                                   int strategy, int rounding, int sliding_window, int max_len,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_evict_layers";
+    int lpr_shift;
+    int rc = check_layer_args(fn, layers, nlayers, nseg, head_dim, kv_dtype, lb_dtype, max_len, &lpr_shift);
+    if (rc) return rc;
+    if (!keep_per_seg && keep < 0) return fail(TRIMKV_ERR_SHAPE, "%s: keep=%d", fn, keep);
+    if (keep_per_seg && keep_layer_stride != 0 && keep_layer_stride != nseg)
+        return fail(TRIMKV_ERR_SHAPE, "%s: keep_layer_stride must be 0 or nseg (got %d)", fn, keep_layer_stride);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    if (rounding != TRIMKV_ROUND_UPCAST && rounding != TRIMKV_ROUND_NATIVE) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown rounding %d", fn, rounding);
+    EvictArgs a = {};
+    a.layers = layers; a.keep_layer_stride = keep_layer_stride;
+    a.nseg = nseg; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
+    a.keep = keep; a.keep_per_seg = keep_per_seg; a.slack = slack < 0 ? 0 : slack;
+    a.strategy = strategy; a.rounding = rounding; a.sliding_window = sliding_window < 0 ? 0 : sliding_window;
+    a.segs_per_group = 1;
+    return launch_evict<true>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream, nlayers);
+}
+
+extern "C" int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int segs_per_group, int head_dim,
+                                               int kv_dtype, int lb_dtype,
+                                               const uint32_t* thr_key, const int32_t* tie_take, int thr_layer_stride,
+                                               const int32_t* tie_base, int strategy, int rounding, int max_len,
+                                               void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_compact_threshold_layers";
+    int lpr_shift;
+    int rc = check_layer_args(fn, layers, nlayers, nseg, head_dim, kv_dtype, lb_dtype, max_len, &lpr_shift);
+    if (rc) return rc;
+    if (!thr_key || !tie_take || !tie_base) return fail(TRIMKV_ERR_NULL, "%s: null threshold pointer", fn);
+    if (segs_per_group <= 0 || nseg % segs_per_group) return fail(TRIMKV_ERR_SHAPE, "%s: segs_per_group=%d does not divide nseg=%d", fn, segs_per_group, nseg);
+    if (thr_layer_stride != 0 && thr_layer_stride != nseg / segs_per_group)
+        return fail(TRIMKV_ERR_SHAPE, "%s: thr_layer_stride must be 0 or nseg/segs_per_group (got %d)", fn, thr_layer_stride);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    EvictArgs a = {};
+    a.layers = layers; a.thr_layer_stride = thr_layer_stride;
+    a.nseg = nseg; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
+    a.strategy = strategy; a.rounding = rounding; a.sliding_window = 0;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.segs_per_group = segs_per_group;
+    return launch_evict<false>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream, nlayers);
+}
+
 extern "C" int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
                                       const void* const* k_slabs, const int32_t* const* seg_lens,
                                       int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
@@ -546,6 +795,51 @@ extern "C" int trimkv_group_threshold(const void* const* lb_slabs, const int64_t
     a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
     a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len;
     hipLaunchKernelGGL(group_threshold_kernel, dim3(nseg / segs_per_group), dim3(GT_THREADS), 0, (hipStream_t)stream, a);
+    return launch_status(fn);
+}
+
+extern "C" size_t trimkv_group_threshold_workspace(int nlayers, int nseg, int segs_per_group) {
+    if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0) return 0;
+    return ((size_t)(nseg / segs_per_group) * 4 * 256 + (size_t)nlayers * nseg * 2) * sizeof(uint32_t);
+}
+
+extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+                                           const void* const* k_slabs, const int32_t* const* seg_lens,
+                                           int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
+                                           int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
+                                           int64_t q_idx, int strategy, int rounding,
+                                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                           void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_group_threshold_wide";
+    if (!lb_slabs || !pos_slabs || !seg_lens || !thr_key || !tie_take || !tie_base || !new_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if (strategy == TRIMKV_SCORE_KNORM_ALPHA && !k_slabs) return fail(TRIMKV_ERR_NULL, "%s: knorm_alpha needs k_slabs", fn);
+    if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
+    if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0) return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
+    if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0 || nseg % segs_per_group || cap <= 0 || head_dim <= 0)
+        return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d segs_per_group=%d cap=%d head_dim=%d", fn, nlayers, nseg, segs_per_group, cap, head_dim);
+    const int ngroups = nseg / segs_per_group;
+    if (nlayers > 65535 || ngroups > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nlayers=%d or groups=%d exceeds the grid limit 65535", fn, nlayers, ngroups);
+    const size_t need = trimkv_group_threshold_workspace(nlayers, nseg, segs_per_group);
+    if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+    if ((uintptr_t)workspace & 3) return fail(TRIMKV_ERR_SHAPE, "%s: workspace must be 4-byte aligned", fn);
+    WideArgs w;
+    GroupArgs& a = w.g;
+    a.lb_slabs = lb_slabs; a.pos_slabs = pos_slabs; a.k_slabs = strategy == TRIMKV_SCORE_KNORM_ALPHA ? k_slabs : nullptr; a.seg_lens = seg_lens;
+    a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
+    a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
+    a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len;
+    w.hist = (uint32_t*)workspace;
+    w.cnt = w.hist + (size_t)ngroups * 4 * 256;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid(segs_per_group, nlayers, ngroups);
+    if (!use_threshold) {
+        const int64_t nh = (int64_t)ngroups * 4 * 256;
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((nh + 255) / 256)), dim3(256), 0, st, w.hist, nh, 0u);
+        for (int pass = 0; pass < 4; ++pass) hipLaunchKernelGGL(group_hist_kernel, grid, dim3(GW_THREADS), 0, st, w, pass);
+    }
+    hipLaunchKernelGGL(group_count_kernel, grid, dim3(GW_THREADS), 0, st, w);
+    hipLaunchKernelGGL(group_scan_kernel, dim3(ngroups), dim3(GW_THREADS), 0, st, w);
     return launch_status(fn);
 }
 
