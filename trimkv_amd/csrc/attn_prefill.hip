@@ -429,35 +429,43 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     auto step = [&](pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
                     __attribute__((always_inline)) {
         constexpr bool HAS_NEXT = decltype(has_next)::value;
-        pf_bf16x8 kf[8], vf[8];
+        // The 16 MFMA operands of a step (8 K fragments, then 8 V fragments) are one stream of LDS reads, each requested
+        // PD MFMAs before the one that consumes it: no burst of reads at the start of a step, a few registers in flight.
+        constexpr int PD = 3;
+        pf_bf16x8 frag[16];
         uint32_t pw[8];
+        auto request = [&](int m) __attribute__((always_inline)) {
+            if (m < 8) {
+                if (HAS_NEXT) frag[m] = *(const pf_bf16x8*)(kbuf + k_off + kkb * 32 * PF2_KROW + m * 32);
+            } else if (m < 16) {
+                frag[m] = v_frag(vbuf, vkb, (m - 8) >> 2, (m - 8) & 3);
+            }
+        };
         if (HAS_NEXT) {
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) kf[ks] = *(const pf_bf16x8*)(kbuf + k_off + kkb * 32 * PF2_KROW + ks * 32);
 #pragma unroll
             for (int v = 0; v < 16; ++v) s_nxt[v] = 0.0f;
         }
+#pragma unroll
+        for (int m = 0; m < PD; ++m) request(m);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
+            request(ks + PD);
             pw[ks] = p_pair(s_cur, ks);
-            if (ks == 2) {
-#pragma unroll
-                for (int db = 0; db < 4; ++db) vf[db] = v_frag(vbuf, vkb, 0, db);
-            }
-            if (ks == 5) {
-#pragma unroll
-                for (int db = 0; db < 4; ++db) vf[4 + db] = v_frag(vbuf, vkb, 1, db);
-            }
-            if (HAS_NEXT) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks], qf[ks], s_nxt, 0, 0, 0);
+            if (HAS_NEXT) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[ks], qf[ks], s_nxt, 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
+        pf_bf16x8 pfrag[2];
 #pragma unroll
         for (int st = 0; st < 2; ++st) {
             const pf_u32x4 pq = {pw[4 * st], pw[4 * st + 1], pw[4 * st + 2], pw[4 * st + 3]};
-            const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pq);
+            pfrag[st] = __builtin_bit_cast(pf_bf16x8, pq);
+        }
 #pragma unroll
-            for (int db = 0; db < 4; ++db) o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[4 * st + db], pfrag, o[db], 0, 0, 0);
+        for (int i = 0; i < 8; ++i) {
+            request(8 + i + PD);
+            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[8 + i], pfrag[i >> 2], o[i & 3], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
