@@ -101,6 +101,18 @@ int trimkv_gate_hidden(const void* x, const void* w1, const void* b1, const void
                        int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
 
 /*
+ * trimkv_gate_hidden_swiglu -- the same first half for the SwiGLU gate `rg3`
+ * (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:227-267, forward :256-264):
+ *     part[j][t][h] = sum over slice j of  w_down[h][u] * ( silu(w_gate[u][:] . x[t][:]) * (w_up[u][:] . x[t][:]) )
+ * x [ntok][hidden] is the reference's concat(K, V) after RoPE, laid out [B, S, Hkv*2*D]; w_gate
+ * and w_up [inter][hidden], w_down [kv_heads][inter], no first-layer bias.  Output layout, slice
+ * count and the fused second half are those of trimkv_gate_hidden.  The gate `rg2` (:182-224) has
+ * the arithmetic of `rg` on that same x and runs on trimkv_gate_hidden with hidden = Hkv*2*D.
+ */
+int trimkv_gate_hidden_swiglu(const void* x, const void* w_gate, const void* w_up, const void* w_down, float* part,
+                              int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
+
+/*
  * trimkv_append_gated -- trimkv_append whose log(beta) is produced inside the append kernel:
  *     lb[b][h][s] = logsigmoid( sum_j part[j][b*s_new + s][h] + gate_bias[h] )
  * rounded to lb_dtype (modeling_trimkv_qwen3.py:177-179, then the transpose at :333).

@@ -10,6 +10,8 @@
   ignored there), bottom-right causal mask when ``Q_LEN > 1`` (``causal=True`` at :144),
   output ``[B, Q_LEN, Hq, D]`` (:147-149).  Computed in fp32.
 * ``retention_gate_rg`` ...... ``src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:171-179``.
+* ``retention_gate_rg2`` ..... the same network on concat(K, V) after RoPE (:213-224, called at :345-347).
+* ``retention_gate_rg3`` ..... the SwiGLU variant (:256-267).
 
 Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
 may import this module.
@@ -79,3 +81,21 @@ def retention_gate_rg(x: torch.Tensor, w1: torch.Tensor, b1: torch.Tensor, w2: t
     """
     h = F.silu(F.linear(x, w1, b1))
     return F.logsigmoid(F.linear(h, w2) + bias)
+
+
+def kv_gate_input(key: torch.Tensor, value: torch.Tensor) -> torch.Tensor:
+    """K, V [B, Hkv, S, D] after RoPE -> the gate input [B, S, Hkv*2*D]: per head K then V, heads side by side
+    (``torch.cat([k, v], dim=-1)`` at qwen3 modeling file :346, then transpose(1, 2) and reshape at :215-216)."""
+    kv = torch.cat([key, value], dim=-1)
+    return kv.transpose(1, 2).reshape(kv.shape[0], kv.shape[2], -1)
+
+
+def retention_gate_rg2(key, value, w1, b1, w2, bias) -> torch.Tensor:
+    """log beta [B,S,Hkv] of ``RetentionGate2``: the `rg` network with ``w1`` [I, Hkv*2*D] on ``kv_gate_input`` (:213-224)."""
+    return retention_gate_rg(kv_gate_input(key, value), w1, b1, w2, bias)
+
+
+def retention_gate_rg3(key, value, w_gate, w_up, w_down, bias) -> torch.Tensor:
+    """log beta [B,S,Hkv] of ``RetentionGate3``: logsigmoid(Wdown (silu(Wgate x) * (Wup x)) + bias), no other bias (:256-267)."""
+    x = kv_gate_input(key, value)
+    return F.logsigmoid(F.linear(F.silu(F.linear(x, w_gate)) * F.linear(x, w_up), w_down) + bias)

@@ -78,6 +78,8 @@ def test_bad_arguments_are_refused_without_a_launch():
     assert lib.trimkv_gate_slices(512) == 32 and lib.trimkv_gate_slices(100) == 0
     assert lib.trimkv_gate_hidden(one, one, one, one, one, 8, 4096, 512, 8, _lib.F32, None) == -3
     assert lib.trimkv_gate_hidden(one, one, one, one, one, 8, 4224, 512, 8, _lib.BF16, None) == -6
+    assert lib.trimkv_gate_hidden_swiglu(one, one, None, one, one, 8, 2048, 512, 8, _lib.BF16, None) == -1   # no up_proj
+    assert lib.trimkv_gate_hidden_swiglu(one, one, one, one, one, 8, 2048, 500, 8, _lib.BF16, None) == -6
     # group selection
     assert lib.trimkv_group_threshold(one, one, None, one, 1, 8, 3, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 0, 1,
                                       one, one, one, one, None) == -2  # 3 does not divide 8

@@ -5,7 +5,7 @@ in a different summation order than torch's bf16 GEMM, so log beta is compared w
 import pytest
 import torch
 
-from oracle.attn_ref import retention_gate_rg
+from oracle.attn_ref import retention_gate_rg, retention_gate_rg2, retention_gate_rg3
 from tests.gpu_util import DEV, draw_kv
 
 pytestmark = pytest.mark.gpu
@@ -57,3 +57,38 @@ def test_append_gated_writes_the_same_log_beta_as_materialize():
     assert torch.equal(cache_a.retention_weights[0], cache_b.retention_weights[0])
     assert torch.equal(cache_a.key_cache[0], cache_b.key_cache[0]) and torch.equal(cache_a.kv_positions[0], cache_b.kv_positions[0])
     assert cache_a.get_cache_length(0) == 7
+
+
+@pytest.mark.parametrize("kind", ["rg2", "rg3"])
+@pytest.mark.parametrize("B,S,H", [(64, 1, 8), (2, 70, 4), (1, 300, 8)])
+def test_kv_gates_match_oracle(kind, B, S, H):
+    """rg2 / rg3 read concat(K, V) after RoPE; fused path against the fp32 oracle and the bf16 torch expression."""
+    from trimkv_amd import LazyLogBeta
+    from trimkv_amd.gate import RetentionGate2, RetentionGate3
+    torch.manual_seed(7)
+    D, inter = 128, 256
+    g = (RetentionGate2 if kind == "rg2" else RetentionGate3)(D, H, inter, bias_init=2.0, initializer_range=0.05)
+    if kind == "rg2":
+        g.linear1.bias.data.normal_(0, 0.1)
+    g = g.to(torch.bfloat16).eval()
+    k = torch.randn(B, H, S, D).to(torch.bfloat16)
+    v = torch.randn(B, H, S, D).to(torch.bfloat16)
+    if kind == "rg2":
+        w = (g.linear1.weight.data, g.linear1.bias.data, g.linear2.weight.data, g.bias.data)
+        oracle = retention_gate_rg2
+    else:
+        w = (g.gate_proj.weight.data, g.up_proj.weight.data, g.down_proj.weight.data, g.bias.data)
+        oracle = retention_gate_rg3
+    want32 = oracle(k.float(), v.float(), *[t.float() for t in w])
+    want16 = oracle(k, v, *w).float()
+    kv = torch.cat([k, v], dim=-1)
+    assert torch.equal(g(kv), oracle(k, v, *w))                     # CPU / non-fused path = torch expression
+    lazy = g.to(DEV)(kv.to(DEV))
+    assert isinstance(lazy, LazyLogBeta) and lazy.shape == (B, S, H)
+    got = lazy.materialize().float().cpu()
+    assert (got <= 0).all()
+    tol = 3e-2 * want32.abs() + 2e-3
+    assert ((got - want32).abs() <= tol).all(), float((got - want32).abs().max())
+    assert (got - want16).abs().mean() <= (want16 - want32).abs().mean() * 2 + 1e-4
+    # [B, S, Hkv, 2D] input with transpose=False is the same thing
+    assert torch.equal(g(kv.to(DEV).transpose(1, 2).contiguous(), transpose=False).materialize().cpu(), lazy.materialize().cpu())

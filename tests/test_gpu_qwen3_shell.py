@@ -72,12 +72,13 @@ def _record_updates(cache, nlayers):
     return rec
 
 
-def test_shell_logits_match_fp32_replay_of_retained_positions():
+@pytest.mark.parametrize("gate", ["rg", "rg2", "rg3"])
+def test_shell_logits_match_fp32_replay_of_retained_positions(gate):
     from trimkv_amd import TrimKVCache, LazyLogBeta
     from trimkv_amd.qwen3 import TrimKVQwen3ForCausalLM
     from trimkv_amd import attn as attn_registry
     torch.manual_seed(0)
-    cfg = _tiny_config()
+    cfg = _tiny_config(retention_gate=gate)
     model = TrimKVQwen3ForCausalLM(cfg).to(torch.bfloat16).eval()
     ref = copy.deepcopy(model).float()
     ref.config = copy.copy(cfg)

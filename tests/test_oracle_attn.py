@@ -2,7 +2,8 @@
 import numpy as np
 import torch
 
-from oracle.attn_ref import eager_attention, ragged_attention, repeat_kv, retention_gate_rg
+from oracle.attn_ref import (eager_attention, kv_gate_input, ragged_attention, repeat_kv, retention_gate_rg, retention_gate_rg2,
+                             retention_gate_rg3)
 
 
 def _softmax64(x):
@@ -97,3 +98,39 @@ def test_retention_gate_matches_float64():
     z = h @ w2.T + bias
     want = np.minimum(z, 0) - np.log1p(np.exp(-np.abs(z)))
     assert got.shape == (B, S, H) and np.allclose(got, want, atol=1e-5) and (got <= 0).all()
+
+
+def test_kv_gates_match_float64_loops():
+    """rg2 / rg3 against per-element float64 loops that index K and V directly: a swapped K/V half, head-major versus
+    token-major flattening, a missing product or a stray first-layer bias all change the result."""
+    rng = np.random.default_rng(5)
+    B, H, S, D, inter = 2, 3, 4, 4, 6
+    k = rng.standard_normal((B, H, S, D)); v = rng.standard_normal((B, H, S, D))
+    w1 = rng.standard_normal((inter, H * 2 * D)) * 0.3; b1 = rng.standard_normal(inter) * 0.2
+    wu = rng.standard_normal((inter, H * 2 * D)) * 0.3
+    w2 = rng.standard_normal((H, inter)) * 0.5; bias = rng.standard_normal(H)
+    t = lambda a: torch.tensor(a, dtype=torch.float32)
+    x = kv_gate_input(t(k), t(v)).numpy()
+    assert x.shape == (B, S, H * 2 * D)
+    silu = lambda z: z / (1 + np.exp(-z))
+    logsig = lambda z: min(z, 0.0) - np.log1p(np.exp(-abs(z)))
+    want2, want3 = np.zeros((B, S, H)), np.zeros((B, S, H))
+    for b in range(B):
+        for s_ in range(S):
+            pre, up = b1.copy(), np.zeros(inter)
+            pre3 = np.zeros(inter)
+            for h in range(H):
+                for d in range(D):
+                    for src, off in ((k, 0), (v, D)):            # column of head h: K in [0, D), V in [D, 2D)
+                        col = h * 2 * D + off + d
+                        assert x[b, s_, col] == np.float32(src[b, h, s_, d])
+                        pre += w1[:, col] * src[b, h, s_, d]
+                        pre3 += w1[:, col] * src[b, h, s_, d]
+                        up += wu[:, col] * src[b, h, s_, d]
+            for h in range(H):
+                want2[b, s_, h] = logsig(float(w2[h] @ silu(pre) + bias[h]))
+                want3[b, s_, h] = logsig(float(w2[h] @ (silu(pre3) * up) + bias[h]))
+    got2 = retention_gate_rg2(t(k), t(v), t(w1), t(b1), t(w2), t(bias)).numpy()
+    got3 = retention_gate_rg3(t(k), t(v), t(w1), t(wu), t(w2), t(bias)).numpy()
+    assert np.allclose(got2, want2, atol=1e-5) and np.allclose(got3, want3, atol=1e-5)
+    assert not np.allclose(got2, got3, atol=1e-3)

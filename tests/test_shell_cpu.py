@@ -25,6 +25,19 @@ def test_parameter_names_follow_the_reference():
     assert keys == want
 
 
+def test_kv_gate_parameter_names_and_shapes():
+    """rg2 / rg3 (modeling_trimkv_qwen3.py:190-200, 235-245): first layer reads Hkv*2*D inputs; rg3 has no biased layer."""
+    import dataclasses
+    for kind, names in (("rg2", {"linear1.weight": (32, 512), "linear1.bias": (32,), "linear2.weight": (2, 32), "bias": (2,)}),
+                        ("rg3", {"gate_proj.weight": (32, 512), "up_proj.weight": (32, 512), "down_proj.weight": (2, 32), "bias": (2,)})):
+        m = TrimKVQwen3ForCausalLM(dataclasses.replace(_tiny(), retention_gate=kind))
+        g = m.model.layers[1].self_attn.retention_gate
+        assert {k: tuple(v.shape) for k, v in g.state_dict().items()} == names
+        assert torch.all(g.bias == 10.0)
+    with pytest.raises(NotImplementedError):
+        TrimKVQwen3ForCausalLM(dataclasses.replace(_tiny(), retention_gate="rg9"))
+
+
 def test_gate_init_matches_reference_reset():
     m = TrimKVQwen3ForCausalLM(_tiny())
     g = m.model.layers[0].self_attn.retention_gate

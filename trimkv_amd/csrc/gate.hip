@@ -9,6 +9,9 @@
 // operand layout: lane l holds 8 consecutive k of row l%16 at k-group l/16); the parts are
 // summed in LDS, then bias, SiLU and the 16-unit contraction with W2 finish on the VALU.
 // Intermediate values are rounded to bf16 where a bf16 torch module rounds them.
+//
+// The SwiGLU gate `rg3` (:227-267) is the same kernel with two first-layer products per unit:
+// part[j][t][h] = sum_u Wdown[h][u] * (silu(Wgate[u].x[t]) * (Wup[u].x[t])), no first-layer bias.
 #include "common.hip.h"
 
 namespace trimkv {
@@ -23,6 +26,7 @@ constexpr int GH_MAX_HEADS = 32;
 
 struct GateArgs {
     const uint16_t* x; const uint16_t* w1; const uint16_t* b1; const uint16_t* w2; float* part;
+    const uint16_t* w_up;   // SwiGLU only: the second first-layer matrix
     int ntok, hidden, inter, kv_heads;
 };
 
@@ -30,10 +34,10 @@ struct GateArgs {
 //   TT = 1, KS = 16: decode (a handful of tokens): many small workgroups and short dependent chains;
 //   TT = 4, KS = 4 : prompts: a W1 slice is reused by 64 tokens.
 // STEPS k-steps of 32 are unrolled with all their loads issued before the first MFMA.
-template <int TT, int STEPS>
+template <int TT, int STEPS, bool SWIGLU>
 __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     constexpr int KS = GH_WAVES / TT, TOKENS = 16 * TT;
-    __shared__ float red[KS][TOKENS][GH_UNITS + 1];
+    __shared__ float red[SWIGLU ? 2 : 1][KS][TOKENS][GH_UNITS + 1];
     const int slice = blockIdx.x, tok0 = blockIdx.y * TOKENS;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int tt = wave % TT, ks = wave / TT;
@@ -44,6 +48,7 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     const int kspan = a.hidden / KS;
     const uint16_t* xp = a.x + (int64_t)tok * a.hidden + ks * kspan + kg * 8;
     const uint16_t* wp = a.w1 + (int64_t)unit * a.hidden + ks * kspan + kg * 8;
+    const uint16_t* up = SWIGLU ? a.w_up + (int64_t)unit * a.hidden + ks * kspan + kg * 8 : wp;
 
     // Epilogue operands do not depend on the products: request them first so that their latency hides under the main loop.
     constexpr int HB = 8;                       // heads per epilogue pass
@@ -59,23 +64,30 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
             if (i < a.kv_heads) w2v[i] = bf16_bits_to_f32(a.w2[(int64_t)i * a.inter + eu]);
     }
 
-    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
     for (int k0 = 0; k0 < kspan; k0 += 32 * STEPS) {
-        bf16x8_t av[STEPS], bv[STEPS];
+        bf16x8_t av[STEPS], bv[STEPS], uv[SWIGLU ? STEPS : 1];
 #pragma unroll
         for (int i = 0; i < STEPS; ++i) {
             const int k = min(k0 + 32 * i, kspan - 32);   // a short last group re-reads its final step (weight 0 below)
             av[i] = *(const bf16x8_t*)(xp + k);
             bv[i] = *(const bf16x8_t*)(wp + k);
+            if constexpr (SWIGLU) uv[i] = *(const bf16x8_t*)(up + k);
         }
 #pragma unroll
         for (int i = 0; i < STEPS; ++i) {
-            if (k0 + 32 * i < kspan) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[i], acc, 0, 0, 0);
+            if (k0 + 32 * i < kspan) {
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[i], acc, 0, 0, 0);
+                if constexpr (SWIGLU) acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], uv[i], acc_up, 0, 0, 0);
+            }
         }
     }
     // D[i][j]: lane holds token i = 4*(lane/16) + v, unit j = lane%16
 #pragma unroll
-    for (int v = 0; v < 4; ++v) red[ks][tt * 16 + kg * 4 + v][row] = acc[v];
+    for (int v = 0; v < 4; ++v) {
+        red[0][ks][tt * 16 + kg * 4 + v][row] = acc[v];
+        if constexpr (SWIGLU) red[1][ks][tt * 16 + kg * 4 + v][row] = acc_up[v];
+    }
     __syncthreads();
 
     // one (token, unit) per thread: bias, SiLU, then the contraction with W2 over the 16 units
@@ -83,11 +95,18 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
         const int t = tid >> 4, u = tid & 15;
         float h = 0.0f;
 #pragma unroll
-        for (int i = 0; i < KS; ++i) h += red[i][t][u];
+        for (int i = 0; i < KS; ++i) h += red[0][i][t][u];
         h += b1v;
         h = bf16_bits_to_f32(f32_to_bf16_bits(h));            // nn.Linear output in bf16
         float act = h / (1.0f + __expf(-h));
         act = bf16_bits_to_f32(f32_to_bf16_bits(act));        // SiLU output in bf16
+        if constexpr (SWIGLU) {
+            float up_v = 0.0f;
+#pragma unroll
+            for (int i = 0; i < KS; ++i) up_v += red[1][i][t][u];
+            up_v = bf16_bits_to_f32(f32_to_bf16_bits(up_v));  // up_proj output in bf16
+            act = bf16_bits_to_f32(f32_to_bf16_bits(act * up_v));
+        }
         for (int h0 = 0; h0 < a.kv_heads; h0 += HB) {
             if (h0 > 0) {                                      // more than HB heads: fetch the next batch of W2
 #pragma unroll
@@ -118,25 +137,38 @@ using namespace trimkv;
 
 extern "C" int trimkv_gate_slices(int inter) { return inter > 0 && inter % GH_UNITS == 0 ? inter / GH_UNITS : 0; }
 
-extern "C" int trimkv_gate_hidden(const void* x, const void* w1, const void* b1, const void* w2, float* part,
-                                  int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream) {
-    const char* fn = "trimkv_gate_hidden";
-    if (!x || !w1 || !w2 || !part) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+static int gate_launch(const char* fn, const void* x, const void* w1, const void* b1, const void* w_up, const void* w2, float* part,
+                       int ntok, int hidden, int inter, int kv_heads, int dtype, bool swiglu, void* stream) {
+    if (!x || !w1 || !w2 || !part || (swiglu && !w_up)) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 gate weights are supported (dtype=%d)", fn, dtype);
     if (ntok <= 0 || hidden <= 0 || inter <= 0 || kv_heads <= 0 || kv_heads > GH_MAX_HEADS)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes ntok=%d hidden=%d inter=%d kv_heads=%d", fn, ntok, hidden, inter, kv_heads);
     if (hidden % (32 * GH_WAVES) || inter % GH_UNITS)
         return fail(TRIMKV_ERR_UNSUPPORTED, "%s: hidden must be a multiple of %d and inter of %d (got %d, %d)", fn, 32 * GH_WAVES, GH_UNITS, hidden, inter);
-    if (((uintptr_t)x | (uintptr_t)w1) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: x and w1 must be 16-byte aligned", fn);
+    if (((uintptr_t)x | (uintptr_t)w1 | (uintptr_t)w_up) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: x and the first-layer weights must be 16-byte aligned", fn);
     GateArgs a;
     a.x = (const uint16_t*)x; a.w1 = (const uint16_t*)w1; a.b1 = (const uint16_t*)b1; a.w2 = (const uint16_t*)w2; a.part = part;
+    a.w_up = (const uint16_t*)w_up;
     a.ntok = ntok; a.hidden = hidden; a.inter = inter; a.kv_heads = kv_heads;
+    hipStream_t st = (hipStream_t)stream;
     if (ntok <= 256) {  // decode-sized: 16-token tiles, 16-way split of the hidden axis
         dim3 grid(inter / GH_UNITS, (ntok + 15) / 16);
-        hipLaunchKernelGGL((gate_hidden_kernel<1, 8>), grid, dim3(GH_THREADS), 0, (hipStream_t)stream, a);
+        if (swiglu) hipLaunchKernelGGL((gate_hidden_kernel<1, 8, true>), grid, dim3(GH_THREADS), 0, st, a);
+        else hipLaunchKernelGGL((gate_hidden_kernel<1, 8, false>), grid, dim3(GH_THREADS), 0, st, a);
     } else {
         dim3 grid(inter / GH_UNITS, (ntok + 63) / 64);
-        hipLaunchKernelGGL((gate_hidden_kernel<4, 8>), grid, dim3(GH_THREADS), 0, (hipStream_t)stream, a);
+        if (swiglu) hipLaunchKernelGGL((gate_hidden_kernel<4, 8, true>), grid, dim3(GH_THREADS), 0, st, a);
+        else hipLaunchKernelGGL((gate_hidden_kernel<4, 8, false>), grid, dim3(GH_THREADS), 0, st, a);
     }
     return launch_status(fn);
+}
+
+extern "C" int trimkv_gate_hidden(const void* x, const void* w1, const void* b1, const void* w2, float* part,
+                                  int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream) {
+    return gate_launch("trimkv_gate_hidden", x, w1, b1, nullptr, w2, part, ntok, hidden, inter, kv_heads, dtype, false, stream);
+}
+
+extern "C" int trimkv_gate_hidden_swiglu(const void* x, const void* w_gate, const void* w_up, const void* w_down, float* part,
+                                         int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream) {
+    return gate_launch("trimkv_gate_hidden_swiglu", x, w_gate, nullptr, w_up, w_down, part, ntok, hidden, inter, kv_heads, dtype, true, stream);
 }

@@ -7,8 +7,8 @@ attention kernels: per layer ``retention_gate(hidden) -> RoPE -> cache.update ->
 ``TrimKVCache`` (:648-652).  Parameter names follow the reference (``model.layers.N.self_attn.q_proj``,
 ``...retention_gate.linear1`` ...), so a local Qwen3 state dict plus ``trimkv_weights.pth`` loads with
 ``load_state_dict``; nothing here downloads anything.  The dense projections, norms and RoPE are plain
-torch ops (rocBLAS/hipBLASLt GEMMs); training, the rg2/rg3 gates and generation utilities beyond greedy
-decoding are out of scope.
+torch ops (rocBLAS/hipBLASLt GEMMs); the gates ``rg``, ``rg2`` and ``rg3`` run on the fused HIP path; training and
+generation utilities beyond greedy decoding are out of scope.
 """
 from __future__ import annotations
 
@@ -22,7 +22,7 @@ import torch.nn.functional as F
 
 from .attn import get_attention_interface
 from .cache_utils import TrimKVCache
-from .gate import RetentionGate
+from .gate import RetentionGate, RetentionGate2, RetentionGate3
 
 
 @dataclass
@@ -110,10 +110,14 @@ class TrimKVQwen3Attention(nn.Module):
         if config.retention_gate == "rg":
             self.retention_gate = RetentionGate(hs, config.num_key_value_heads, config.retention_gate_intermediate_size,
                                                 config.retention_gate_bias_init, config.initializer_range, config.hidden_act)
+        elif config.retention_gate in ("rg2", "rg3"):
+            kind = RetentionGate2 if config.retention_gate == "rg2" else RetentionGate3
+            self.retention_gate = kind(d, config.num_key_value_heads, config.retention_gate_intermediate_size,
+                                       config.retention_gate_bias_init, config.initializer_range, config.hidden_act)
         elif config.retention_gate is None:
             self.retention_gate = None
         else:
-            raise NotImplementedError(f"retention gate {config.retention_gate!r}: only 'rg' is built")
+            raise NotImplementedError(f"retention gate {config.retention_gate!r}: 'rg', 'rg2', 'rg3' or None")
 
     def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
         B, S, _ = hidden_states.shape
@@ -121,10 +125,12 @@ class TrimKVQwen3Attention(nn.Module):
         q = self.q_norm(self.q_proj(hidden_states).view(shape)).transpose(1, 2)
         k = self.k_norm(self.k_proj(hidden_states).view(shape)).transpose(1, 2)
         v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
-        # the gate sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
-        retention = self.retention_gate(hidden_states).transpose(1, 2) if self.retention_gate is not None else None
+        # `rg` sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
+        retention = self.retention_gate(hidden_states).transpose(1, 2) if self.config.retention_gate == "rg" else None
         cos, sin = position_embeddings
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        if self.config.retention_gate in ("rg2", "rg3"):   # these see concat(K, V) after RoPE (qwen3:345-347)
+            retention = self.retention_gate(torch.cat([k, v], dim=-1)).transpose(1, 2)
         offset = past_key_values.get_seq_length(self.layer_idx)
         k, v, retention, kv_positions, fa_kwargs = past_key_values.update(
             k, v, retention, cache_position, self.layer_idx,
