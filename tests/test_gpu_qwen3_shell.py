@@ -1,4 +1,4 @@
-"""End to end through the thin Qwen3 shell: fused gate -> RoPE -> cache.update -> HIP attention per layer, compress after
+"""End to end through the thin decoder shells (Qwen3, and the Llama and Phi-3 call-order variants): fused gate -> RoPE -> cache.update -> HIP attention per layer, compress after
 the final norm, in the reference's call order (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:315-388, 751-760).
 
 The logits of the bf16 GPU model are checked against the same weights evaluated in fp32 on the CPU by a replay that keeps
@@ -15,13 +15,28 @@ from tests.gpu_util import DEV
 pytestmark = pytest.mark.gpu
 
 
-def _tiny_config(**kw):
-    from trimkv_amd.qwen3 import TrimKVQwen3Config
+def _family(name):
+    if name == "llama":
+        from trimkv_amd.llama import TrimKVLlamaConfig, TrimKVLlamaForCausalLM
+        return TrimKVLlamaConfig, TrimKVLlamaForCausalLM
+    if name == "phi3":
+        from trimkv_amd.phi3 import TrimKVPhi3Config, TrimKVPhi3ForCausalLM
+        return TrimKVPhi3Config, TrimKVPhi3ForCausalLM
+    from trimkv_amd.qwen3 import TrimKVQwen3Config, TrimKVQwen3ForCausalLM
+    return TrimKVQwen3Config, TrimKVQwen3ForCausalLM
+
+
+def _tiny_config(family="qwen3", **kw):
     base = dict(vocab_size=512, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
                 num_key_value_heads=2, head_dim=128, retention_gate_intermediate_size=64, retention_gate_bias_init=2.0,
                 memory_size=64, buffer_size=16, rope_theta=10000.0)
+    if family == "llama":      # Llama-3 frequency scaling with a short original context so that it bites at these lengths
+        base["rope_scaling"] = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                    original_max_position_embeddings=64)
+    if family == "phi3":       # three query heads per KV head, rotary on 3/4 of the features, tied embeddings
+        base.update(num_attention_heads=6, hidden_size=1024, tie_word_embeddings=True, partial_rotary_factor=0.75)
     base.update(kw)
-    return TrimKVQwen3Config(**base)
+    return _family(family)[0](**base)
 
 
 class _ReplayCache:
@@ -72,14 +87,14 @@ def _record_updates(cache, nlayers):
     return rec
 
 
-@pytest.mark.parametrize("gate", ["rg", "rg2", "rg3"])
-def test_shell_logits_match_fp32_replay_of_retained_positions(gate):
+@pytest.mark.parametrize("family,gate", [("qwen3", "rg"), ("qwen3", "rg2"), ("qwen3", "rg3"), ("llama", "rg"), ("llama", "rg2"),
+                                         ("phi3", "rg"), ("phi3", "rg2")])
+def test_shell_logits_match_fp32_replay_of_retained_positions(family, gate):
     from trimkv_amd import TrimKVCache, LazyLogBeta
-    from trimkv_amd.qwen3 import TrimKVQwen3ForCausalLM
     from trimkv_amd import attn as attn_registry
     torch.manual_seed(0)
-    cfg = _tiny_config(retention_gate=gate)
-    model = TrimKVQwen3ForCausalLM(cfg).to(torch.bfloat16).eval()
+    cfg = _tiny_config(family, retention_gate=gate)
+    model = _family(family)[1](cfg).to(torch.bfloat16).eval()
     ref = copy.deepcopy(model).float()
     ref.config = copy.copy(cfg)
     for m in ref.modules():

@@ -38,6 +38,55 @@ def test_kv_gate_parameter_names_and_shapes():
         TrimKVQwen3ForCausalLM(dataclasses.replace(_tiny(), retention_gate="rg9"))
 
 
+def test_llama_and_phi3_parameter_names_follow_the_reference():
+    """Llama: no q/k norms (modeling_trimkv_llama.py:280-291); Phi-3: fused qkv_proj and gate_up_proj
+    (modeling_trimkv_phi3.py:98-99, 336-338); both accept rg and rg2 only."""
+    from trimkv_amd.llama import TrimKVLlamaConfig, TrimKVLlamaForCausalLM
+    from trimkv_amd.phi3 import TrimKVPhi3Config, TrimKVPhi3ForCausalLM
+    tiny = dict(vocab_size=64, hidden_size=512, intermediate_size=128, num_hidden_layers=1, num_attention_heads=4,
+                num_key_value_heads=2, head_dim=128, retention_gate_intermediate_size=32)
+    gate = ["self_attn.retention_gate.linear1.weight", "self_attn.retention_gate.linear1.bias",
+            "self_attn.retention_gate.linear2.weight", "self_attn.retention_gate.bias"]
+    norms = ["input_layernorm.weight", "post_attention_layernorm.weight"]
+    top = {"model.embed_tokens.weight", "model.norm.weight", "lm_head.weight"}
+    llama = set(TrimKVLlamaForCausalLM(TrimKVLlamaConfig(**tiny)).state_dict())
+    assert llama == top | {"model.layers.0." + k for k in gate + norms + [
+        "self_attn.q_proj.weight", "self_attn.k_proj.weight", "self_attn.v_proj.weight", "self_attn.o_proj.weight",
+        "mlp.gate_proj.weight", "mlp.up_proj.weight", "mlp.down_proj.weight"]}
+    m = TrimKVPhi3ForCausalLM(TrimKVPhi3Config(**tiny))
+    assert set(m.state_dict()) == top | {"model.layers.0." + k for k in gate + norms + [
+        "self_attn.qkv_proj.weight", "self_attn.o_proj.weight", "mlp.gate_up_proj.weight", "mlp.down_proj.weight"]}
+    assert m.model.layers[0].self_attn.qkv_proj.weight.shape == ((4 + 2 * 2) * 128, 512)
+    assert m.lm_head.weight is m.model.embed_tokens.weight                      # tied, as Phi-4-mini ships
+    for cfg_cls, model_cls in ((TrimKVLlamaConfig, TrimKVLlamaForCausalLM), (TrimKVPhi3Config, TrimKVPhi3ForCausalLM)):
+        with pytest.raises(NotImplementedError):
+            model_cls(cfg_cls(retention_gate="rg3", **tiny))
+        assert cfg_cls().memory_size == 2048 and cfg_cls().buffer_size == 1      # configuration_trimkv_llama.py:29, 36
+
+
+def test_partial_rotary_and_llama3_scaling():
+    pos = torch.arange(50)[None]
+    x = torch.randn(1, 2, 50, 128, generator=torch.Generator().manual_seed(0))
+    cos, sin = rotary_tables(pos, 128, 10000.0, torch.float32, rotary_dim=96)
+    assert cos.shape == (1, 50, 96)
+    y = apply_rope(x, cos, sin)
+    assert torch.equal(y[..., 96:], x[..., 96:])                                 # the last quarter passes through
+    full_cos, full_sin = rotary_tables(pos, 96, 10000.0, torch.float32)
+    assert torch.allclose(y[..., :96], apply_rope(x[..., :96].contiguous(), full_cos, full_sin))
+    # llama3 scaling: factor 1 is the identity; otherwise the fastest frequency is untouched and the slowest divided by the factor
+    rs = dict(rope_type="llama3", factor=1.0, low_freq_factor=1.0, high_freq_factor=4.0, original_max_position_embeddings=8192)
+    c0, s0 = rotary_tables(pos, 128, 500000.0, torch.float64)
+    c1, s1 = rotary_tables(pos, 128, 500000.0, torch.float64, rope_scaling=rs)
+    assert torch.allclose(c0, c1) and torch.allclose(s0, s1)
+    rs["factor"] = 8.0
+    c8, s8 = rotary_tables(pos, 128, 500000.0, torch.float64, rope_scaling=rs)
+    assert torch.allclose(c8[..., 0], c0[..., 0])                                # wavelength 2*pi << 8192/4: kept
+    inv_last = 500000.0 ** (-126 / 128)                                         # wavelength >> 8192: slowed by 8
+    assert torch.allclose(s8[0, :, 63], torch.sin(pos[0].double() * inv_last / 8.0), atol=1e-6)
+    with pytest.raises(NotImplementedError):
+        rotary_tables(pos, 128, 1e4, torch.float32, rope_scaling={"rope_type": "longrope"})
+
+
 def test_gate_init_matches_reference_reset():
     m = TrimKVQwen3ForCausalLM(_tiny())
     g = m.model.layers[0].self_attn.retention_gate

@@ -70,36 +70,59 @@ class RMSNorm(nn.Module):
 class MLP(nn.Module):
     def __init__(self, config: TrimKVQwen3Config):
         super().__init__()
-        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
-        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
-        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+        bias = getattr(config, "mlp_bias", False)
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=bias)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=bias)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=bias)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
 
 
-def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype):
-    """cos, sin [B, S, head_dim] of the default RoPE (frequencies theta^(-2i/d), halves concatenated)."""
-    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, device=position_ids.device, dtype=torch.float32) / head_dim))
+def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype,
+                  rotary_dim: Optional[int] = None, rope_scaling: Optional[dict] = None):
+    """cos, sin [B, S, rotary_dim] of RoPE (frequencies theta^(-2i/rotary_dim), halves concatenated).  ``rope_scaling``:
+    None/"default", or the published "llama3" rule (wavelengths above ``original/low_freq_factor`` are slowed by
+    ``factor``, those below ``original/high_freq_factor`` kept, a linear blend in between)."""
+    rd = head_dim if rotary_dim is None else rotary_dim
+    inv_freq = 1.0 / (theta ** (torch.arange(0, rd, 2, device=position_ids.device, dtype=torch.float32) / rd))
+    kind = (rope_scaling or {}).get("rope_type", (rope_scaling or {}).get("type", "default"))
+    if kind == "llama3":
+        factor, lo, hi = rope_scaling["factor"], rope_scaling["low_freq_factor"], rope_scaling["high_freq_factor"]
+        orig = rope_scaling["original_max_position_embeddings"]
+        wavelen = 2 * torch.pi / inv_freq
+        blend = ((orig / wavelen - lo) / (hi - lo)).clamp(0.0, 1.0)
+        inv_freq = (1 - blend) * inv_freq / factor + blend * inv_freq
+    elif kind != "default":
+        raise NotImplementedError(f"rope scaling {kind!r}")
     ang = position_ids[..., None].float() * inv_freq
     emb = torch.cat([ang, ang], dim=-1)
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
 def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
-    """x [B, H, S, D]; cos/sin [B, S, D]."""
-    half = x.shape[-1] // 2
-    rot = torch.cat([-x[..., half:], x[..., :half]], dim=-1)
-    return x * cos[:, None] + rot * sin[:, None]
+    """x [B, H, S, D]; cos/sin [B, S, R] with R <= D: the first R features are rotated, the rest pass through."""
+    rd = cos.shape[-1]
+    xr = x[..., :rd]
+    half = rd // 2
+    rot = torch.cat([-xr[..., half:], xr[..., :half]], dim=-1)
+    out = xr * cos[:, None] + rot * sin[:, None]
+    return out if rd == x.shape[-1] else torch.cat([out, x[..., rd:]], dim=-1)
 
 
 class TrimKVQwen3Attention(nn.Module):
+    gate_kinds = ("rg", "rg2", "rg3")   # the gates the reference's Qwen3 attention accepts (qwen3:295-302)
+
     def __init__(self, config: TrimKVQwen3Config, layer_idx: int):
         super().__init__()
         self.config, self.layer_idx = config, layer_idx
         self.head_dim = config.head_dim
         self.num_key_value_groups = config.num_attention_heads // config.num_key_value_heads
         self.scaling = self.head_dim ** -0.5
+        self._build_projections(config)
+        self.retention_gate = self._build_gate(config)
+
+    def _build_projections(self, config) -> None:
         hs, d = config.hidden_size, config.head_dim
         self.q_proj = nn.Linear(hs, config.num_attention_heads * d, bias=config.attention_bias)
         self.k_proj = nn.Linear(hs, config.num_key_value_heads * d, bias=config.attention_bias)
@@ -107,24 +130,31 @@ class TrimKVQwen3Attention(nn.Module):
         self.o_proj = nn.Linear(config.num_attention_heads * d, hs, bias=config.attention_bias)
         self.q_norm = RMSNorm(d, config.rms_norm_eps)
         self.k_norm = RMSNorm(d, config.rms_norm_eps)
-        if config.retention_gate == "rg":
-            self.retention_gate = RetentionGate(hs, config.num_key_value_heads, config.retention_gate_intermediate_size,
-                                                config.retention_gate_bias_init, config.initializer_range, config.hidden_act)
-        elif config.retention_gate in ("rg2", "rg3"):
-            kind = RetentionGate2 if config.retention_gate == "rg2" else RetentionGate3
-            self.retention_gate = kind(d, config.num_key_value_heads, config.retention_gate_intermediate_size,
-                                       config.retention_gate_bias_init, config.initializer_range, config.hidden_act)
-        elif config.retention_gate is None:
-            self.retention_gate = None
-        else:
-            raise NotImplementedError(f"retention gate {config.retention_gate!r}: 'rg', 'rg2', 'rg3' or None")
 
-    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
+    def _build_gate(self, config):
+        kind = config.retention_gate
+        if kind is None:
+            return None
+        if kind not in self.gate_kinds:
+            raise NotImplementedError(f"retention gate {kind!r}: one of {self.gate_kinds} or None")
+        common = (config.num_key_value_heads, config.retention_gate_intermediate_size, config.retention_gate_bias_init,
+                  config.initializer_range, config.hidden_act)
+        if kind == "rg":
+            return RetentionGate(config.hidden_size, *common)
+        return (RetentionGate2 if kind == "rg2" else RetentionGate3)(config.head_dim, *common)
+
+    def _qkv(self, hidden_states: torch.Tensor):
+        """q [B,Hq,S,D], k and v [B,Hkv,S,D] before RoPE (qwen3:326-328, 335-337: per-head RMS norm on q and k)."""
         B, S, _ = hidden_states.shape
         shape = (B, S, -1, self.head_dim)
         q = self.q_norm(self.q_proj(hidden_states).view(shape)).transpose(1, 2)
         k = self.k_norm(self.k_proj(hidden_states).view(shape)).transpose(1, 2)
         v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
+        return q, k, v
+
+    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
+        B, S, _ = hidden_states.shape
+        q, k, v = self._qkv(hidden_states)
         # `rg` sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
         retention = self.retention_gate(hidden_states).transpose(1, 2) if self.config.retention_gate == "rg" else None
         cos, sin = position_embeddings
@@ -143,10 +173,12 @@ class TrimKVQwen3Attention(nn.Module):
 
 
 class TrimKVQwen3DecoderLayer(nn.Module):
+    attention_cls, mlp_cls = TrimKVQwen3Attention, MLP
+
     def __init__(self, config: TrimKVQwen3Config, layer_idx: int):
         super().__init__()
-        self.self_attn = TrimKVQwen3Attention(config, layer_idx)
-        self.mlp = MLP(config)
+        self.self_attn = self.attention_cls(config, layer_idx)
+        self.mlp = self.mlp_cls(config)
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
@@ -157,11 +189,13 @@ class TrimKVQwen3DecoderLayer(nn.Module):
 
 
 class TrimKVQwen3Model(nn.Module):
+    layer_cls = TrimKVQwen3DecoderLayer
+
     def __init__(self, config: TrimKVQwen3Config):
         super().__init__()
         self.config = config
         self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
-        self.layers = nn.ModuleList([TrimKVQwen3DecoderLayer(config, i) for i in range(config.num_hidden_layers)])
+        self.layers = nn.ModuleList([self.layer_cls(config, i) for i in range(config.num_hidden_layers)])
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
     def forward(self, input_ids=None, past_key_values=None, inputs_embeds=None, cache_position=None, position_ids=None,
@@ -177,7 +211,9 @@ class TrimKVQwen3Model(nn.Module):
             cache_position = torch.arange(seen, seen + inputs_embeds.shape[1], device=inputs_embeds.device)
         if position_ids is None:
             position_ids = cache_position.unsqueeze(0)
-        position_embeddings = rotary_tables(position_ids, self.config.head_dim, self.config.rope_theta, inputs_embeds.dtype)
+        c = self.config
+        position_embeddings = rotary_tables(position_ids, c.head_dim, c.rope_theta, inputs_embeds.dtype,
+                                            int(c.head_dim * getattr(c, "partial_rotary_factor", 1.0)), getattr(c, "rope_scaling", None))
         hidden_states = inputs_embeds
         for layer in self.layers:
             hidden_states = layer(hidden_states, position_embeddings, attention_mask, past_key_values, cache_position)
@@ -191,10 +227,12 @@ class TrimKVQwen3Model(nn.Module):
 
 
 class TrimKVQwen3ForCausalLM(nn.Module):
+    model_cls = TrimKVQwen3Model
+
     def __init__(self, config: TrimKVQwen3Config):
         super().__init__()
         self.config = config
-        self.model = TrimKVQwen3Model(config)
+        self.model = self.model_cls(config)
         self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
         if config.tie_word_embeddings:
             self.lm_head.weight = self.model.embed_tokens.weight
