@@ -19,7 +19,7 @@ def _family(name):
     if name == "llama":
         from trimkv_amd.llama import TrimKVLlamaConfig, TrimKVLlamaForCausalLM
         return TrimKVLlamaConfig, TrimKVLlamaForCausalLM
-    if name == "phi3":
+    if name in ("phi3", "phi3mini"):
         from trimkv_amd.phi3 import TrimKVPhi3Config, TrimKVPhi3ForCausalLM
         return TrimKVPhi3Config, TrimKVPhi3ForCausalLM
     from trimkv_amd.qwen3 import TrimKVQwen3Config, TrimKVQwen3ForCausalLM
@@ -35,6 +35,8 @@ def _tiny_config(family="qwen3", **kw):
                                     original_max_position_embeddings=64)
     if family == "phi3":       # three query heads per KV head, rotary on 3/4 of the features, tied embeddings
         base.update(num_attention_heads=6, hidden_size=1024, tie_word_embeddings=True, partial_rotary_factor=0.75)
+    if family == "phi3mini":   # the released TrimKV Phi-3-mini shape in small: one query head per KV head, 96 features per head
+        base.update(num_attention_heads=4, num_key_value_heads=4, head_dim=96, hidden_size=1024, partial_rotary_factor=1.0)
     base.update(kw)
     return _family(family)[0](**base)
 
@@ -88,7 +90,7 @@ def _record_updates(cache, nlayers):
 
 
 @pytest.mark.parametrize("family,gate", [("qwen3", "rg"), ("qwen3", "rg2"), ("qwen3", "rg3"), ("llama", "rg"), ("llama", "rg2"),
-                                         ("phi3", "rg"), ("phi3", "rg2")])
+                                         ("phi3", "rg"), ("phi3", "rg2"), ("phi3mini", "rg")])
 def test_shell_logits_match_fp32_replay_of_retained_positions(family, gate):
     from trimkv_amd import TrimKVCache, LazyLogBeta
     from trimkv_amd import attn as attn_registry

@@ -32,7 +32,7 @@ typedef float f32x2_t __attribute__((ext_vector_type(2)));
 
 constexpr int AT_THREADS = 256;
 constexpr int AT_WAVES = 4;
-constexpr int AT_D = 128;            // head_dim
+constexpr int AT_D = 128;            // head_dim the lane layout is built for; 64 and 96 run zero-padded to it
 constexpr int AT_BLOCK_ROWS = 128;   // rows one wavefront scores before it touches V
 constexpr float AT_NEG = -1.0e30f;   // "minus infinity" that stays finite under subtraction
 
@@ -97,8 +97,11 @@ struct AttnArgs {
 // Attention of the G query heads of segment `seg` over its rows [t0, t1): the body shared by both kernels.
 // `direct`: normalise and write the output; otherwise the unnormalised accumulator and (max, sum) go to partial
 // slot `slot` of the workspace.  All 256 threads of the workgroup must call it together (it uses barriers).
-template <int G>
+// ROW16: 16-byte pieces per K/V/q row (head_dim / 8).  With fewer than 16, lanes c >= ROW16 of each 16-lane row group
+// re-read the row's last piece and hold q = 0, so they add nothing to the scores; what they accumulate is not stored.
+template <int G, int ROW16>
 __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base) {
+    constexpr int D_REAL = ROW16 * 8;
     using C = AttnCfg<G>;
     constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
 
@@ -114,15 +117,19 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     const int w0 = t0 + w * pw, w1 = min(t1, w0 + pw);
 
     const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
-    const uint4* kp = a.k + row0 * 16 + c;  // 16 uint4 per 256-byte row; this lane's 16-byte column
-    const uint4* vp = a.v + row0 * 16 + c;
+    const int cc = ROW16 == 16 ? c : min(c, ROW16 - 1);
+    const uint4* kp = a.k + row0 * ROW16 + cc;  // ROW16 uint4 per row; this lane's 16-byte column
+    const uint4* vp = a.v + row0 * ROW16 + cc;
 
     // q is loaded and waited for before the first K/V prefetch is issued: if its loads were still
     // outstanding behind the prefetches, the wait for q at the first q.K (static code, executed by
     // every block) would drain the whole prefetch ring each time.
     uint4 qv[G];
 #pragma unroll
-    for (int g = 0; g < G; ++g) qv[g] = a.q[((int64_t)seg * G + g) * 16 + c];
+    for (int g = 0; g < G; ++g) {
+        qv[g] = a.q[((int64_t)seg * G + g) * ROW16 + cc];
+        if (ROW16 < 16 && c >= ROW16) qv[g] = make_uint4(0u, 0u, 0u, 0u);
+    }
 #pragma unroll
     for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
 
@@ -147,7 +154,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             const int row = min(row_begin + j * 4 + r, w1 - 1);  // rows past the end re-read the last one (weight 0)
             // K/V are read once per step and never again before they have left every cache: a non-temporal load
             // (streaming hint) moves them about 13 % faster than a plain one on this part
-            const at_u32x4 t = __builtin_nontemporal_load((const at_u32x4*)(base + (int64_t)row * 16));
+            const at_u32x4 t = __builtin_nontemporal_load((const at_u32x4*)(base + (int64_t)row * ROW16));
             dst[j] = make_uint4(t.x, t.y, t.z, t.w);
         }
     };
@@ -335,7 +342,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         }
         if (direct) {
             const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-            ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
+            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = f32_to_bf16_bits(y);
         } else {
             const int64_t slot = slot_base * G + g;
             a.ws_o[slot * AT_D + d] = acc;
@@ -344,7 +351,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     }
 }
 
-template <int G>
+template <int G, int ROW16>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2))) void decode_attn_kernel(AttnArgs a) {
     // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
     // axis so that consecutive ids are different segments: with the split as the fast axis and 8
@@ -362,13 +369,13 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
     const int nsp = (n + a.chunk - 1) / a.chunk;
     if (split >= nsp) {
         if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
-            for (int i = threadIdx.x; i < G * AT_D; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * AT_D + i] = 0;
+            for (int i = threadIdx.x; i < G * ROW16 * 8; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * (ROW16 * 8) + i] = 0;
         }
         return;
     }
     const int rps = (n + nsp - 1) / nsp;
     const int t0 = split * rps, t1 = min(n, t0 + rps);
-    attend_rows<G>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split);
+    attend_rows<G, ROW16>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split);
 }
 
 // Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
@@ -376,7 +383,7 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 // kernel boundary is what makes partials written on one XCD visible on another; doing the same
 // inside one kernel needs device-scope fences (an L2 write-back and invalidate per workgroup on
 // this part), which costs far more than the launch.
-template <int G>
+template <int G, int ROW16>
 __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
     const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
@@ -410,7 +417,7 @@ __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a)
         lsum += f * a.ws_ml[slot * 2 + 1];
     }
     const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-    ((uint16_t*)a.out)[((int64_t)seg * G + g) * AT_D + d] = f32_to_bf16_bits(y);
+    if (d < ROW16 * 8) ((uint16_t*)a.out)[((int64_t)seg * G + g) * (ROW16 * 8) + d] = f32_to_bf16_bits(y);
 }
 
 static int pick_chunk(int nseg, int max_len) {
@@ -425,10 +432,17 @@ static int pick_chunk(int nseg, int max_len) {
     return chunk < whole ? chunk : whole;
 }
 
+template <int G, int ROW16>
+static void launch_attn_rows(const AttnArgs& a, hipStream_t st) {
+    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
+    if (!a.direct) hipLaunchKernelGGL((decode_attn_merge_kernel<G, ROW16>), dim3(a.nseg), dim3(G * AT_D), 0, st, a);
+}
+
 template <int G>
-static void launch_attn(const AttnArgs& a, hipStream_t st) {
-    hipLaunchKernelGGL(decode_attn_kernel<G>, dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
-    if (!a.direct) hipLaunchKernelGGL(decode_attn_merge_kernel<G>, dim3(a.nseg), dim3(G * AT_D), 0, st, a);
+static void launch_attn(const AttnArgs& a, int head_dim, hipStream_t st) {
+    if (head_dim == 128) launch_attn_rows<G, 16>(a, st);
+    else if (head_dim == 96) launch_attn_rows<G, 12>(a, st);
+    else launch_attn_rows<G, 8>(a, st);
 }
 
 }  // namespace trimkv
@@ -440,7 +454,7 @@ extern "C" size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim
     if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
     const int nsplit = (max_len + chunk - 1) / chunk;
     if (nsplit <= 1) return 0;
-    return (size_t)nseg * nsplit * group * (head_dim + 2) * sizeof(float);
+    return (size_t)nseg * nsplit * group * (AT_D + 2) * sizeof(float);   // partial rows are padded to 128 features
 }
 
 extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
@@ -450,7 +464,7 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     const char* fn = "trimkv_decode_attn";
     if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
-    if (head_dim != AT_D) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be %d (got %d)", fn, AT_D, head_dim);
+    if (head_dim != 128 && head_dim != 96 && head_dim != 64) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be 64, 96 or 128 (got %d)", fn, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
     if (!seg_start && max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
@@ -474,14 +488,14 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     }
     hipStream_t st = (hipStream_t)stream;
     switch (group) {
-        case 1: launch_attn<1>(a, st); break;
-        case 2: launch_attn<2>(a, st); break;
-        case 3: launch_attn<3>(a, st); break;
-        case 4: launch_attn<4>(a, st); break;
-        case 5: launch_attn<5>(a, st); break;
-        case 6: launch_attn<6>(a, st); break;
-        case 7: launch_attn<7>(a, st); break;
-        default: launch_attn<8>(a, st); break;
+        case 1: launch_attn<1>(a, head_dim, st); break;
+        case 2: launch_attn<2>(a, head_dim, st); break;
+        case 3: launch_attn<3>(a, head_dim, st); break;
+        case 4: launch_attn<4>(a, head_dim, st); break;
+        case 5: launch_attn<5>(a, head_dim, st); break;
+        case 6: launch_attn<6>(a, head_dim, st); break;
+        case 7: launch_attn<7>(a, head_dim, st); break;
+        default: launch_attn<8>(a, head_dim, st); break;
     }
     return launch_status(fn);
 }

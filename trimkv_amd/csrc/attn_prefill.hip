@@ -35,7 +35,7 @@ typedef float pf_f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 pf_bf16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t pf_u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int PF_D = 128;
+constexpr int PF_D = 128;                  // head_dim the tiles are built for; 64 and 96 run zero-padded to it (q = 0 there)
 constexpr int PF_BN = 32;                  // keys per tile
 constexpr int PF_ROW = 272;                // LDS bytes per K/V row: 256 + 16 keeps b128 alignment and spreads banks
 constexpr float PF_NEG = -1.0e30f;
@@ -46,6 +46,7 @@ struct PrefillArgs {
     const char* k; const char* v;
     const int32_t* seg_len; const int32_t* seg_start;
     int kv_heads, group, q_len, cap, max_len;
+    int hd;                                         // real head_dim: rows of K, V, q and out hold hd elements
     float scale_log2;
 };
 
@@ -89,7 +90,11 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
     {
         const uint16_t* qrow = a.q + (int64_t)b * a.q_sb + (int64_t)(h * G + g) * a.q_sh + (int64_t)min(t_q, Q - 1) * a.q_st;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const pf_bf16x8*)(qrow + ig * 32 + ks * 8);
+        for (int ks = 0; ks < 4; ++ks) {
+            const int e0 = ig * 32 + ks * 8;
+            qf[ks] = *(const pf_bf16x8*)(qrow + min(e0, a.hd - 8));
+            if (e0 >= a.hd) qf[ks] = pf_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};   // padded features: whatever K holds there counts for nothing
+        }
     }
 
     pf_f32x4 oe[4], oo[4];  // O^T accumulators: d = 2*(pb*16 + 4*ig + v) (even) and +1 (odd), query j
@@ -112,7 +117,7 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
             if (p < 2 * PF_BN * 16) {
                 const int isv = p >= PF_BN * 16, q16 = p & 15, key = (p >> 4) & (PF_BN - 1);
                 const int row = min(kbase + key, max(n - 1, 0));
-                const char* src = (isv ? a.v : a.k) + (row0 + row) * (int64_t)(PF_D * 2) + q16 * 16;
+                const char* src = (isv ? a.v : a.k) + (row0 + row) * (int64_t)(a.hd * 2) + min(q16 * 16, a.hd * 2 - 16);
                 stage[i] = *(const pf_u32x4*)src;
             }
         }
@@ -212,11 +217,12 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
     l_run += __shfl_xor(l_run, 32, 64);
     if (q_ok) {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        uint32_t* orow = (uint32_t*)(a.out + (((int64_t)b * Q + t_q) * (a.kv_heads * G) + (h * G + g)) * PF_D);
+        uint32_t* orow = (uint32_t*)(a.out + (((int64_t)b * Q + t_q) * (a.kv_heads * G) + (h * G + g)) * a.hd);
 #pragma unroll
         for (int pb = 0; pb < 4; ++pb) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) orow[pb * 16 + 4 * ig + v] = pack_bf16(oe[pb][v] * inv, oo[pb][v] * inv);
+            for (int v = 0; v < 4; ++v)
+                if (2 * (pb * 16 + 4 * ig + v) < a.hd) orow[pb * 16 + 4 * ig + v] = pack_bf16(oe[pb][v] * inv, oo[pb][v] * inv);
         }
     }
 }
@@ -290,7 +296,11 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     {
         const uint16_t* qrow = a.q + (int64_t)b * a.q_sb + (int64_t)(h * G + g) * a.q_sh + (int64_t)min(t_q, Q - 1) * a.q_st;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qf[ks] = *(const pf_bf16x8*)(qrow + ks * 16 + hl * 8);
+        for (int ks = 0; ks < 8; ++ks) {
+            const int e0 = ks * 16 + hl * 8;
+            qf[ks] = *(const pf_bf16x8*)(qrow + min(e0, a.hd - 8));
+            if (e0 >= a.hd) qf[ks] = pf_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};   // padded features: whatever K holds there counts for nothing
+        }
     }
 
     pf_f32x16 o[4];   // O^T: o[db][v] = d (db * 32 + 8 * (v / 4) + 4 * hl + v % 4) of query j
@@ -314,32 +324,33 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     // Per-thread pieces are fixed; only the tile base moves.  Rows are addressed as 32-bit byte offsets from the
     // segment's (wave-uniform) base and clamped to the last row, so every load is unconditional.
     pf_u32x4 kst[PF2_KPIECES], vst[PF2_VPIECES][2];
-    const char* kseg = a.k + row0 * (int64_t)(PF_D * 2);
-    const char* vseg = a.v + row0 * (int64_t)(PF_D * 2);
+    const uint32_t row_bytes = (uint32_t)a.hd * 2u;
+    const char* kseg = a.k + row0 * (int64_t)row_bytes;
+    const char* vseg = a.v + row0 * (int64_t)row_bytes;
     int k_row[PF2_KPIECES], v_row[PF2_VPIECES];
     uint32_t k_col[PF2_KPIECES], v_col[PF2_VPIECES];
 #pragma unroll
     for (int i = 0; i < PF2_KPIECES; ++i) {
         const int p = tid + i * PF2_THREADS;
         k_row[i] = p >> 4;
-        k_col[i] = (p & 15) * 16;
+        k_col[i] = min((uint32_t)(p & 15) * 16u, row_bytes - 16u);   // pieces past a short row re-read its last one
     }
 #pragma unroll
     for (int i = 0; i < PF2_VPIECES; ++i) {
         const int p = tid + i * PF2_THREADS;
         v_row[i] = pf2_key_of_slot(pf2_vpiece_sp(p) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
-        v_col[i] = pf2_vpiece_dchunk(p) * 16;
+        v_col[i] = min((uint32_t)pf2_vpiece_dchunk(p) * 16u, row_bytes - 16u);
     }
     auto fetch = [&](int kbase) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < PF2_KPIECES; ++i) {
-            const uint32_t off = (uint32_t)min(kbase + k_row[i], last_row) * (uint32_t)(PF_D * 2) + k_col[i];
+            const uint32_t off = (uint32_t)min(kbase + k_row[i], last_row) * row_bytes + k_col[i];
             kst[i] = *(const pf_u32x4*)(kseg + off);
         }
 #pragma unroll
         for (int i = 0; i < PF2_VPIECES; ++i) {
-            const uint32_t o0 = (uint32_t)min(kbase + v_row[i], last_row) * (uint32_t)(PF_D * 2) + v_col[i];
-            const uint32_t o1 = (uint32_t)min(kbase + v_row[i] + 1, last_row) * (uint32_t)(PF_D * 2) + v_col[i];
+            const uint32_t o0 = (uint32_t)min(kbase + v_row[i], last_row) * row_bytes + v_col[i];
+            const uint32_t o1 = (uint32_t)min(kbase + v_row[i] + 1, last_row) * row_bytes + v_col[i];
             vst[i][0] = *(const pf_u32x4*)(vseg + o0);
             vst[i][1] = *(const pf_u32x4*)(vseg + o1);
         }
@@ -521,14 +532,14 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     l_run += __shfl_xor(l_run, 32, 64);
     if (q_ok) {
         const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
-        char* orow = (char*)(a.out + (((int64_t)b * Q + t_q) * (a.kv_heads * G) + (h * G + g)) * PF_D);
+        char* orow = (char*)(a.out + (((int64_t)b * Q + t_q) * (a.kv_heads * G) + (h * G + g)) * a.hd);
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const uint2 pk = make_uint2(pack_bf16(o[db][4 * c] * inv, o[db][4 * c + 1] * inv),
                                             pack_bf16(o[db][4 * c + 2] * inv, o[db][4 * c + 3] * inv));
-                *(uint2*)(orow + (db * 32 + 8 * c + 4 * hl) * 2) = pk;
+                if (db * 32 + 8 * c + 4 * hl < a.hd) *(uint2*)(orow + (db * 32 + 8 * c + 4 * hl) * 2) = pk;
             }
         }
     }
@@ -566,7 +577,7 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
     const char* fn = "trimkv_prefill_attn";
     if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
-    if (head_dim != PF_D) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be %d (got %d)", fn, PF_D, head_dim);
+    if (head_dim != 128 && head_dim != 96 && head_dim != 64) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be 64, 96 or 128 (got %d)", fn, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (batch <= 0 || kv_heads <= 0 || q_len <= 0 || cap <= 0 || max_len <= 0)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes batch=%d kv_heads=%d q_len=%d cap=%d max_len=%d", fn, batch, kv_heads, q_len, cap, max_len);
@@ -578,7 +589,7 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
     PrefillArgs a;
     a.q = (const uint16_t*)q; a.q_sb = q_stride_b; a.q_sh = q_stride_h; a.q_st = q_stride_t; a.out = (uint16_t*)out;
     a.k = (const char*)k_slab; a.v = (const char*)v_slab; a.seg_len = seg_len; a.seg_start = seg_start;
-    a.kv_heads = kv_heads; a.group = group; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.scale_log2 = scale * 1.4426950408889634f;
+    a.kv_heads = kv_heads; a.group = group; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.hd = head_dim; a.scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
     int rc = 0;
     switch (group) {

@@ -166,6 +166,7 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
     const int lpr = 1 << lpr_shift;
     const int rpp = EV_THREADS >> lpr_shift;  // rows per pass
     const int piece = threadIdx.x & (lpr - 1), rl = threadIdx.x >> lpr_shift;
+    const bool piece_ok = (piece << 4) < row_bytes;   // rows that are not a power of two long (head_dim 96) leave lanes idle
     const int tile_rows = rpp * EV_ROW_PASSES;
     for (int base = (first_moved / tile_rows) * tile_rows; base < kept; base += tile_rows) {
         uint4 kk[EV_ROW_PASSES], vv[EV_ROW_PASSES];
@@ -176,7 +177,7 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
             mv[p] = false;
             kk[p] = make_uint4(0, 0, 0, 0);
             vv[p] = make_uint4(0, 0, 0, 0);
-            if (r < kept) {
+            if (r < kept && piece_ok) {
                 const int src = (int)idx[r];
                 if (src != r) {
                     mv[p] = true;
@@ -623,8 +624,8 @@ __global__ void cu_seqlens_kernel(const int32_t* seg_len, int nseg, int32_t* cu)
 }
 
 static int lpr_shift_of(int row_bytes) {
-    const int lpr = row_bytes / 16;
-    if (row_bytes % 16 || lpr <= 0 || (lpr & (lpr - 1)) || lpr > 64) return -1;
+    const int lpr = row_bytes / 16;   // 16-byte pieces per row; a thread group of the next power of two moves a row
+    if (row_bytes % 16 || lpr <= 0 || lpr > 64) return -1;
     int s = 0;
     while ((1 << s) < lpr) ++s;
     return s;
@@ -670,7 +671,7 @@ static int check_slab_args(const char* fn, const void* k, const void* v, const v
     if (nseg <= 0 || cap <= 0 || head_dim <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d head_dim=%d max_len=%d", fn, nseg, cap, head_dim, max_len);
     if (max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
     *lpr_shift = lpr_shift_of(head_dim * 2);
-    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be 16 * a power of two <= 1024 (head_dim=%d)", fn, head_dim);
+    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be a multiple of 16, at most 1024 (head_dim=%d)", fn, head_dim);
     if (((uintptr_t)k & 15) || ((uintptr_t)v & 15)) return fail(TRIMKV_ERR_SHAPE, "%s: slabs must be 16-byte aligned", fn);
     return TRIMKV_OK;
 }
@@ -726,7 +727,7 @@ static int check_layer_args(const char* fn, const trimkv_layer_slabs* layers, in
     if (nlayers <= 0 || nlayers > 65535 || nseg <= 0 || head_dim <= 0 || max_len <= 0)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d head_dim=%d max_len=%d", fn, nlayers, nseg, head_dim, max_len);
     *lpr_shift = lpr_shift_of(head_dim * 2);
-    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be 16 * a power of two <= 1024 (head_dim=%d)", fn, head_dim);
+    if (*lpr_shift < 0) return fail(TRIMKV_ERR_SHAPE, "%s: head_dim*2 bytes must be a multiple of 16, at most 1024 (head_dim=%d)", fn, head_dim);
     return TRIMKV_OK;
 }
 

@@ -3,8 +3,8 @@
 Against the Qwen3 shell it differs where the reference's Phi-3 file differs: one fused ``qkv_proj`` split into q | k | v
 (:353-357), a fused ``gate_up_proj`` in the MLP (:98-108), no per-head q/k norm, RoPE on the first
 ``partial_rotary_factor * head_dim`` features only (:179-186), the gates ``rg`` and ``rg2`` (:331-334).  Residual dropouts
-(:450-451) are identities at inference and have no parameters, so they are left out.  The attention kernels need
-``head_dim == 128`` (Phi-3-medium, Phi-4-mini); Phi-3-mini's 96 is refused by the library.
+(:450-451) are identities at inference and have no parameters, so they are left out.  The attention kernels take
+``head_dim`` 128 (Phi-3-medium, Phi-4-mini), 96 (Phi-3-mini) and 64.
 """
 from __future__ import annotations
 
