@@ -115,3 +115,48 @@ def test_no_cpu_fallback():
     m = TrimKVQwen3ForCausalLM(_tiny()).eval()
     with pytest.raises((TrimKVLibraryError, RuntimeError)):
         m(torch.zeros(1, 3, dtype=torch.long))
+
+
+def test_from_pretrained_reads_local_files_only(tmp_path):
+    """Base checkpoint directory (HF config.json + safetensors) and a TrimKV directory (config.json naming the base and
+    the trainable parameters + trimkv_weights.pth), as modeling_trimkv_qwen3.py:541-573 lays them out."""
+    import json
+    from safetensors.torch import save_file
+    from trimkv_amd.llama import TrimKVLlamaForCausalLM
+    torch.manual_seed(0)
+    src = TrimKVQwen3ForCausalLM(_tiny())
+    for p in src.parameters():
+        p.data.normal_(0, 0.05)
+    full = {k: v.clone() for k, v in src.state_dict().items()}
+    gate = {k: v for k, v in full.items() if "retention_gate" in k}
+    base_dir, trim_dir = tmp_path / "base", tmp_path / "trimkv"
+    base_dir.mkdir(); trim_dir.mkdir()
+    save_file({k: v.contiguous() for k, v in full.items() if k not in gate}, str(base_dir / "model.safetensors"))
+    hf = dict(vocab_size=64, hidden_size=512, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4, num_key_value_heads=2,
+              rms_norm_eps=1e-6, rope_parameters={"rope_theta": 12345.0, "rope_type": "default"}, architectures=["Qwen3ForCausalLM"])
+    (base_dir / "config.json").write_text(json.dumps(hf))
+    (trim_dir / "config.json").write_text(json.dumps(dict(hf, base_model=str(base_dir), retention_gate="rg", memory_size=77,
+                                                          retention_gate_intermediate_size=32, trainable_params="retention_gate")))
+    torch.save(gate, str(trim_dir / "trimkv_weights.pth"))
+    m = TrimKVQwen3ForCausalLM.from_pretrained(str(trim_dir), torch_dtype=None, buffer_size=5)
+    assert m.config.head_dim == 128 and m.config.rope_theta == 12345.0 and m.config.memory_size == 77 and m.config.buffer_size == 5
+    assert not m.training
+    got = m.state_dict()
+    assert set(got) == set(full) and all(torch.equal(got[k], full[k]) for k in full)
+    assert TrimKVQwen3ForCausalLM.from_pretrained(str(trim_dir)).lm_head.weight.dtype == torch.bfloat16
+    # a gate file whose keys are not the trainable parameters is refused, as in the reference (:559-567)
+    torch.save({k: v for k, v in list(gate.items())[:-1]}, str(trim_dir / "trimkv_weights.pth"))
+    with pytest.raises(ValueError, match="Mismatch"):
+        TrimKVQwen3ForCausalLM.from_pretrained(str(trim_dir))
+    with pytest.raises(RuntimeError, match="network"):
+        TrimKVQwen3ForCausalLM.from_pretrained("someone/some-model", download_from="huggingface")
+    with pytest.raises(ValueError):
+        TrimKVQwen3ForCausalLM.from_pretrained(str(tmp_path / "nowhere"))
+    # a base directory loaded on its own (load_trimkv_weights=False) keeps freshly initialised gates; missing base tensors are an error
+    m2 = TrimKVLlamaForCausalLM.from_pretrained(str(base_dir), load_trimkv_weights=False, retention_gate_intermediate_size=32)
+    assert torch.all(m2.model.layers[0].self_attn.retention_gate.bias == 10.0)
+    assert torch.equal(m2.model.layers[1].mlp.up_proj.weight, full["model.layers.1.mlp.up_proj.weight"].to(torch.bfloat16))
+    (base_dir / "model.safetensors").unlink()
+    save_file({k: v.contiguous() for k, v in full.items() if k not in gate and "mlp" not in k}, str(base_dir / "model.safetensors"))
+    with pytest.raises(ValueError, match="lacks"):
+        TrimKVLlamaForCausalLM.from_pretrained(str(base_dir), load_trimkv_weights=False, retention_gate_intermediate_size=32)

@@ -57,4 +57,5 @@ class TrimKVLlamaModel(TrimKVQwen3Model):
 
 
 class TrimKVLlamaForCausalLM(TrimKVQwen3ForCausalLM):
+    config_cls = TrimKVLlamaConfig
     model_cls = TrimKVLlamaModel

@@ -73,4 +73,5 @@ class TrimKVPhi3Model(TrimKVQwen3Model):
 
 
 class TrimKVPhi3ForCausalLM(TrimKVQwen3ForCausalLM):
+    config_cls = TrimKVPhi3Config
     model_cls = TrimKVPhi3Model

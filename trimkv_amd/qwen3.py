@@ -12,6 +12,10 @@ generation utilities beyond greedy decoding are out of scope.
 """
 from __future__ import annotations
 
+import dataclasses
+import glob
+import json
+import os
 from dataclasses import dataclass
 from types import SimpleNamespace
 from typing import Optional
@@ -52,7 +56,26 @@ class TrimKVQwen3Config:
     floor_budget_ratio: float = 0.0
     alpha_threshold: float = 0.0
     max_seq_len: int = 131072
+    base_model: Optional[str] = None          # directory of the base checkpoint (qwen3:545-549)
+    trainable_params: str = "retention_gate"  # "|"-separated substrings naming the parameters kept in trimkv_weights.pth
     _attn_implementation: str = "trimkv_hip"
+
+    @classmethod
+    def from_dict(cls, d: dict, **overrides):
+        """Pick this dataclass's fields out of an HF ``config.json`` dictionary (unknown keys are ignored; ``head_dim``
+        defaults to hidden/heads; ``rope_parameters`` of newer configs is unpacked into theta and scaling)."""
+        d = dict(d)
+        rp = d.pop("rope_parameters", None)
+        if isinstance(rp, dict):
+            d.setdefault("rope_theta", rp.get("rope_theta", d.get("rope_theta")))
+            if rp.get("rope_type", "default") != "default":
+                d.setdefault("rope_scaling", rp)
+        if d.get("head_dim") is None and "hidden_size" in d and "num_attention_heads" in d:
+            d["head_dim"] = d["hidden_size"] // d["num_attention_heads"]
+        names = {f.name for f in dataclasses.fields(cls)}
+        kept = {k: v for k, v in d.items() if k in names and v is not None}
+        kept.update({k: v for k, v in overrides.items() if k in names})
+        return cls(**kept)
 
 
 class RMSNorm(nn.Module):
@@ -226,8 +249,66 @@ class TrimKVQwen3Model(nn.Module):
         return SimpleNamespace(last_hidden_state=hidden_states, past_key_values=past_key_values)
 
 
+def _load_checkpoint_tensors(directory: str) -> dict:
+    """All tensors of a local HF checkpoint directory: ``*.safetensors`` shards, else ``pytorch_model*.bin`` read with
+    ``weights_only=True`` (nothing in the files is executed)."""
+    shards = sorted(glob.glob(os.path.join(directory, "*.safetensors")))
+    state = {}
+    if shards:
+        from safetensors.torch import load_file
+        for f in shards:
+            state.update(load_file(f))
+        return state
+    for f in sorted(glob.glob(os.path.join(directory, "pytorch_model*.bin"))):
+        state.update(torch.load(f, map_location="cpu", weights_only=True))
+    if not state:
+        raise FileNotFoundError(f"no *.safetensors or pytorch_model*.bin under {directory}")
+    return state
+
+
 class TrimKVQwen3ForCausalLM(nn.Module):
     model_cls = TrimKVQwen3Model
+    config_cls = TrimKVQwen3Config
+
+    @classmethod
+    def from_pretrained(cls, pretrained_model_name_or_path: str, load_trimkv_weights: bool = True, download_from: str = "local",
+                        torch_dtype: Optional[torch.dtype] = torch.bfloat16, **kwargs):
+        """Local-files counterpart of the reference's loader (qwen3:510-577): ``config.json`` of the TrimKV directory (keyword
+        arguments that name config fields override it), base weights from ``config.base_model`` (a local directory; the
+        TrimKV directory itself when the field is absent), then ``trimkv_weights.pth``, whose keys must be exactly the
+        model's parameters selected by ``config.trainable_params``.  Nothing is downloaded: the ``wandb`` and
+        ``huggingface`` sources of the reference raise here."""
+        if download_from in ("wandb", "huggingface"):
+            raise RuntimeError(f"download_from={download_from!r} needs the network; fetch the files and pass the local directory")
+        if download_from != "local":
+            raise ValueError(f"Unsupported download_from value: {download_from}")
+        path = pretrained_model_name_or_path
+        if not os.path.isdir(path):
+            raise ValueError(f"Path {path} does not exist.")
+        with open(os.path.join(path, "config.json")) as f:
+            raw = json.load(f)
+        config = cls.config_cls.from_dict(raw, **kwargs)
+        base = config.base_model if (load_trimkv_weights and config.base_model) else path
+        if not os.path.isdir(base):
+            raise ValueError(f"base model {base!r} is not a local directory (nothing is downloaded here)")
+        config.base_model = base
+        model = cls(config)
+        state = _load_checkpoint_tensors(base)
+        if config.tie_word_embeddings and "lm_head.weight" not in state:
+            state["lm_head.weight"] = state["model.embed_tokens.weight"]
+        gate_keys = [k for k in model.state_dict() if any(t in k for t in config.trainable_params.split("|"))]
+        missing, unexpected = model.load_state_dict(state, strict=False)
+        not_gate = [k for k in missing if k not in gate_keys]
+        if not_gate:
+            raise ValueError(f"base checkpoint {base} lacks {not_gate[:4]}{' ...' if len(not_gate) > 4 else ''}")
+        if load_trimkv_weights:
+            gate_weights = torch.load(os.path.join(path, "trimkv_weights.pth"), map_location="cpu", weights_only=True)
+            if set(gate_keys) != set(gate_weights):
+                raise ValueError(f"Mismatch between trainable gate state keys: {gate_keys} and loaded weights keys: {list(gate_weights)}")
+            model.load_state_dict(gate_weights, strict=False)
+        if torch_dtype is not None:
+            model = model.to(torch_dtype)
+        return model.eval()
 
     def __init__(self, config: TrimKVQwen3Config):
         super().__init__()
