@@ -555,11 +555,14 @@ static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
         hipLaunchKernelGGL(prefill_small_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
         return 0;
     }
-    static bool lds_opted_in = false;   // > 64 KB of dynamic LDS needs the attribute once
-    if (!lds_opted_in) {
+    // > 64 KB of dynamic LDS needs the attribute once per device (the flag is only ever set, so a race repeats the call at worst)
+    static bool lds_opted_in[64] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+    if (dev < 0 || !lds_opted_in[dev]) {
         hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
         if (e != hipSuccess) return (int)e;
-        lds_opted_in = true;
+        if (dev >= 0) lds_opted_in[dev] = true;
     }
     const int bt = (PF2_WAVES * 32) / G;
     hipLaunchKernelGGL(prefill_attn_kernel, dim3((a.q_len + bt - 1) / bt, nseg), dim3(PF2_THREADS), PF2_LDS, st, a);

@@ -635,11 +635,15 @@ template <bool SELECT>
 static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st, int nlayers = 1) {
     const size_t key_bytes = (size_t)max_len * 4;
     if (key_bytes <= (size_t)EV_LDS_KEY_BYTES) {
-        static bool attr_set = false;
-        if (!attr_set) {  // allow more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per workgroup)
+        // allow more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per workgroup): once per device and
+        // instantiation; the flag is only ever set, so a race repeats the call at worst
+        static bool attr_set[64] = {};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
+        if (dev < 0 || !attr_set[dev]) {
             hipError_t e = hipFuncSetAttribute((const void*)evict_kernel<true, SELECT>, hipFuncAttributeMaxDynamicSharedMemorySize, EV_LDS_KEY_BYTES);
             if (e != hipSuccess) return fail((int)e, "%s: hipFuncSetAttribute: %s", fn, hipGetErrorString(e));
-            attr_set = true;
+            if (dev >= 0) attr_set[dev] = true;
         }
         hipLaunchKernelGGL((evict_kernel<true, SELECT>), dim3(a.nseg, nlayers), dim3(EV_THREADS), key_bytes, st, a);
     } else {
