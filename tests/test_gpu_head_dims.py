@@ -122,3 +122,20 @@ def test_other_head_dims_are_refused():
           "batch_size": 1, "num_kv_heads": 2}
     with pytest.raises(_lib.TrimKVLibraryError):
         attn(_Mod(), torch.zeros(1, 2, 1, D, dtype=torch.bfloat16, device=DEV), k, k, None, flash_attn_kwargs=kw)
+
+
+@pytest.mark.parametrize("G", [12, 16])
+def test_groups_wider_than_one_launch(G):
+    """More than 8 query heads per KV head: the group is attended in slices (K/V are read once per slice)."""
+    from trimkv_amd import get_attention_interface
+    attn = get_attention_interface("trimkv_hip")
+    gen = torch.Generator().manual_seed(G)
+    B, H, D, n = 2, 2, 128, 300
+    k, v = draw_kv(gen, B, H, n, D)
+    for Q in (1, 70):
+        q = torch.randn(B, Q, H * G, D, generator=gen).to(torch.bfloat16).transpose(1, 2)
+        out, _, _ = attn(_Mod(), q.to(DEV), k.to(DEV), v.to(DEV), None, scaling=D ** -0.5)
+        want, _ = eager_attention(q.float(), k.float(), v.float(), G, D ** -0.5, _bottom_right_mask(Q, n) if Q > 1 else None)
+        assert out.shape == (B, Q, H * G, D)
+        ok, err = attn_close(out, want)
+        assert ok, f"G={G} Q={Q}: max abs err {err}"

@@ -26,6 +26,12 @@ from torch import nn
 from .. import _lib
 
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
+_MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
+
+
+def _group_slice(group: int) -> int:
+    """Largest divisor of ``group`` that one launch takes."""
+    return max(g for g in range(1, _MAX_GROUP + 1) if group % g == 0)
 
 
 def _workspace(device, nbytes: int) -> Optional[torch.Tensor]:
@@ -46,6 +52,12 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
     ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only)."""
     if not query.is_cuda:
         raise _lib.TrimKVLibraryError("decode attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
+    if group > _MAX_GROUP:   # more query heads per KV head than one launch takes: several launches over slices of the group
+        g1 = _group_slice(group)
+        q3 = query.view(nseg, group, -1)
+        outs = [decode_attention(q3[:, a:a + g1].reshape(nseg * g1, -1), k_rows, v_rows, nseg, g1, seg_len, seg_start, cap, max_len,
+                                 scale, chunk, seg_order).view(nseg, g1, -1) for a in range(0, group, g1)]
+        return torch.cat(outs, dim=1).view(nseg * group, -1)
     lib = _lib.load()
     d = query.shape[-1]
     out = torch.empty_like(query)
@@ -67,6 +79,15 @@ def prefill_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.T
         raise _lib.TrimKVLibraryError("prefill attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
     lib = _lib.load()
     B, Hq, Q, D = query.shape
+    if group > _MAX_GROUP:
+        g1 = _group_slice(group)
+        q5 = query.reshape(B, kv_heads, group, Q, D)
+        out = torch.empty(B, Q, kv_heads, group, D, dtype=query.dtype, device=query.device)
+        for a in range(0, group, g1):
+            part = prefill_attention(q5[:, :, a:a + g1].reshape(B, kv_heads * g1, Q, D), k_rows, v_rows, batch, kv_heads, g1, seg_len,
+                                     seg_start, cap, max_len, scale)
+            out[:, :, :, a:a + g1] = part.view(B, Q, kv_heads, g1, D)
+        return out.view(B, Q, Hq, D)
     if query.stride(3) != 1 or any(s % 8 for s in query.stride()[:3]) or query.data_ptr() % 16:
         query = query.contiguous()
     out = torch.empty(B, Q, Hq, D, dtype=query.dtype, device=query.device)
