@@ -16,9 +16,11 @@
 //     packed bf16 pairs, and P.V is v_dot2_f32_bf16 over two rows at a time (v_perm_b32
 //     interleaves the rows);
 //   * the four wavefronts of a workgroup own disjoint quarters of the workgroup's rows and merge
-//     (max, sum, accumulator) in LDS; with 512 segments or more one workgroup covers a whole
-//     segment and writes the output itself, otherwise segments are split and a second, tiny
-//     kernel merges the partials.
+//     (max, sum, accumulator) in LDS; with 128 segments or more (or when the caller's chunk covers
+//     the longest segment) one workgroup covers a whole segment and writes the output itself,
+//     otherwise segments are split and a second, tiny kernel merges the partials;
+//   * rows of 96 or 64 features keep their length in memory: the 16-lane row group then has 12 or 8
+//     loading lanes, the others repeat the last piece against q = 0.
 #include "common.hip.h"
 
 #include <type_traits>

@@ -8,7 +8,7 @@
 //
 // Two kernels share the formulation below.  prefill_attn_kernel (chunks of 64 queries and more) gives
 // a wavefront 32 queries of one head and uses v_mfma_f32_32x32x16_bf16 on 64-key tiles that are
-// double-buffered in LDS, V stored transposed; prefill_small_kernel (short chunks) gives a wavefront
+// rotating through three LDS buffers, V stored transposed; prefill_small_kernel (short chunks) gives a wavefront
 // 16 queries and uses v_mfma_f32_16x16x32_bf16 on 32-key tiles.
 //
 // A workgroup owns BT consecutive query times of one segment for all G query heads of its KV head,
