@@ -176,6 +176,21 @@ int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* po
                            void* stream);
 
 /*
+ * trimkv_group_threshold_each_layer -- trimkv_group_threshold with one budget per (layer, group)
+ * instead of one per group across the layers: the layer-wise strategies of the flat caches
+ * (cache_utils.py:356-416, 719-834), every layer of one `compress` in one launch of
+ * ngroups x nlayers workgroups.  Same arguments; thr_key and tie_take are [nlayers][ngroups],
+ * tie_base and new_len [nlayers][nseg], ties counted inside each layer.
+ */
+int trimkv_group_threshold_each_layer(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+                                      const void* const* k_slabs, const int32_t* const* seg_lens,
+                                      int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
+                                      int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
+                                      int64_t q_idx, int strategy, int rounding,
+                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                      void* stream);
+
+/*
  * trimkv_group_threshold_wide -- the same selection with the same outputs, spread over one
  * workgroup per (layer, segment) instead of one per group: four histogram launches (one per key
  * byte), a count launch and a scan launch.  For large groups -- one sequence's budget over all

@@ -38,6 +38,8 @@ SIGNATURES = {
                           _p, _i, _p, _sz, _p]),
     "trimkv_group_threshold": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
                                     _p, _p, _p, _p, _p]),
+    "trimkv_group_threshold_each_layer": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
+                                    _p, _p, _p, _p, _p]),
     "trimkv_group_threshold_workspace": (_sz, [_i, _i, _i]),
     "trimkv_group_threshold_wide": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
                                          _p, _p, _p, _p, _p, _sz, _p]),

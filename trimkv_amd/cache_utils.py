@@ -659,6 +659,29 @@ class _RaggedCache(_SlabBacked):
         self._keepalive = (lb_t, pos_t, k_t, len_t)  # the launch reads these tables asynchronously
         return thr, take, tie_base, new_len
 
+    def _group_select_each(self, layers: List[int], segs_per_group: int, budget: int, strategy: str):
+        """One budget per (layer, group) -- the layer-wise strategies: every layer of ``layers`` (one shape and capacity)
+        in one ``trimkv_group_threshold_each_layer`` launch.
+        Returns (thr_key [L,groups], tie_take [L,groups], tie_base [L,nseg], new_len [L,nseg])."""
+        slabs = [self._slabs[l] for l in layers]
+        s0 = slabs[0]
+        dev = s0.k.device
+        L, nseg = len(slabs), s0.nseg
+        ngroups = nseg // segs_per_group
+        thr = torch.empty(L, ngroups, dtype=torch.int32, device=dev)
+        take = torch.empty(L, ngroups, dtype=torch.int32, device=dev)
+        tie_base = torch.empty(L, nseg, dtype=torch.int32, device=dev)
+        new_len = torch.empty(L, nseg, dtype=torch.int32, device=dev)
+        tables = [self._ptr_table([getattr(s, name) for s in slabs], dev) for name in ("lb", "pos", "k", "seg_len")]
+        rc = _lib.load().trimkv_group_threshold_each_layer(
+            tables[0].data_ptr(), tables[1].data_ptr(), tables[2].data_ptr(), tables[3].data_ptr(), L, nseg, segs_per_group, s0.cap, s0.D,
+            _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype), int(budget), 0, 0.0, self.get_seq_length() + 1,
+            self._strategy_code(strategy), _lib.ROUND_NATIVE, thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(),
+            _lib.current_stream(dev))
+        _lib.check(rc, "trimkv_group_threshold_each_layer")
+        self._keepalive = tuple(tables)  # the launch reads these tables asynchronously
+        return thr, take, tie_base, new_len
+
     def _compact(self, layer: int, segs_per_group: int, thr, take, tie_base_l, strategy: str) -> None:
         slab = self._slabs[layer]
         lib = _lib.load()
@@ -671,10 +694,12 @@ class _RaggedCache(_SlabBacked):
         _lib.check(rc, "trimkv_compact_threshold")
 
     def _compact_layers(self, layers: List[int], segs_per_group: int, thr, take, tie_base, strategy: str) -> None:
-        """One budget across ``layers``: every layer compacted against the same group thresholds, in one launch."""
+        """Every layer of ``layers`` compacted in one launch: against the same group thresholds (``thr`` [groups], one
+        budget across the layers) or against its own row of ``thr`` [L, groups] (layer-wise budgets)."""
+        per_layer = thr.dim() == 2
         if len(layers) == 1 or not self._layers_alike(layers):
             for i, l in enumerate(layers):
-                self._compact(l, segs_per_group, thr, take, tie_base[i], strategy)
+                self._compact(l, segs_per_group, thr[i] if per_layer else thr, take[i] if per_layer else take, tie_base[i], strategy)
             return
         s0 = self._slabs[layers[0]]
         dev = s0.k.device
@@ -685,7 +710,7 @@ class _RaggedCache(_SlabBacked):
         ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
         rc = lib.trimkv_compact_threshold_layers(table.data_ptr(), len(layers), s0.nseg, segs_per_group, s0.D,
                                                  _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
-                                                 thr.data_ptr(), take.data_ptr(), 0, tie_base.data_ptr(),
+                                                 thr.data_ptr(), take.data_ptr(), thr.shape[1] if per_layer else 0, tie_base.data_ptr(),
                                                  self._strategy_code(strategy), _lib.ROUND_NATIVE, max_len,
                                                  _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
         _lib.check(rc, "trimkv_compact_threshold_layers")
@@ -818,18 +843,25 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             if base not in ("alpha", "knorm_alpha"):
                 raise ValueError(f"Unknown compression strategy: {base}")
             todo = [l for l in range(num_layers) if self._layer_tokens(l) > B * H * (memory_size + buffer_size)]
-            for l in todo:
+            if not todo:
+                return
+            alike = self._layers_alike(todo) and len({self._slabs[l].cap for l in todo}) == 1
+            for part in ([todo] if alike else [[l] for l in todo]):   # layers of one shape go through together
                 if floor_budget_ratio > 0:
                     budget = int(memory_size * H * (1 - floor_budget_ratio))
-                    _, _, _, new_len = self._group_select([l], H, budget, base)
-                    chosen = new_len[0].cpu().numpy().astype(np.int64)
+                    _, _, _, new_len = self._group_select_each(part, H, budget, base)
+                    chosen = new_len.cpu().numpy().astype(np.int64)
                     floor_per_head = int(memory_size * floor_budget_ratio)
                     # top-up (:789-806): a head keeps its best max(chosen, floor) tokens, at most all of them
-                    keep = np.minimum(np.maximum(chosen, floor_per_head), self._slabs[l].lens)
-                    self._evict_per_segment(l, keep, base)
+                    keep = np.minimum(np.maximum(chosen, floor_per_head), np.stack([self._slabs[l].lens for l in part]))
+                    if len(part) > 1:
+                        q = self.get_seq_length() + 1
+                        self._evict_layers(part, 0, keep, 0, self._strategy_code(base), _lib.ROUND_NATIVE, 0, lambda l: q)
+                    else:
+                        self._evict_per_segment(part[0], keep[0], base)
                 else:
-                    thr, take, tie_base, _ = self._group_select([l], H, memory_size * H, base)
-                    self._compact(l, H, thr, take, tie_base[0], base)
+                    thr, take, tie_base, _ = self._group_select_each(part, H, memory_size * H, base)
+                    self._compact_layers(part, H, thr, take, tie_base, base)
             self._refresh(todo)
         else:  # cache_utils.py:836-945; floor_budget_ratio is not used by this variant
             tokens_per_batch = sum(self._layer_tokens(l) for l in range(num_layers)) // B
@@ -879,10 +911,12 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             todo = [l for l in range(num_layers) if not H * (memory_size + buffer_size) >= self._layer_tokens(l)]
             if todo and base not in ("alpha", "knorm_alpha"):
                 raise ValueError(f"Unknown compression strategy: {base}")
-            for l in todo:
-                thr, take, tie_base, _ = self._group_select([l], H, H * memory_size, base)
-                self._compact(l, H, thr, take, tie_base[0], base)
-            self._refresh(todo)
+            if todo:
+                alike = self._layers_alike(todo) and len({self._slabs[l].cap for l in todo}) == 1
+                for part in ([todo] if alike else [[l] for l in todo]):
+                    thr, take, tie_base, _ = self._group_select_each(part, H, H * memory_size, base)
+                    self._compact_layers(part, H, thr, take, tie_base, base)
+                self._refresh(todo)
             return
         # all layers at once, cache_utils.py:418-536
         total_budget = num_layers * H * memory_size

@@ -324,6 +324,7 @@ struct GroupArgs {
     int64_t budget; int use_threshold; float threshold_score;
     int64_t q_idx; int strategy, rounding;
     uint32_t* thr_key; int32_t* tie_take; int32_t* tie_base; int32_t* new_len;
+    int per_layer;   // one budget per (layer, group): blockIdx.y = layer, results are [nlayers][groups]
 };
 
 __device__ __forceinline__ ScoreArgs group_segment(const GroupArgs& a, int layer, int seg) {
@@ -352,6 +353,14 @@ __global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a
     __shared__ unsigned long long hist[256];
     __shared__ uint64_t red[GT_THREADS / 64];
     __shared__ unsigned long long sel[2];
+    if (a.per_layer) {   // this workgroup's layer stands alone: step every table and result to it
+        const int layer = blockIdx.y;
+        a.lb_slabs += layer; a.pos_slabs += layer; a.seg_lens += layer;
+        if (a.k_slabs) a.k_slabs += layer;
+        a.thr_key += (int64_t)layer * gridDim.x; a.tie_take += (int64_t)layer * gridDim.x;
+        a.tie_base += (int64_t)layer * a.nseg; a.new_len += (int64_t)layer * a.nseg;
+        a.nlayers = 1;
+    }
     const int g = blockIdx.x;
     const int seg0 = g * a.segs_per_group;
 
@@ -779,14 +788,13 @@ extern "C" int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers,
     return launch_evict<false>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream, nlayers);
 }
 
-extern "C" int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
+static int group_threshold_common(const char* fn, int per_layer, const void* const* lb_slabs, const int64_t* const* pos_slabs,
                                       const void* const* k_slabs, const int32_t* const* seg_lens,
                                       int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                                       int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                                       int64_t q_idx, int strategy, int rounding,
                                       uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
                                       void* stream) {
-    const char* fn = "trimkv_group_threshold";
     if (!lb_slabs || !pos_slabs || !seg_lens || !thr_key || !tie_take || !tie_base || !new_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (strategy == TRIMKV_SCORE_KNORM_ALPHA && !k_slabs) return fail(TRIMKV_ERR_NULL, "%s: knorm_alpha needs k_slabs", fn);
     if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
@@ -798,9 +806,24 @@ extern "C" int trimkv_group_threshold(const void* const* lb_slabs, const int64_t
     a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
     a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
     a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
-    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len;
-    hipLaunchKernelGGL(group_threshold_kernel, dim3(nseg / segs_per_group), dim3(GT_THREADS), 0, (hipStream_t)stream, a);
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.per_layer = per_layer;
+    if (per_layer && nlayers > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nlayers=%d exceeds the grid limit 65535", fn, nlayers);
+    hipLaunchKernelGGL(group_threshold_kernel, dim3(nseg / segs_per_group, per_layer ? nlayers : 1), dim3(GT_THREADS), 0, (hipStream_t)stream, a);
     return launch_status(fn);
+}
+
+
+#define TRIMKV_GROUP_PARAMS const void* const* lb_slabs, const int64_t* const* pos_slabs, const void* const* k_slabs, \
+    const int32_t* const* seg_lens, int nlayers, int nseg, int segs_per_group, int cap, int head_dim, int kv_dtype, int lb_dtype, \
+    int64_t budget, int use_threshold, float threshold_score, int64_t q_idx, int strategy, int rounding, \
+    uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, void* stream
+#define TRIMKV_GROUP_ARGS lb_slabs, pos_slabs, k_slabs, seg_lens, nlayers, nseg, segs_per_group, cap, head_dim, kv_dtype, lb_dtype, budget, \
+    use_threshold, threshold_score, q_idx, strategy, rounding, thr_key, tie_take, tie_base, new_len, stream
+
+extern "C" int trimkv_group_threshold(TRIMKV_GROUP_PARAMS) { return group_threshold_common("trimkv_group_threshold", 0, TRIMKV_GROUP_ARGS); }
+
+extern "C" int trimkv_group_threshold_each_layer(TRIMKV_GROUP_PARAMS) {
+    return group_threshold_common("trimkv_group_threshold_each_layer", 1, TRIMKV_GROUP_ARGS);
 }
 
 extern "C" size_t trimkv_group_threshold_workspace(int nlayers, int nseg, int segs_per_group) {
@@ -833,7 +856,7 @@ extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const in
     a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
     a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
     a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
-    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.per_layer = 0;
     w.hist = (uint32_t*)workspace;
     w.cnt = w.hist + (size_t)ngroups * 4 * 256;
     hipStream_t st = (hipStream_t)stream;
