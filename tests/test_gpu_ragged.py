@@ -365,3 +365,23 @@ def test_wide_group_threshold_equals_the_single_workgroup_selection(nlayers, B, 
     if threshold is None:
         want = np.minimum(budget, lens.reshape(nlayers, B, H).sum(axis=(0, 2)))
         assert (nl.reshape(nlayers, B, H).sum(axis=(0, 2)) == want).all()      # every group keeps exactly its budget
+
+
+@pytest.mark.parametrize("strategy", ["alpha", "layer_wise_alpha"])
+def test_layers_of_different_capacity_share_a_budget(strategy):
+    """Layers grow their slabs on their own (after a shared-budget eviction their longest segments differ), so a later
+    cross-layer selection meets layers of different row capacity; it must still select exactly what the oracle selects."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache
+    B, H, L, M, buf = 2, 3, 3, 40, 4
+    d = _Driver(BatchedDynamicBudgetTrimKVCache(), BatchedRaggedCacheRef(), B, H, L, seed=23)
+    d.append(70)
+    kw = dict(strategy=strategy, memory_size=M, buffer_size=buf, num_layers=L, num_key_value_heads=H)
+    d.ref.compress(**kw); d.cache.compress(**kw)
+    _same(d.cache, d.ref)
+    d.cache._slabs[1].regrow(d.cache._slabs[1].cap + 64)       # what an uneven append history does to one layer
+    assert len({s.cap for s in d.cache._slabs}) > 1
+    d.append(9)
+    snap = _snapshot(d.ref, strategy)
+    d.ref.compress(**kw); d.cache.compress(**kw)
+    _assert_no_tie_at_a_cut(snap, d.ref)
+    _same(d.cache, d.ref)

@@ -623,6 +623,15 @@ class _RaggedCache(_SlabBacked):
     def _ptr_table(self, tensors: List[torch.Tensor], device) -> torch.Tensor:
         return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64).to(device)
 
+    @staticmethod
+    def _equalise_capacity(slabs: List[_Slab]) -> None:
+        """The cross-layer selection kernels address every layer with one row capacity.  Layers grow on their own (their
+        longest segments differ once a shared budget has been applied), so bring them to the largest capacity first."""
+        cap = max(s.cap for s in slabs)
+        for s in slabs:
+            if s.cap != cap:
+                s.regrow(cap)
+
     def _group_select(self, layers: List[int], segs_per_group: int, budget: int, strategy: str,
                       threshold: Optional[float] = None):
         """Run ``trimkv_group_threshold`` over ``layers`` (all of one shape); returns the device
@@ -630,8 +639,9 @@ class _RaggedCache(_SlabBacked):
         slabs = [self._slabs[l] for l in layers]
         s0 = slabs[0]
         for s in slabs:
-            if (s.nseg, s.cap, s.D, s.k.dtype, s.lb.dtype) != (s0.nseg, s0.cap, s0.D, s0.k.dtype, s0.lb.dtype):
-                raise _lib.TrimKVLibraryError("cross-layer selection needs layers of one shape and capacity")
+            if (s.nseg, s.D, s.k.dtype, s.lb.dtype) != (s0.nseg, s0.D, s0.k.dtype, s0.lb.dtype):
+                raise _lib.TrimKVLibraryError("cross-layer selection needs layers of one shape")
+        self._equalise_capacity(slabs)
         dev = s0.k.device
         L = len(slabs)
         ngroups = s0.nseg // segs_per_group
@@ -664,6 +674,7 @@ class _RaggedCache(_SlabBacked):
         in one ``trimkv_group_threshold_each_layer`` launch.
         Returns (thr_key [L,groups], tie_take [L,groups], tie_base [L,nseg], new_len [L,nseg])."""
         slabs = [self._slabs[l] for l in layers]
+        self._equalise_capacity(slabs)
         s0 = slabs[0]
         dev = s0.k.device
         L, nseg = len(slabs), s0.nseg
@@ -845,7 +856,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             todo = [l for l in range(num_layers) if self._layer_tokens(l) > B * H * (memory_size + buffer_size)]
             if not todo:
                 return
-            alike = self._layers_alike(todo) and len({self._slabs[l].cap for l in todo}) == 1
+            alike = self._layers_alike(todo)
             for part in ([todo] if alike else [[l] for l in todo]):   # layers of one shape go through together
                 if floor_budget_ratio > 0:
                     budget = int(memory_size * H * (1 - floor_budget_ratio))
@@ -912,7 +923,7 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             if todo and base not in ("alpha", "knorm_alpha"):
                 raise ValueError(f"Unknown compression strategy: {base}")
             if todo:
-                alike = self._layers_alike(todo) and len({self._slabs[l].cap for l in todo}) == 1
+                alike = self._layers_alike(todo)
                 for part in ([todo] if alike else [[l] for l in todo]):
                     thr, take, tie_base, _ = self._group_select_each(part, H, H * memory_size, base)
                     self._compact_layers(part, H, thr, take, tie_base, base)
