@@ -122,3 +122,38 @@ def test_random_walk_ragged_matches_oracle(seed):
             if any(cache.head_lens[l].cpu().tolist() != ref.head_lens[l].tolist() for l in range(L)):
                 return
         _same(cache, ref)
+
+
+@pytest.mark.parametrize("seed", list(range(16)))
+def test_random_walk_single_sequence_matches_oracle(seed):
+    """Batch-1 ragged cache: shared budget over all layers, layer-wise, score threshold, and the floor branch."""
+    from oracle.ragged_ref import SingleRaggedCacheRef
+    from tests.test_gpu_ragged import _same, _snapshot
+    from trimkv_amd import DynamicBudgetTrimKVCache
+    rng = np.random.default_rng(9000 + seed)
+    H, L = int(rng.integers(1, 6)), int(rng.integers(1, 5))
+    D = int(rng.choice([64, 128]))
+    M, buf = int(rng.integers(6, 100)), int(rng.choice([0, 3, 16]))
+    strategy, floor = [("alpha", 0.0), ("layer_wise_alpha", 0.0), ("alpha_threshold", 0.0), ("alpha", 0.25), ("alpha", 0.5)][int(rng.integers(0, 5))]
+    thr = float(rng.uniform(0.3, 0.95))
+    gen = torch.Generator().manual_seed(seed)
+    cache, ref = DynamicBudgetTrimKVCache(), SingleRaggedCacheRef()
+    T = 0
+    for S in [int(rng.choice([1, 1, 2, 7, 33, 90])) for _ in range(int(rng.integers(5, 18)))]:
+        pos = torch.arange(T, T + S)
+        for l in range(L):
+            k, v = draw_kv(gen, 1, H, S, D)
+            lb = draw_log_beta(gen, 1, H, S, sigma=1.5)
+            ref.update(k, v, lb, pos, l)
+            cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), l)
+        T += S
+        snap = _snapshot(ref, strategy)
+        kw = dict(strategy=strategy, memory_size=M, buffer_size=buf, floor_budget_ratio=floor, alpha_threshold=thr,
+                  num_layers=L, num_key_value_heads=H)
+        ref.compress(**kw)
+        cache.compress(**kw)
+        scores = torch.cat([s for s, _, _ in snap])
+        if scores.unique().numel() != scores.numel():     # equal scores may straddle a cut: selection undefined from here on
+            if any(cache.head_lens[l].cpu().tolist() != ref.head_lens[l].tolist() for l in range(L)):
+                return
+        _same(cache, ref)
