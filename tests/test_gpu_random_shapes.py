@@ -157,3 +157,33 @@ def test_random_walk_single_sequence_matches_oracle(seed):
             if any(cache.head_lens[l].cpu().tolist() != ref.head_lens[l].tolist() for l in range(L)):
                 return
         _same(cache, ref)
+
+
+@pytest.mark.parametrize("seed", list(range(40)))
+def test_random_ragged_attention_shapes(seed):
+    """Packed ragged K/V with random segment lengths (some empty or shorter than the query block), group sizes, head dims
+    and query-block lengths straddling the kernels' tile sizes, against the fp32 oracle."""
+    from oracle.attn_ref import ragged_attention
+    from trimkv_amd import get_attention_interface
+    attn = get_attention_interface("db_attn_flash_batched")
+    rng = np.random.default_rng(seed)
+    B, H = int(rng.integers(1, 4)), int(rng.integers(1, 5))
+    G, D = int(rng.integers(1, 9)), int(rng.choice([64, 96, 128, 128]))
+    Q = int(rng.choice([1, 1, 2, 3, 15, 16, 17, 63, 64, 65, 100, 256, 300]))
+    nseg = B * H
+    lens = rng.integers(0, 2500, size=nseg)
+    lens[rng.random(nseg) < 0.15] = rng.integers(0, 4)
+    if rng.random() < 0.2:
+        lens[:] = int(rng.integers(Q, 3000))
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    tot = int(cu[-1])
+    gen = torch.Generator().manual_seed(seed)
+    K = torch.randn(max(tot, 1), D, generator=gen).to(torch.bfloat16)
+    V = torch.randn(max(tot, 1), D, generator=gen).to(torch.bfloat16)
+    q = torch.randn(B, H * G, Q, D, generator=gen).to(torch.bfloat16) * float(rng.choice([1.0, 1.0, 3.0]))
+    kw = {"head_lens": torch.from_numpy(lens.astype(np.int32)).to(DEV), "cu_seqlens_k": torch.from_numpy(cu).to(DEV),
+          "batch_size": B, "num_kv_heads": H}
+    out, _, _ = attn(_Mod(), q.to(DEV), K.to(DEV), V.to(DEV), None, flash_attn_kwargs=kw)
+    want = ragged_attention(q, K[:tot], V[:tot], torch.from_numpy(cu), H)
+    ok, err = attn_close(out, want)
+    assert ok and torch.isfinite(out.float()).all(), f"seed {seed} (B={B} H={H} G={G} D={D} Q={Q}): max abs err {err}"
