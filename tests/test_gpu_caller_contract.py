@@ -130,3 +130,40 @@ def test_attention_block_call_order(kind):
                 for seg in range(B * HKV):
                     assert got[l][seg].tolist() == want_pos[l][seg].tolist(), f"layer {l} segment {seg}"
     assert evictions >= 4 and cache.get_seq_length() == T == 88
+
+
+def test_cache_follows_the_callers_current_stream():
+    """Everything is enqueued on torch's current stream: the same decode steps on a side stream (with the producer of the
+    inputs on that stream too) give the same state and outputs as on the default stream."""
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    attn = get_attention_interface("trimkv_hip")
+
+    class Mod:
+        training = False
+
+    def run(stream):
+        gen = torch.Generator(device=DEV).manual_seed(3)
+        cache, outs = TrimKVCache(), []
+        with torch.cuda.stream(stream):
+            T = 0
+            for S in (200, 1, 1, 1, 1, 1):
+                for l in range(2):
+                    k = torch.randn(2, 4, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+                    v = torch.randn(2, 4, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+                    lb = -torch.rand(2, 4, S, generator=gen, device=DEV) - 0.01
+                    q = torch.randn(2, 16, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+                    K, V, _, _, kw = cache.update(k, v, lb, torch.arange(T, T + S, device=DEV), l)
+                    outs.append(attn(Mod(), q, K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)[0])
+                T += S
+                cache.compress("alpha", 128, 3)
+        stream.synchronize()
+        return cache, outs
+
+    c0, o0 = run(torch.cuda.current_stream())
+    c1, o1 = run(torch.cuda.Stream())
+    torch.cuda.synchronize()
+    assert c1.get_cache_length(0) == c0.get_cache_length(0) < 205      # evictions ran on both
+    for a, b in zip(o0, o1):
+        assert torch.equal(a, b)
+    for l in range(2):
+        assert torch.equal(c0.kv_positions[l], c1.kv_positions[l]) and torch.equal(c0.key_cache[l], c1.key_cache[l])
