@@ -784,25 +784,37 @@ class _RaggedCache(_SlabBacked):
         layers = [l for l in range(len(self._slabs)) if self._slabs[l] is not None] if layers is None else layers
         lib = _lib.load()
         code = self._strategy_code(strategy)
+        due = []
         for l in layers:
             slab = self._slabs[l]
             kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[l]
             hit = (slab.lens > kh) & (slab.lens >= kh + buffer_size)
-            if not hit.any():
-                continue
-            key = (l if self._budgets_host.ndim == 2 else -1, str(slab.k.device))
-            keep = self._budgets_dev.get(key)
-            if keep is None:
-                keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(slab.k.device)
-                self._budgets_dev[key] = keep
-            st = _lib.current_stream(slab.k.device)
-            ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
-            rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
-                                  slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
-                                  0, keep.data_ptr(), buffer_size, self.get_seq_length() + 1, code, _lib.ROUND_NATIVE,
-                                  0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(), st)
-            _lib.check(rc, "trimkv_evict")
-            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), st)
+            if hit.any():
+                due.append((l, kh, hit))
+        if not due:
+            return
+        if len(due) > 1 and self._layers_alike([l for l, _, _ in due]):   # the layers that are due: one launch
+            q = self.get_seq_length() + 1
+            self._evict_layers([l for l, _, _ in due], 0, np.stack([kh for _, kh, _ in due]), buffer_size, code, _lib.ROUND_NATIVE, 0,
+                               lambda l: q)
+        else:
+            for l, kh, _ in due:
+                slab = self._slabs[l]
+                key = (l if self._budgets_host.ndim == 2 else -1, str(slab.k.device))
+                keep = self._budgets_dev.get(key)
+                if keep is None:
+                    keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(slab.k.device)
+                    self._budgets_dev[key] = keep
+                ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
+                rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                                      slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                                      0, keep.data_ptr(), buffer_size, self.get_seq_length() + 1, code, _lib.ROUND_NATIVE,
+                                      0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(),
+                                      _lib.current_stream(slab.k.device))
+                _lib.check(rc, "trimkv_evict")
+        for l, kh, hit in due:
+            slab = self._slabs[l]
+            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
             _lib.check(rc, "trimkv_build_cu_seqlens")
             slab.lens = np.where(hit, kh, slab.lens)
             slab.max_len = int(slab.lens.max())
