@@ -294,7 +294,7 @@ int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlen
  * that the long segments do not form the tail of the launch (about 15 % at lognormal lengths).  It
  * changes scheduling only; entries are clamped to [0, nseg).
  * head_dim must be 128, 96 or 64 (the kernel is laid out for 128; shorter rows run zero-padded to
- * it); group in [1, 8]; dtype bf16.
+ * it); group in [1, 8]; dtype bf16 or fp16 (q, K, V and out alike).
  */
 size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim, int max_len, int chunk);
 int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
@@ -315,7 +315,7 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
  * contiguous, strides multiples of 8); out is [batch][q_len][kv_heads*group][head_dim],
  * contiguous.  Segment batch b, kv head h is attended by query heads h*group .. h*group+group-1
  * (flash_attn.py:120-125).  K/V rows as in trimkv_decode_attn (seg_start or seg*cap; seg_len may be
- * NULL for a dense cache of max_len rows).  head_dim must be 128, 96 or 64; group in [1, 8]; dtype bf16.
+ * NULL for a dense cache of max_len rows).  head_dim must be 128, 96 or 64; group in [1, 8]; dtype bf16 or fp16.
  */
 int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_stride_h, int64_t q_stride_t, void* out,
                         const void* k_slab, const void* v_slab, const int32_t* seg_len, const int32_t* seg_start,

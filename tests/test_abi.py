@@ -56,7 +56,7 @@ def test_bad_arguments_are_refused_without_a_launch():
         a = dict(base); a.update(kw)
         return lib.trimkv_decode_attn(one, one, one, one, one, None, None, a["nseg"], a["cap"], a["D"], a["G"], a["dt"], 0.1,
                                       a["max_len"], a["chunk"], None, 0, None)
-    assert attn(D=80) == -6 and attn(D=256) == -6 and attn(G=9) == -6 and attn(dt=_lib.F16) == -3
+    assert attn(D=80) == -6 and attn(D=256) == -6 and attn(G=9) == -6 and attn(dt=_lib.F32) == -3
     assert attn(max_len=128) == -4            # longer than the slab
     assert attn(cap=4096, max_len=4096, chunk=256) == -5  # split-K needs a workspace
     assert attn(chunk=100) == -2

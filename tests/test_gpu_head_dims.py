@@ -139,3 +139,42 @@ def test_groups_wider_than_one_launch(G):
         assert out.shape == (B, Q, H * G, D)
         ok, err = attn_close(out, want)
         assert ok, f"G={G} Q={Q}: max abs err {err}"
+
+
+@pytest.mark.parametrize("D,G", [(128, 4), (96, 1), (64, 5)])
+def test_fp16_cache_and_attention(D, G):
+    """fp16 K/V/q: the same kernels with the fp16 dot and matrix instructions; prompt chunk (short and long kernels), decode
+    (direct and split-K), eviction -- state bit-exact, attention within the tolerance of the fp32 oracle."""
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    attn = get_attention_interface("trimkv_hip")
+    gen = torch.Generator().manual_seed(7 * D + G)
+    B, H, M, buf = 2, 2, 300, 20
+    cache, ref = TrimKVCache(), DenseCacheRef()
+    T = 0
+    for S in (200, 30, 1, 1, 130, 1, 1):
+        k, v = draw_kv(gen, B, H, S, D, dtype=torch.float16)
+        lb = draw_log_beta(gen, B, H, S, sigma=1.5)
+        q = torch.randn(B, H * G, S, D, generator=gen).to(torch.float16)
+        pos = torch.arange(T, T + S)
+        rk, rv, _, _, _ = ref.update(k, v, lb, pos, 0)
+        K, V, _, _, kw = cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), 0)
+        out, _, _ = attn(_Mod(), q.to(DEV), K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+        n = rk.shape[2]
+        want, _ = eager_attention(q.float(), rk.float(), rv.float(), G, D ** -0.5, _bottom_right_mask(S, n) if S > 1 else None)
+        assert out.dtype == torch.float16 and out.shape == (B, S, H * G, D)
+        ok, err = attn_close(out, want)
+        assert ok, f"S={S} n={n}: max abs err {err}"
+        T += S
+        ref.compress("alpha", M, buf)
+        cache.compress("alpha", M, buf)
+        kk, vv, ll, pp = cache[0]
+        assert kk.dtype == torch.float16 and torch.equal(pp.cpu(), ref.kv_positions[0]) and torch.equal(kk.cpu(), ref.key_cache[0])
+    # a long segment: split-K decode and the 32x32 MFMA chunk kernel
+    n = 3000
+    k, v = draw_kv(gen, 1, 2, n, D, dtype=torch.float16)
+    for Q in (1, 256):
+        q = torch.randn(1, 2 * G, Q, D, generator=gen).to(torch.float16)
+        out, _, _ = attn(_Mod(), q.to(DEV), k.to(DEV), v.to(DEV), None, scaling=D ** -0.5)
+        want, _ = eager_attention(q.float(), k.float(), v.float(), G, D ** -0.5, _bottom_right_mask(Q, n) if Q > 1 else None)
+        ok, err = attn_close(out, want)
+        assert ok, f"Q={Q}: max abs err {err}"

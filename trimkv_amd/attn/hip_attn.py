@@ -127,7 +127,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             seg_len = None
         out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale)
         return out.view(B, 1, Hq, D), None, None
-    if attention_mask is None and query.dtype == torch.bfloat16 and D in (64, 96, 128):
+    if attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
               and value.stride() == key.stride() and key.stride(1) % D == 0)
         if not ok:

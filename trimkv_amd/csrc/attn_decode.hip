@@ -60,9 +60,15 @@ constexpr int DPP_QUAD_XOR2 = 0x4E;       // quad_perm [2,3,0,1]
 constexpr int DPP_ROW_HALF_MIRROR = 0x141;
 constexpr int DPP_ROW_ROR8 = 0x128;
 
-__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float c) {
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+// c + a.lo * b.lo + a.hi * b.hi on packed bf16 (v_dot2_f32_bf16) or fp16 (v_dot2_f32_f16) pairs
+template <bool F16>
+__device__ __forceinline__ float dot2_kv(uint32_t a, uint32_t b, float c) {
+    if constexpr (F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+    else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
 }
+template <bool F16>
+__device__ __forceinline__ uint16_t to_kv_bits(float f) { return F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f); }
 
 // Sum 16 per-lane values over the 16 lanes of a row group, leaving value x(c) in lane c, where
 // x(c) = bit2(c)<<3 | bit0(c)<<2 | bit1(c)<<1 | bit3(c).  Each step halves the values a lane
@@ -101,7 +107,7 @@ struct AttnArgs {
 // slot `slot` of the workspace.  All 256 threads of the workgroup must call it together (it uses barriers).
 // ROW16: 16-byte pieces per K/V/q row (head_dim / 8).  With fewer than 16, lanes c >= ROW16 of each 16-lane row group
 // re-read the row's last piece and hold q = 0, so they add nothing to the scores; what they accumulate is not stored.
-template <int G, int ROW16>
+template <int G, int ROW16, bool F16>
 __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base) {
     constexpr int D_REAL = ROW16 * 8;
     using C = AttnCfg<G>;
@@ -182,10 +188,10 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             for (int j = 0; j < NJ; ++j) {
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    float acc = dot2_bf16(kt[j].x, qv[g].x, 0.0f);
-                    acc = dot2_bf16(kt[j].y, qv[g].y, acc);
-                    acc = dot2_bf16(kt[j].z, qv[g].z, acc);
-                    acc = dot2_bf16(kt[j].w, qv[g].w, acc);
+                    float acc = dot2_kv<F16>(kt[j].x, qv[g].x, 0.0f);
+                    acc = dot2_kv<F16>(kt[j].y, qv[g].y, acc);
+                    acc = dot2_kv<F16>(kt[j].z, qv[g].z, acc);
+                    acc = dot2_kv<F16>(kt[j].w, qv[g].w, acc);
                     part[j * G + g] = acc;
                 }
             }
@@ -218,7 +224,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
                 if (t * TILE_ROWS < nrows) {
                     const float p = my_valid ? __builtin_amdgcn_exp2f(s[t] - m_mine) : 0.0f;
                     l_lane += p;
-                    if (my_valid) pw16[(t * 4 + r) * PS + my_g * NJ + my_j] = f32_to_bf16_bits(p);
+                    if (my_valid) pw16[(t * 4 + r) * PS + my_g * NJ + my_j] = to_kv_bits<F16>(p);
                 }
             }
         };
@@ -238,8 +244,8 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
 #pragma unroll
                     for (int g = 0; g < G; ++g) {
                         const uint32_t pp = pd[(g * NJ) / 2 + u];
-                        o[g][2 * i] = dot2_bf16(lo, pp, o[g][2 * i]);
-                        o[g][2 * i + 1] = dot2_bf16(hi, pp, o[g][2 * i + 1]);
+                        o[g][2 * i] = dot2_kv<F16>(lo, pp, o[g][2 * i]);
+                        o[g][2 * i + 1] = dot2_kv<F16>(hi, pp, o[g][2 * i + 1]);
                     }
                 }
             }
@@ -344,7 +350,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         }
         if (direct) {
             const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = f32_to_bf16_bits(y);
+            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = to_kv_bits<F16>(y);
         } else {
             const int64_t slot = slot_base * G + g;
             a.ws_o[slot * AT_D + d] = acc;
@@ -353,7 +359,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     }
 }
 
-template <int G, int ROW16>
+template <int G, int ROW16, bool F16>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2))) void decode_attn_kernel(AttnArgs a) {
     // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
     // axis so that consecutive ids are different segments: with the split as the fast axis and 8
@@ -377,7 +383,7 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
     }
     const int rps = (n + nsp - 1) / nsp;
     const int t0 = split * rps, t1 = min(n, t0 + rps);
-    attend_rows<G, ROW16>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split);
+    attend_rows<G, ROW16, F16>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split);
 }
 
 // Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
@@ -385,7 +391,7 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 // kernel boundary is what makes partials written on one XCD visible on another; doing the same
 // inside one kernel needs device-scope fences (an L2 write-back and invalidate per workgroup on
 // this part), which costs far more than the launch.
-template <int G, int ROW16>
+template <int G, int ROW16, bool F16>
 __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
     const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
@@ -419,7 +425,7 @@ __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a)
         lsum += f * a.ws_ml[slot * 2 + 1];
     }
     const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-    if (d < ROW16 * 8) ((uint16_t*)a.out)[((int64_t)seg * G + g) * (ROW16 * 8) + d] = f32_to_bf16_bits(y);
+    if (d < ROW16 * 8) ((uint16_t*)a.out)[((int64_t)seg * G + g) * (ROW16 * 8) + d] = to_kv_bits<F16>(y);
 }
 
 static int pick_chunk(int nseg, int max_len) {
@@ -435,17 +441,23 @@ static int pick_chunk(int nseg, int max_len) {
     return chunk < whole ? chunk : whole;
 }
 
-template <int G, int ROW16>
+template <int G, int ROW16, bool F16>
 static void launch_attn_rows(const AttnArgs& a, hipStream_t st) {
-    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
-    if (!a.direct) hipLaunchKernelGGL((decode_attn_merge_kernel<G, ROW16>), dim3(a.nseg), dim3(G * AT_D), 0, st, a);
+    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16, F16>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
+    if (!a.direct) hipLaunchKernelGGL((decode_attn_merge_kernel<G, ROW16, F16>), dim3(a.nseg), dim3(G * AT_D), 0, st, a);
+}
+
+template <int G, bool F16>
+static void launch_attn_dtype(const AttnArgs& a, int head_dim, hipStream_t st) {
+    if (head_dim == 128) launch_attn_rows<G, 16, F16>(a, st);
+    else if (head_dim == 96) launch_attn_rows<G, 12, F16>(a, st);
+    else launch_attn_rows<G, 8, F16>(a, st);
 }
 
 template <int G>
-static void launch_attn(const AttnArgs& a, int head_dim, hipStream_t st) {
-    if (head_dim == 128) launch_attn_rows<G, 16>(a, st);
-    else if (head_dim == 96) launch_attn_rows<G, 12>(a, st);
-    else launch_attn_rows<G, 8>(a, st);
+static void launch_attn(const AttnArgs& a, int head_dim, int dtype, hipStream_t st) {
+    if (dtype == TRIMKV_F16) launch_attn_dtype<G, true>(a, head_dim, st);
+    else launch_attn_dtype<G, false>(a, head_dim, st);
 }
 
 }  // namespace trimkv
@@ -466,7 +478,7 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
                                   int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_decode_attn";
     if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
-    if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
+    if (dtype != TRIMKV_BF16 && dtype != TRIMKV_F16) return fail(TRIMKV_ERR_DTYPE, "%s: K/V/q must be bf16 or fp16 (dtype=%d)", fn, dtype);
     if (head_dim != 128 && head_dim != 96 && head_dim != 64) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be 64, 96 or 128 (got %d)", fn, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
@@ -491,14 +503,14 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
     }
     hipStream_t st = (hipStream_t)stream;
     switch (group) {
-        case 1: launch_attn<1>(a, head_dim, st); break;
-        case 2: launch_attn<2>(a, head_dim, st); break;
-        case 3: launch_attn<3>(a, head_dim, st); break;
-        case 4: launch_attn<4>(a, head_dim, st); break;
-        case 5: launch_attn<5>(a, head_dim, st); break;
-        case 6: launch_attn<6>(a, head_dim, st); break;
-        case 7: launch_attn<7>(a, head_dim, st); break;
-        default: launch_attn<8>(a, head_dim, st); break;
+        case 1: launch_attn<1>(a, head_dim, dtype, st); break;
+        case 2: launch_attn<2>(a, head_dim, dtype, st); break;
+        case 3: launch_attn<3>(a, head_dim, dtype, st); break;
+        case 4: launch_attn<4>(a, head_dim, dtype, st); break;
+        case 5: launch_attn<5>(a, head_dim, dtype, st); break;
+        case 6: launch_attn<6>(a, head_dim, dtype, st); break;
+        case 7: launch_attn<7>(a, head_dim, dtype, st); break;
+        default: launch_attn<8>(a, head_dim, dtype, st); break;
     }
     return launch_status(fn);
 }

@@ -59,13 +59,43 @@ struct SmallCfg {
     static constexpr int PIECES = (2 * PF_BN * 16 + THREADS - 1) / THREADS;  // 16-byte pieces per thread per tile (K and V)
 };
 
+typedef _Float16 pf_f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 pf_f16x2 __attribute__((ext_vector_type(2)));
+// K, V, q and P travel as raw 16-bit pairs (the bf16 vector types are only carriers); F16 selects how the matrix and dot
+// instructions read them and how fp32 results are rounded.
+template <bool F16>
+__device__ __forceinline__ pf_f32x4 mfma_16x16x32(pf_bf16x8 a, pf_bf16x8 b, pf_f32x4 c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pf_f16x8, a), __builtin_bit_cast(pf_f16x8, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+typedef float pf_f32x16_fwd __attribute__((ext_vector_type(16)));
+template <bool F16>
+__device__ __forceinline__ pf_f32x16_fwd mfma_32x32x16(pf_bf16x8 a, pf_bf16x8 b, pf_f32x16_fwd c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_f16x8, a), __builtin_bit_cast(pf_f16x8, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+    pf_f32x2 f = {lo, hi};
+    pf_f16x2 b = __builtin_convertvector(f, pf_f16x2);
+    return __builtin_bit_cast(uint32_t, b);
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi);
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_kv(float lo, float hi) { return F16 ? pack_f16(lo, hi) : pack_bf16(lo, hi); }
+// l + p.lo + p.hi for a packed pair of probabilities (a dot product with a pair of ones)
+template <bool F16>
+__device__ __forceinline__ float add_pair(uint32_t pw, float l) {
+    if constexpr (F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(pf_f16x2, pw), __builtin_bit_cast(pf_f16x2, 0x3C003C00u), l, false);
+    else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pf_bf16x2, pw), __builtin_bit_cast(pf_bf16x2, 0x3F803F80u), l, false);
+}
+
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     pf_f32x2 f = {lo, hi};
     pf_bf16x2 b = __builtin_convertvector(f, pf_bf16x2);
     return __builtin_bit_cast(uint32_t, b);
 }
 
-template <int G>
+template <int G, bool F16>
 __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(PrefillArgs a) {
     using C = SmallCfg<G>;
     __shared__ __attribute__((aligned(16))) char lds_k[PF_BN * PF_ROW];
@@ -149,7 +179,7 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
                     const pf_bf16x8 kf = *(const pf_bf16x8*)(lds_k + (kb * 16 + j) * PF_ROW + ig * 64 + ks * 16);
-                    s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[kb], 0, 0, 0);
+                    s[kb] = mfma_16x16x32<F16>(kf, qf[ks], s[kb]);
                 }
             }
             // lane holds keys kbase + kb*16 + 4*ig + v of query j
@@ -187,8 +217,8 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
                 for (int v = 0; v < 4; ++v) { oe[pb][v] *= alpha; oo[pb][v] *= alpha; }
             }
             // P^T operand: k index e <-> key (e < 4 ? 4*ig + e : 16 + 4*ig + e - 4), all in this lane
-            const uint4 pw = make_uint4(pack_bf16(p[0][0], p[0][1]), pack_bf16(p[0][2], p[0][3]),
-                                        pack_bf16(p[1][0], p[1][1]), pack_bf16(p[1][2], p[1][3]));
+            const uint4 pw = make_uint4(pack_kv<F16>(p[0][0], p[0][1]), pack_kv<F16>(p[0][2], p[0][3]),
+                                        pack_kv<F16>(p[1][0], p[1][1]), pack_kv<F16>(p[1][2], p[1][3]));
             const pf_bf16x8 pfrag = __builtin_bit_cast(pf_bf16x8, pw);
             // ---- O^T += V^T . P^T: A = 8 keys at d pair (pb*16 + j): dwords (d, d+1), split even/odd ----
 #pragma unroll
@@ -206,8 +236,8 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
                     od[x] = __builtin_amdgcn_perm(dw[2 * x + 1], dw[2 * x], 0x07060302u);
                 }
                 const uint4 evq = make_uint4(ev[0], ev[1], ev[2], ev[3]), odq = make_uint4(od[0], od[1], od[2], od[3]);
-                oe[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, evq), pfrag, oe[pb], 0, 0, 0);
-                oo[pb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(pf_bf16x8, odq), pfrag, oo[pb], 0, 0, 0);
+                oe[pb] = mfma_16x16x32<F16>(__builtin_bit_cast(pf_bf16x8, evq), pfrag, oe[pb]);
+                oo[pb] = mfma_16x16x32<F16>(__builtin_bit_cast(pf_bf16x8, odq), pfrag, oo[pb]);
             }
         }
     }
@@ -222,7 +252,7 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
         for (int pb = 0; pb < 4; ++pb) {
 #pragma unroll
             for (int v = 0; v < 4; ++v)
-                if (2 * (pb * 16 + 4 * ig + v) < a.hd) orow[pb * 16 + 4 * ig + v] = pack_bf16(oe[pb][v] * inv, oo[pb][v] * inv);
+                if (2 * (pb * 16 + 4 * ig + v) < a.hd) orow[pb * 16 + 4 * ig + v] = pack_kv<F16>(oe[pb][v] * inv, oo[pb][v] * inv);
         }
     }
 }
@@ -270,6 +300,7 @@ __device__ __forceinline__ int pf2_key_of_slot(int slot) {
     return kb * 32 + st * 16 + hl * 4 + (e & 3) + ((e >> 2) << 3);
 }
 
+template <bool F16>
 __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
 
@@ -392,7 +423,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
-            s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], s, 0, 0, 0);
+            s = mfma_32x32x16<F16>(kf, qf[ks], s);
         }
         return s;
     };
@@ -426,8 +457,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     auto p_pair = [&](const pf_f32x16& s, int x) __attribute__((always_inline)) {
         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x], a.scale_log2, -m_ref));
         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x + 1], a.scale_log2, -m_ref));
-        const uint32_t pw = pack_bf16(p0, p1);
-        l_run = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pf_bf16x2, pw), __builtin_bit_cast(pf_bf16x2, 0x3F803F80u), l_run, false);
+        const uint32_t pw = pack_kv<F16>(p0, p1);
+        l_run = add_pair<F16>(pw, l_run);
         return pw;
     };
     auto v_frag = [&](const char* buf, int kb, int st, int db) __attribute__((always_inline)) {
@@ -463,7 +494,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         for (int ks = 0; ks < 8; ++ks) {
             request(ks + PD);
             pw[ks] = p_pair(s_cur, ks);
-            if (HAS_NEXT) s_nxt = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[ks], qf[ks], s_nxt, 0, 0, 0);
+            if (HAS_NEXT) s_nxt = mfma_32x32x16<F16>(frag[ks], qf[ks], s_nxt);
             __builtin_amdgcn_sched_barrier(0);
         }
         pf_bf16x8 pfrag[2];
@@ -475,7 +506,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             request(8 + i + PD);
-            o[i & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag[8 + i], pfrag[i >> 2], o[i & 3], 0, 0, 0);
+            o[i & 3] = mfma_32x32x16<F16>(frag[8 + i], pfrag[i >> 2], o[i & 3]);
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -537,22 +568,22 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         for (int db = 0; db < 4; ++db) {
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                const uint2 pk = make_uint2(pack_bf16(o[db][4 * c] * inv, o[db][4 * c + 1] * inv),
-                                            pack_bf16(o[db][4 * c + 2] * inv, o[db][4 * c + 3] * inv));
+                const uint2 pk = make_uint2(pack_kv<F16>(o[db][4 * c] * inv, o[db][4 * c + 1] * inv),
+                                            pack_kv<F16>(o[db][4 * c + 2] * inv, o[db][4 * c + 3] * inv));
                 if (db * 32 + 8 * c + 4 * hl < a.hd) *(uint2*)(orow + (db * 32 + 8 * c + 4 * hl) * 2) = pk;
             }
         }
     }
 }
 
-template <int G>
+template <int G, bool F16>
 static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
     // short chunks: 16 queries per wavefront waste fewer MFMA columns; a non-positive scale: the large kernel takes
     // row maxima before scaling, which needs scale > 0
     if (a.q_len < 64 || !(a.scale_log2 > 0.0f)) {
         using C = SmallCfg<G>;
         const int tiles = (a.q_len + C::BT - 1) / C::BT;
-        hipLaunchKernelGGL(prefill_small_kernel<G>, dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
+        hipLaunchKernelGGL((prefill_small_kernel<G, F16>), dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
         return 0;
     }
     // > 64 KB of dynamic LDS needs the attribute once per device (the flag is only ever set, so a race repeats the call at worst)
@@ -560,12 +591,12 @@ static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = -1;
     if (dev < 0 || !lds_opted_in[dev]) {
-        hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
+        hipError_t e = hipFuncSetAttribute((const void*)prefill_attn_kernel<F16>, hipFuncAttributeMaxDynamicSharedMemorySize, PF2_LDS);
         if (e != hipSuccess) return (int)e;
         if (dev >= 0) lds_opted_in[dev] = true;
     }
     const int bt = (PF2_WAVES * 32) / G;
-    hipLaunchKernelGGL(prefill_attn_kernel, dim3((a.q_len + bt - 1) / bt, nseg), dim3(PF2_THREADS), PF2_LDS, st, a);
+    hipLaunchKernelGGL(prefill_attn_kernel<F16>, dim3((a.q_len + bt - 1) / bt, nseg), dim3(PF2_THREADS), PF2_LDS, st, a);
     return 0;
 }
 
@@ -579,7 +610,7 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
                                    int max_len, void* stream) {
     const char* fn = "trimkv_prefill_attn";
     if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
-    if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 K/V/q are supported (dtype=%d)", fn, dtype);
+    if (dtype != TRIMKV_BF16 && dtype != TRIMKV_F16) return fail(TRIMKV_ERR_DTYPE, "%s: K/V/q must be bf16 or fp16 (dtype=%d)", fn, dtype);
     if (head_dim != 128 && head_dim != 96 && head_dim != 64) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be 64, 96 or 128 (got %d)", fn, head_dim);
     if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
     if (batch <= 0 || kv_heads <= 0 || q_len <= 0 || cap <= 0 || max_len <= 0)
@@ -594,16 +625,17 @@ extern "C" int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_
     a.k = (const char*)k_slab; a.v = (const char*)v_slab; a.seg_len = seg_len; a.seg_start = seg_start;
     a.kv_heads = kv_heads; a.group = group; a.q_len = q_len; a.cap = cap; a.max_len = max_len; a.hd = head_dim; a.scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
+    const bool f16 = dtype == TRIMKV_F16;
     int rc = 0;
     switch (group) {
-        case 1: rc = launch_prefill<1>(a, (int)nseg, st); break;
-        case 2: rc = launch_prefill<2>(a, (int)nseg, st); break;
-        case 3: rc = launch_prefill<3>(a, (int)nseg, st); break;
-        case 4: rc = launch_prefill<4>(a, (int)nseg, st); break;
-        case 5: rc = launch_prefill<5>(a, (int)nseg, st); break;
-        case 6: rc = launch_prefill<6>(a, (int)nseg, st); break;
-        case 7: rc = launch_prefill<7>(a, (int)nseg, st); break;
-        default: rc = launch_prefill<8>(a, (int)nseg, st); break;
+        case 1: rc = f16 ? launch_prefill<1, true>(a, (int)nseg, st) : launch_prefill<1, false>(a, (int)nseg, st); break;
+        case 2: rc = f16 ? launch_prefill<2, true>(a, (int)nseg, st) : launch_prefill<2, false>(a, (int)nseg, st); break;
+        case 3: rc = f16 ? launch_prefill<3, true>(a, (int)nseg, st) : launch_prefill<3, false>(a, (int)nseg, st); break;
+        case 4: rc = f16 ? launch_prefill<4, true>(a, (int)nseg, st) : launch_prefill<4, false>(a, (int)nseg, st); break;
+        case 5: rc = f16 ? launch_prefill<5, true>(a, (int)nseg, st) : launch_prefill<5, false>(a, (int)nseg, st); break;
+        case 6: rc = f16 ? launch_prefill<6, true>(a, (int)nseg, st) : launch_prefill<6, false>(a, (int)nseg, st); break;
+        case 7: rc = f16 ? launch_prefill<7, true>(a, (int)nseg, st) : launch_prefill<7, false>(a, (int)nseg, st); break;
+        default: rc = f16 ? launch_prefill<8, true>(a, (int)nseg, st) : launch_prefill<8, false>(a, (int)nseg, st); break;
     }
     if (rc) return fail(rc, "%s: hipFuncSetAttribute failed (%d)", fn, rc);
     return launch_status(fn);
