@@ -214,7 +214,7 @@ def prefill_main(args):
         "config": {"workload": f"BASELINE config 5 ({c['name']} shape) prompt phase: {L} layers, batch {B}, {Hkv} KV heads, {Hq} query heads, "
                                f"head_dim {D}, chunks of {S} tokens on {M} retained tokens per head, eviction {n} -> {M} after every chunk",
                    "note": "secondary workload; the headline metric is the default run"},
-        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel", "achieved": round(flops / avg_s / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
+        "roofline": {"bound": "mfma", "kernel": "prefill_attn_kernel<false>", "achieved": round(flops / avg_s / 1e12, 1), "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": round(flops / avg_s / 1e12 / 2500.0, 4), "traffic": None, "avg_launch_us": round(avg_s * 1e6, 1),
                      "launches_sampled": len(events), "algorithmic_flops_per_launch": int(flops)},
     }
@@ -321,7 +321,7 @@ def ragged_main(args):
     if events:
         avg_s = sum(e0.elapsed_time(e1) for e0, e1, _ in events) * 1e-3 / len(events)
         avg_b = sum(n * 2 * D * 2 + nseg * 2 * G * D * 2 for _, _, n in events) / len(events)
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16> + decode_attn_merge_kernel<{G}, 16>", "achieved": round(avg_b / avg_s / 1e9, 1),
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false> + decode_attn_merge_kernel<{G}, 16, false>", "achieved": round(avg_b / avg_s / 1e9, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(avg_b / avg_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(events), "algorithmic_bytes_per_launch": int(avg_b)}
     out_json = {
@@ -480,7 +480,7 @@ def main():
         avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16>" + ("" if B * Hkv >= 160 else f" + decode_attn_merge_kernel<{G}, 16>"), "achieved": round(achieved, 1),
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false>" + ("" if B * Hkv >= 160 else f" + decode_attn_merge_kernel<{G}, 16, false>"), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
