@@ -91,7 +91,7 @@ int trimkv_append(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, 
  *     part[j][t][h] = sum over the j-th slice of intermediate units u of
  *                     W2[h][u] * silu( W1[u][:] . x[t][:] + b1[u] )
  * (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:171-176).  x [ntok][hidden], w1
- * [inter][hidden], b1 [inter] (nullable), w2 [kv_heads][inter], all `dtype` (bf16);
+ * [inter][hidden], b1 [inter] (nullable), w2 [kv_heads][inter], all `dtype` (bf16 or fp16);
  * part is f32 [nslice][ntok][kv_heads] with nslice = trimkv_gate_slices(inter).
  * The second half (sum of slices + bias, logsigmoid, :177-179) is fused into
  * trimkv_append_gated.

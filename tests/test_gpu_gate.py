@@ -92,3 +92,33 @@ def test_kv_gates_match_oracle(kind, B, S, H):
     assert (got - want16).abs().mean() <= (want16 - want32).abs().mean() * 2 + 1e-4
     # [B, S, Hkv, 2D] input with transpose=False is the same thing
     assert torch.equal(g(kv.to(DEV).transpose(1, 2).contiguous(), transpose=False).materialize().cpu(), lazy.materialize().cpu())
+
+
+@pytest.mark.parametrize("kind", ["rg", "rg3"])
+def test_fp16_gates_run_fused(kind):
+    """An fp16 model: the same kernels with the fp16 matrix instruction and fp16 roundings; the append epilogue writes what
+    materialize() computes."""
+    from trimkv_amd import LazyLogBeta, TrimKVCache
+    from trimkv_amd.gate import RetentionGate, RetentionGate3
+    torch.manual_seed(11)
+    B, S, H, D, inter = 3, 40, 4, 128, 128
+    if kind == "rg":
+        g = RetentionGate(1024, H, inter, bias_init=2.0, initializer_range=0.05)
+        g.linear1.bias.data.normal_(0, 0.1)
+        x = torch.randn(B, S, 1024)
+    else:
+        g = RetentionGate3(D, H, inter, bias_init=2.0, initializer_range=0.05)
+        x = torch.randn(B, H, S, 2 * D)
+    want32 = g(x)                                              # fp32 module on the CPU
+    g = g.to(torch.float16).eval().to(DEV)
+    lazy = g(x.to(torch.float16).to(DEV))
+    assert isinstance(lazy, LazyLogBeta) and lazy.dtype == torch.float16
+    got = lazy.materialize()
+    assert got.dtype == torch.float16
+    err = (got.float().cpu() - want32).abs()
+    assert (err <= 1e-2 * want32.abs() + 2e-3).all(), float(err.max())
+    k = torch.randn(B, H, S, D).to(torch.float16).to(DEV)
+    a, b = TrimKVCache(), TrimKVCache()
+    a.update(k, k, lazy.transpose(1, 2), torch.arange(S, device=DEV), 0)
+    b.update(k, k, lazy.transpose(1, 2).materialize(), torch.arange(S, device=DEV), 0)
+    assert a.retention_weights[0].dtype == torch.float16 and torch.equal(a.retention_weights[0], b.retention_weights[0])

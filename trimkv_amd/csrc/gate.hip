@@ -18,6 +18,18 @@ namespace trimkv {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+// 16-bit values travel as raw bits (bf16x8_t is only the carrier); F16 selects the matrix instruction and the roundings.
+template <bool F16>
+__device__ __forceinline__ f32x4_t gate_mfma(bf16x8_t a, bf16x8_t b, f32x4_t c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+template <bool F16> __device__ __forceinline__ float gate_load(uint16_t b) { return F16 ? f16_bits_to_f32(b) : bf16_bits_to_f32(b); }
+template <bool F16> __device__ __forceinline__ float gate_round(float f) {
+    return F16 ? f16_bits_to_f32(f32_to_f16_bits(f)) : bf16_bits_to_f32(f32_to_bf16_bits(f));
+}
 
 constexpr int GH_THREADS = 1024;
 constexpr int GH_WAVES = 16;
@@ -34,7 +46,7 @@ struct GateArgs {
 //   TT = 1, KS = 16: decode (a handful of tokens): many small workgroups and short dependent chains;
 //   TT = 4, KS = 4 : prompts: a W1 slice is reused by 64 tokens.
 // STEPS k-steps of 32 are unrolled with all their loads issued before the first MFMA.
-template <int TT, int STEPS, bool SWIGLU>
+template <int TT, int STEPS, bool SWIGLU, bool F16>
 __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
     constexpr int KS = GH_WAVES / TT, TOKENS = 16 * TT;
     __shared__ float red[SWIGLU ? 2 : 1][KS][TOKENS][GH_UNITS + 1];
@@ -58,10 +70,10 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
 #pragma unroll
     for (int i = 0; i < HB; ++i) w2v[i] = 0.0f;
     if (epi) {
-        if (a.b1) b1v = bf16_bits_to_f32(a.b1[eu]);
+        if (a.b1) b1v = gate_load<F16>(a.b1[eu]);
 #pragma unroll
         for (int i = 0; i < HB; ++i)
-            if (i < a.kv_heads) w2v[i] = bf16_bits_to_f32(a.w2[(int64_t)i * a.inter + eu]);
+            if (i < a.kv_heads) w2v[i] = gate_load<F16>(a.w2[(int64_t)i * a.inter + eu]);
     }
 
     f32x4_t acc = {0.f, 0.f, 0.f, 0.f}, acc_up = {0.f, 0.f, 0.f, 0.f};
@@ -77,8 +89,8 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
 #pragma unroll
         for (int i = 0; i < STEPS; ++i) {
             if (k0 + 32 * i < kspan) {
-                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], bv[i], acc, 0, 0, 0);
-                if constexpr (SWIGLU) acc_up = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av[i], uv[i], acc_up, 0, 0, 0);
+                acc = gate_mfma<F16>(av[i], bv[i], acc);
+                if constexpr (SWIGLU) acc_up = gate_mfma<F16>(av[i], uv[i], acc_up);
             }
         }
     }
@@ -97,21 +109,21 @@ __global__ __launch_bounds__(GH_THREADS) void gate_hidden_kernel(GateArgs a) {
 #pragma unroll
         for (int i = 0; i < KS; ++i) h += red[0][i][t][u];
         h += b1v;
-        h = bf16_bits_to_f32(f32_to_bf16_bits(h));            // nn.Linear output in bf16
+        h = gate_round<F16>(h);            // nn.Linear output in the model dtype
         float act = h / (1.0f + __expf(-h));
-        act = bf16_bits_to_f32(f32_to_bf16_bits(act));        // SiLU output in bf16
+        act = gate_round<F16>(act);        // SiLU output in the model dtype
         if constexpr (SWIGLU) {
             float up_v = 0.0f;
 #pragma unroll
             for (int i = 0; i < KS; ++i) up_v += red[1][i][t][u];
-            up_v = bf16_bits_to_f32(f32_to_bf16_bits(up_v));  // up_proj output in bf16
-            act = bf16_bits_to_f32(f32_to_bf16_bits(act * up_v));
+            up_v = gate_round<F16>(up_v);  // up_proj output in the model dtype
+            act = gate_round<F16>(act * up_v);
         }
         for (int h0 = 0; h0 < a.kv_heads; h0 += HB) {
             if (h0 > 0) {                                      // more than HB heads: fetch the next batch of W2
 #pragma unroll
                 for (int i = 0; i < HB; ++i)
-                    w2v[i] = h0 + i < a.kv_heads ? bf16_bits_to_f32(a.w2[(int64_t)(h0 + i) * a.inter + eu]) : 0.0f;
+                    w2v[i] = h0 + i < a.kv_heads ? gate_load<F16>(a.w2[(int64_t)(h0 + i) * a.inter + eu]) : 0.0f;
             }
             float p[HB];
 #pragma unroll
@@ -140,7 +152,7 @@ extern "C" int trimkv_gate_slices(int inter) { return inter > 0 && inter % GH_UN
 static int gate_launch(const char* fn, const void* x, const void* w1, const void* b1, const void* w_up, const void* w2, float* part,
                        int ntok, int hidden, int inter, int kv_heads, int dtype, bool swiglu, void* stream) {
     if (!x || !w1 || !w2 || !part || (swiglu && !w_up)) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
-    if (dtype != TRIMKV_BF16) return fail(TRIMKV_ERR_DTYPE, "%s: only bf16 gate weights are supported (dtype=%d)", fn, dtype);
+    if (dtype != TRIMKV_BF16 && dtype != TRIMKV_F16) return fail(TRIMKV_ERR_DTYPE, "%s: gate weights must be bf16 or fp16 (dtype=%d)", fn, dtype);
     if (ntok <= 0 || hidden <= 0 || inter <= 0 || kv_heads <= 0 || kv_heads > GH_MAX_HEADS)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes ntok=%d hidden=%d inter=%d kv_heads=%d", fn, ntok, hidden, inter, kv_heads);
     if (hidden % (32 * GH_WAVES) || inter % GH_UNITS)
@@ -151,15 +163,18 @@ static int gate_launch(const char* fn, const void* x, const void* w1, const void
     a.w_up = (const uint16_t*)w_up;
     a.ntok = ntok; a.hidden = hidden; a.inter = inter; a.kv_heads = kv_heads;
     hipStream_t st = (hipStream_t)stream;
-    if (ntok <= 256) {  // decode-sized: 16-token tiles, 16-way split of the hidden axis
-        dim3 grid(inter / GH_UNITS, (ntok + 15) / 16);
-        if (swiglu) hipLaunchKernelGGL((gate_hidden_kernel<1, 8, true>), grid, dim3(GH_THREADS), 0, st, a);
-        else hipLaunchKernelGGL((gate_hidden_kernel<1, 8, false>), grid, dim3(GH_THREADS), 0, st, a);
+    const bool f16 = dtype == TRIMKV_F16;
+    const bool small = ntok <= 256;   // decode-sized: 16-token tiles, 16-way split of the hidden axis; else 64-token tiles
+    const dim3 grid(inter / GH_UNITS, small ? (ntok + 15) / 16 : (ntok + 63) / 64);
+#define TRIMKV_GATE_LAUNCH(TT, SW, F) hipLaunchKernelGGL((gate_hidden_kernel<TT, 8, SW, F>), grid, dim3(GH_THREADS), 0, st, a)
+    if (small) {
+        if (swiglu) { if (f16) TRIMKV_GATE_LAUNCH(1, true, true); else TRIMKV_GATE_LAUNCH(1, true, false); }
+        else { if (f16) TRIMKV_GATE_LAUNCH(1, false, true); else TRIMKV_GATE_LAUNCH(1, false, false); }
     } else {
-        dim3 grid(inter / GH_UNITS, (ntok + 63) / 64);
-        if (swiglu) hipLaunchKernelGGL((gate_hidden_kernel<4, 8, true>), grid, dim3(GH_THREADS), 0, st, a);
-        else hipLaunchKernelGGL((gate_hidden_kernel<4, 8, false>), grid, dim3(GH_THREADS), 0, st, a);
+        if (swiglu) { if (f16) TRIMKV_GATE_LAUNCH(4, true, true); else TRIMKV_GATE_LAUNCH(4, true, false); }
+        else { if (f16) TRIMKV_GATE_LAUNCH(4, false, true); else TRIMKV_GATE_LAUNCH(4, false, false); }
     }
+#undef TRIMKV_GATE_LAUNCH
     return launch_status(fn);
 }
 

@@ -48,7 +48,8 @@ class RetentionGate(nn.Module):
         return F.logsigmoid(self.linear2(act(self.linear1(x))) + self.bias)
 
     def _use_hip(self, x: torch.Tensor) -> bool:
-        return (self.fused and not self.training and x.is_cuda and x.dtype == torch.bfloat16
+        return (self.fused and not self.training and x.is_cuda and x.dtype in (torch.bfloat16, torch.float16)
+                and self.bias.dtype == x.dtype
                 and self.hidden_act == "silu" and x.shape[-1] % 512 == 0
                 and self.retention_gate_intermediate_size % 16 == 0)
 
@@ -62,7 +63,7 @@ class RetentionGate(nn.Module):
     def _launch(self, lib, x2, part, ntok, hidden) -> None:
         w1, b1, w2 = self.linear1.weight, self.linear1.bias, self.linear2.weight
         rc = lib.trimkv_gate_hidden(x2.data_ptr(), w1.data_ptr(), b1.data_ptr(), w2.data_ptr(), part.data_ptr(), ntok, hidden,
-                                    self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.BF16,
+                                    self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.dtype_code(x2.dtype),
                                     _lib.current_stream(x2.device))
         _lib.check(rc, "trimkv_gate_hidden")
 
@@ -130,7 +131,7 @@ class RetentionGate3(RetentionGate):
     def _launch(self, lib, x2, part, ntok, hidden) -> None:
         rc = lib.trimkv_gate_hidden_swiglu(x2.data_ptr(), self.gate_proj.weight.data_ptr(), self.up_proj.weight.data_ptr(),
                                            self.down_proj.weight.data_ptr(), part.data_ptr(), ntok, hidden,
-                                           self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.BF16,
+                                           self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.dtype_code(x2.dtype),
                                            _lib.current_stream(x2.device))
         _lib.check(rc, "trimkv_gate_hidden_swiglu")
 
