@@ -89,14 +89,16 @@ def _record_updates(cache, nlayers):
     return rec
 
 
-@pytest.mark.parametrize("family,gate", [("qwen3", "rg"), ("qwen3", "rg2"), ("qwen3", "rg3"), ("llama", "rg"), ("llama", "rg2"),
-                                         ("phi3", "rg"), ("phi3", "rg2"), ("phi3mini", "rg")])
-def test_shell_logits_match_fp32_replay_of_retained_positions(family, gate):
+@pytest.mark.parametrize("family,gate,dtype", [("qwen3", "rg", torch.bfloat16), ("qwen3", "rg2", torch.bfloat16), ("qwen3", "rg3", torch.bfloat16),
+                                               ("llama", "rg", torch.bfloat16), ("llama", "rg2", torch.bfloat16), ("phi3", "rg", torch.bfloat16),
+                                               ("phi3", "rg2", torch.bfloat16), ("phi3mini", "rg", torch.bfloat16),
+                                               ("qwen3", "rg", torch.float16), ("phi3mini", "rg", torch.float16)])
+def test_shell_logits_match_fp32_replay_of_retained_positions(family, gate, dtype):
     from trimkv_amd import TrimKVCache, LazyLogBeta
     from trimkv_amd import attn as attn_registry
     torch.manual_seed(0)
     cfg = _tiny_config(family, retention_gate=gate)
-    model = _family(family)[1](cfg).to(torch.bfloat16).eval()
+    model = _family(family)[1](cfg).to(dtype).eval()
     ref = copy.deepcopy(model).float()
     ref.config = copy.copy(cfg)
     for m in ref.modules():
