@@ -187,3 +187,16 @@ def test_random_ragged_attention_shapes(seed):
     want = ragged_attention(q, K[:tot], V[:tot], torch.from_numpy(cu), H)
     ok, err = attn_close(out, want)
     assert ok and torch.isfinite(out.float()).all(), f"seed {seed} (B={B} H={H} G={G} D={D} Q={Q}): max abs err {err}"
+
+
+@pytest.mark.parametrize("Q", [1, 2, 65])
+def test_all_segments_empty(Q):
+    """Nothing cached anywhere (packed rows, zero total length): attention is defined as zeros, not an error."""
+    from trimkv_amd import get_attention_interface
+    attn = get_attention_interface("db_attn_flash_batched")
+    kw = {"head_lens": torch.zeros(2, dtype=torch.int32, device=DEV), "cu_seqlens_k": torch.zeros(3, dtype=torch.int32, device=DEV),
+          "batch_size": 1, "num_kv_heads": 2}
+    k = torch.zeros(1, 128, dtype=torch.bfloat16, device=DEV)
+    q = torch.randn(1, 4, Q, 128).to(torch.bfloat16).to(DEV)
+    out, _, _ = attn(_Mod(), q, k, k, None, flash_attn_kwargs=kw)
+    assert out.shape == (1, Q, 4, 128) and not out.any()

@@ -169,7 +169,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         max_len = kw.get("max_len")
         if max_len is None:
             max_len = int(head_lens.max().item())  # the reference synchronises here as well (flash_attn.py:58, 133)
-        cap = max_len
+        cap = max(1, max_len)   # unused with packed rows; the library only wants it positive (every segment may be empty)
     else:
         max_len, cap = kw["max_len"], kw["seg_cap"]
     if Q == 1:
