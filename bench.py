@@ -484,7 +484,7 @@ def main():
         avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false>" + ("" if B * Hkv >= 160 else f" + decode_attn_merge_kernel<{G}, 16, false>"), "achieved": round(achieved, 1),
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false>" + ("" if B * Hkv >= 128 else f" + decode_attn_merge_kernel<{G}, 16, false>"), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),

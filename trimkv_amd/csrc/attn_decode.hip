@@ -16,7 +16,7 @@
 //     packed bf16 pairs, and P.V is v_dot2_f32_bf16 over two rows at a time (v_perm_b32
 //     interleaves the rows);
 //   * the four wavefronts of a workgroup own disjoint quarters of the workgroup's rows and merge
-//     (max, sum, accumulator) in LDS; with 160 segments or more (or when the caller's chunk covers
+//     (max, sum, accumulator) in LDS; with 128 segments or more (or when the caller's chunk covers
 //     the longest segment) one workgroup covers a whole segment and writes the output itself,
 //     otherwise segments are split and a second, tiny kernel merges the partials;
 //   * rows of 96 or 64 features keep their length in memory: the 16-lane row group then has 12 or 8
@@ -429,12 +429,13 @@ __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a)
 }
 
 static int pick_chunk(int nseg, int max_len) {
-    // One workgroup per segment streams at full rate from about 160 segments on (a workgroup keeps 12 tiles in flight;
-    // measured: at 128 segments two splits and the merge launch are 7-12 % faster than whole segments, at 160 and more
-    // they are slower); with fewer, segments are cut so that about 256 workgroups exist, but not below 512 rows each
-    // (one full block per wavefront).
+    // One workgroup per segment streams at full rate already with 128 segments (a workgroup keeps 12 tiles in flight).  In a
+    // decode step over 28 layers (nothing of a layer survives in the last-level cache until its next turn) two splits plus
+    // the merge launch took 25.6 + 3.9 us per layer at 128 segments x 2112 rows against 28.6 us for whole segments; a
+    // single layer replayed from the last-level cache had suggested the opposite.  With fewer segments they are cut so
+    // that about 256 workgroups exist, but not below 512 rows each (one full block per wavefront).
     const int whole = ((max_len + 63) / 64) * 64;
-    if (nseg >= 160) return whole;
+    if (nseg >= 128) return whole;
     const int nsplit = (256 + nseg - 1) / nseg;
     int chunk = (((max_len + nsplit - 1) / nsplit + 63) / 64) * 64;
     if (chunk < 512) chunk = 512;
