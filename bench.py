@@ -8,7 +8,11 @@ logsigmoid(N(mu, sigma)) in fp32, random bf16 queries) and resident in HBM befor
 
     python bench.py [--gpus 1] [--steps 1024] [--warmup 128] [--config 3]
 
-prints ONE JSON line.  `value` = batch * steps / seconds (decode tokens/s for the whole job).
+prints ONE JSON line.  `value` = batch / seconds per step (decode tokens/s for the whole job).  With --steps of at
+least one eviction cycle (buffer_size steps) the evictions fall inside the timed steps and seconds per step is wall
+clock / steps.  A shorter window holds no eviction: it is then placed in the middle of the cycle (mean attended
+length = the cycle mean), one eviction of all layers is timed right after it, and
+ms_per_step = ms_append_attend + ms_evict_round / buffer_size (both raw figures are in `config`).
 `roofline` prices the dominant kernel (decode attention) against the 8 TB/s HBM peak using its
 algorithmic bytes and HIP-event durations sampled inside the timed region; `cpu_baseline` times the
 CPU oracle (the reference's pure-PyTorch path restated) on a bounded sample of the same workload.
@@ -108,16 +112,13 @@ def cpu_baseline(c, budget_s=20.0):
             "os_cpu_count": cores}
 
 
-def parity_gate(cache, c, attn_fn, mod):
-    """Outside the timed region: one more eviction on layer 0 checked against torch.topk on the same fp32 scores
-    (retained indices bit-exact for every segment) and the attention of a few segments against fp32 softmax.
+def attention_gate(cache, c, attn_fn, mod):
+    """Outside the timed region: the attention of a few segments of layer 0 against fp32 softmax.
     (The full oracle comparison lives in tests/; this gate only guards the run that was just timed.)"""
     import torch
 
     slab = cache._slabs[0]
     n = slab.max_len
-    lb = slab.lb[:, :n].cpu()
-    pos = slab.pos[:, :n].cpu()
     k = slab.k[:8, :n].float().cpu()
     v = slab.v[:8, :n].float().cpu()
     G = c["Hq"] // c["Hkv"]
@@ -130,18 +131,45 @@ def parity_gate(cache, c, attn_fn, mod):
     got = out.reshape(-1, G, D)[:8].float().cpu()
     err = (got - want).abs()
     attn_ok = bool((err <= 2e-2 + 1e-2 * want.abs()).all())
-    result = {"attention_max_abs_err": float(err.max()), "attention_within_2e-2_abs_1e-2_rel": attn_ok}
-    if n > c["M"]:
-        q_idx = cache.get_seq_length(0) + 1
+    return {"attention_max_abs_err": float(err.max()), "attention_within_2e-2_abs_1e-2_rel": attn_ok}
+
+
+def timed_checked_eviction(cache, c, layers_to_check):
+    """One all-layer ``compress`` (every layer is due: the single launch over all layers that the timed steps use),
+    bracketed by HIP events, with the retained rows of ``layers_to_check`` compared against torch.topk on the scores
+    snapshotted just before it: fp32(log beta) * fp32(age), indices sorted ascending, bit-exact on every segment
+    whose cut is not a tie.  Returns (milliseconds, parity dict)."""
+    import torch
+
+    M, buf = c["M"], c["buf"]
+    snaps = {}
+    for l in layers_to_check:
+        slab = cache._slabs[l]
+        n = slab.max_len
+        assert n >= M + buf, "the eviction is not due yet"
+        snaps[l] = (slab.lb[:, :n].clone(), slab.pos[:, :n].clone(), cache.get_seq_length(l) + 1)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    cache.compress("alpha", M, buf)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1)
+    checked = mismatches = ties = 0
+    for l, (lb, pos, q_idx) in snaps.items():
+        slab = cache._slabs[l]
+        assert slab.max_len == M
         sc = lb.float() * (q_idx - pos).float()          # fp32(log beta) * fp32(age), one rounding
-        top = torch.topk(sc, c["M"] + 1, dim=-1).values
-        ties = int((top[:, c["M"] - 1] == top[:, c["M"]]).sum())
-        want_idx = torch.topk(sc, c["M"], dim=-1).indices.sort(dim=-1).values
-        got_idx = cache.compress_layer(0, c["M"], return_indices=True).view(-1, c["M"]).cpu().long()
-        same = (got_idx == want_idx).all(dim=-1)
-        result.update({"evicted_segments_checked": int(same.numel()), "retained_index_mismatches": int((~same).sum()),
-                       "boundary_tie_rows": ties})
-    return result
+        top = torch.topk(sc, M + 1, dim=-1)
+        tie = top.values[:, M - 1] == top.values[:, M]
+        want_idx = top.indices[:, :M].sort(dim=-1).values
+        want_pos = pos.gather(1, want_idx)
+        same = (slab.pos[:, :M] == want_pos).all(dim=-1) & (slab.lb[:, :M] == lb.gather(1, want_idx)).all(dim=-1)
+        same &= (slab.seg_len == M)
+        checked += int(same.numel())
+        ties += int(tie.sum())
+        mismatches += int((~same & ~tie).sum())
+    return ms, {"evicted_layers_checked": list(snaps), "evicted_segments_checked": checked, "retained_index_mismatches": mismatches,
+                "boundary_tie_rows": ties, "launch": "all layers in one trimkv_evict_layers launch"}
 
 
 def prefill_main(args):
@@ -399,9 +427,10 @@ def main():
         _orig = hip_attn.decode_attention
         hip_attn.decode_attention = lambda *a, **k: _orig(*a, **{**k, "chunk": args.chunk})
 
-    # steady-state cache: M + buf tokens per head, so the first step appends, attends and evicts
+    # Cycle of the steady state: an eviction takes every head to M rows, the next buf steps attend M+1 .. M+buf rows and the
+    # last of them evicts again.  The cache starts one row short of the trigger, so the first warm-up step evicts.
     cache = TrimKVCache()
-    n0 = M + buf
+    n0 = M + buf - 1
     pos0 = torch.arange(n0, device=dev)
     for l in range(L):
         k = torch.randn(B, Hkv, n0, D, generator=gen, device=dev, dtype=torch.float32).to(torch.bfloat16)
@@ -438,61 +467,116 @@ def main():
         del src, dst
 
     T = n0
+    tick = 0
     events = []
+    nseg = B * Hkv
+    attn_bytes = lambda n: nseg * (2 * n * D * 2 + 2 * G * D * 2)                    # K and V rows read once, q read, o written
+    append_bytes = nseg * (2 * D * 2 + 12)                                          # one K row, one V row, log beta, position
+    evict_round_bytes = L * nseg * (12 * (M + buf) + 2 * 12 * M + 2 * 2 * M * D * 2)  # one eviction of every layer, M+buf -> M
 
-    def step(t, sample):
-        nonlocal T
+    def layers_pass(sample):
+        """Append + attend for every layer: one decode step without its eviction.  Returns the bytes it had to move."""
+        nonlocal T, tick
         pos = torch.full((1,), T, dtype=torch.int64, device=dev)
+        moved = 0
         for l in range(L):
-            kn, vn, lbn, q = pool[l][t % POOL]
+            kn, vn, lbn, q = pool[l][tick % POOL]
             if args.gate:
                 lbn = gates[l](hidden_pool[l]).transpose(1, 2)   # LazyLogBeta: finished inside the append kernel
             K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
+            n = cache.get_cache_length(l)
+            moved += attn_bytes(n) + append_bytes
             if sample:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
                 attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
                 e1.record()
-                events.append((e0, e1, cache.get_cache_length(l)))
+                events.append((e0, e1, n))
             else:
                 attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
         T += 1
+        tick += 1
+        return moved
+
+    def step(sample=False):
+        """One full decode step; returns (bytes moved, 1 if it evicted)."""
+        moved = layers_pass(sample)
         before = cache.get_cache_length(0)
         cache.compress("alpha", M, buf)
-        evictions[0] += cache.get_cache_length(0) < before    # host-side lengths: no synchronisation
+        evicted = int(cache.get_cache_length(0) < before)    # host-side lengths: no synchronisation
+        return moved + evicted * evict_round_bytes, evicted
 
-    evictions = [0]
-    for t in range(args.warmup):
-        step(t, False)
+    amortised = args.steps < buf
+    extra_untimed = 0
+    for _ in range(args.warmup):
+        step()
+    if amortised:
+        # A window shorter than one eviction cycle cannot contain a representative share of evictions.  It is placed in the
+        # middle of the cycle (its mean attended length is the cycle mean M + (buf+1)/2) and holds no eviction; one eviction
+        # of all layers is timed right after it and charged at 1/buf per step.
+        if args.warmup == 0:
+            step()   # the first step evicts: the window must start inside a cycle
+            extra_untimed += 1
+        want_n = M + (buf - args.steps) // 2
+        while cache.get_cache_length(0) != want_n:
+            step()
+            extra_untimed += 1
     torch.cuda.synchronize()
-    evictions[0] = 0
+    window_first_n = cache.get_cache_length(0) + 1
+    moved_bytes = 0
+    evictions = 0
     t0 = time.perf_counter()
     for t in range(args.steps):
-        step(args.warmup + t, args.event_every > 0 and t % args.event_every == 0)
+        b_, e_ = step(args.event_every > 0 and t % args.event_every == 0)
+        moved_bytes += b_
+        evictions += e_
     torch.cuda.synchronize()
     seconds = time.perf_counter() - t0
+    window_last_n = window_first_n + args.steps - 1 if amortised else None
 
-    ms_per_step = seconds * 1e3 / args.steps
-    value = B * args.steps / seconds
+    # one more eviction of all layers, timed on its own and checked against torch.topk (layers first, middle, last)
+    while cache.get_cache_length(0) + 1 < M + buf:
+        step()
+    layers_pass(False)
+    ms_evict_round, evict_parity = timed_checked_eviction(cache, c, sorted({0, L // 2, L - 1}))
+
+    ms_window = seconds * 1e3 / args.steps
+    if amortised:
+        assert evictions == 0
+        ms_per_step = ms_window + ms_evict_round / buf
+        bytes_per_step = moved_bytes / args.steps + evict_round_bytes / buf
+    else:
+        ms_per_step = ms_window
+        bytes_per_step = moved_bytes / args.steps
+    value = B / (ms_per_step * 1e-3)
     ab = algorithmic_bytes(c)
-    nseg = B * Hkv
     roof = None
     if events:
         durs = [e0.elapsed_time(e1) * 1e-3 for e0, e1, _ in events]
         lens = [n for _, _, n in events]
         avg_s = sum(durs) / len(durs)
-        avg_bytes = sum(nseg * (2 * n * D * 2 + 2 * G * D * 2) for n in lens) / len(lens)
+        avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
         roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false>" + ("" if B * Hkv >= 128 else f" + decode_attn_merge_kernel<{G}, 16, false>"), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
+                "traffic_measured_in_run": False,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
                 "algorithmic_bytes_per_launch": int(avg_bytes),
                 "mfma_utilisation": 0.0,
                 "mfma_note": f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
                              "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
-    parity = parity_gate(cache, c, attn_fn, mod)
+    parity = attention_gate(cache, c, attn_fn, mod)
+    parity.update(evict_parity)
+    timing = {"ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}
+    if amortised:
+        timing.update({"evictions_timed": "1 (amortised: ms_per_step = ms_append_attend + ms_evict_round / buffer_size)",
+                       "window_attended_rows": [window_first_n, window_last_n], "cycle_mean_attended_rows": M + (buf + 1) / 2,
+                       "extra_untimed_steps_to_reach_mid_cycle": extra_untimed})
+    else:
+        timing.update({"evictions_timed": evictions, "note": "evictions fall inside the timed steps; ms_per_step is wall clock / steps "
+                       "(ms_append_attend includes them); ms_evict_round is one further eviction timed on its own"})
     out = {
         "metric": METRIC, "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -500,11 +584,11 @@ def main():
         "config": {"workload": f"BASELINE config {args.config} ({c['name']} shape): {L} layers, batch {B}, {Hkv} KV heads, {Hq} query heads, "
                                f"head_dim {D}, memory_size {M}, buffer_size {buf}, steady-state decode (append + attend per layer, "
                                f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
-                   "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(), "evictions_in_timed_region": evictions[0],
-                   "eviction_note": (None if evictions[0] else f"no eviction fell into the {args.steps} timed steps (one is due every {buf}): "
-                                     "the value leaves out the eviction's amortised cost (run at least that many steps to include it)")},
-        "step_hbm": {"algorithmic_bytes_per_step": int(ab["step"]), "achieved_GBps": round(ab["step"] / (seconds / args.steps) / 1e9, 1),
-                     "frac_of_8TBps": round(ab["step"] / (seconds / args.steps) / 1e9 / HBM_PEAK_GBS, 4)},
+                   "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(), **timing},
+        "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
+                     "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "cycle_mean_algorithmic_bytes_per_step": int(ab["step"]),
+                     "note": "bytes of the steps and evictions that were executed and timed (algorithmic: rows at their actual lengths)"},
         "roofline": roof,
         "parity": parity,
     }

@@ -99,10 +99,10 @@ def test_config2_qwen3_1p7b_prefill_compression():
 
 
 def test_config5_qwen3_14b_chunk_eviction_gqa5():
-    """8 KV heads, G=5, M=8192, buffer 512: a 4096-token chunk on top of 8192 cached, select 8192 of 12288
-    (batch 2 of the config's 8 to bound memory; the kernel's grid is per segment)."""
+    """Batch 8, 8 KV heads, G=5, M=8192, buffer 512: a 4096-token chunk on top of 8192 cached, select 8192 of 12288;
+    then decode attention over the 64 segments of 8192 rows (4 splits + merge)."""
     from trimkv_amd import get_attention_interface
-    B, H, G, M, n = 2, 8, 5, 8192, 12288
+    B, H, G, M, n = 8, 8, 5, 8192, 12288
     cache, k, v, lb, gen = _fill_dense(B, H, n, 2.0, 2.0, seed=5)
     ties = _check_eviction(cache, k, v, lb, n, M, seen=n)
     assert ties <= 1
@@ -114,6 +114,102 @@ def test_config5_qwen3_14b_chunk_eviction_gqa5():
     want = torch.einsum("sgn,snd->sgd", p, V.reshape(B * H, M, 128).float())
     ok, err = attn_close(out.view(B * H, G, 128), want)
     assert ok, err
+
+
+def _fp32_attention_on_segments(q, K, V, segs, G, n):
+    """softmax(q K^T / sqrt(D)) V in fp32 for the listed segments; K/V are [nseg, >=n, D] slabs."""
+    q32 = q.reshape(-1, G, 128)[segs].float()
+    k32, v32 = K[segs, :n].float(), V[segs, :n].float()
+    p = torch.softmax(torch.einsum("sgd,snd->sgn", q32, k32) * 128 ** -0.5, -1)
+    return torch.einsum("sgn,snd->sgd", p, v32)
+
+
+@pytest.mark.parametrize("n", [2049, 2112, 2176])
+def test_config2_decode_attention_full_shape(n):
+    """BASELINE config 2's decode shape: batch 16 x 8 KV heads = 128 segments of 2049..2176 rows, 16 query heads (G=2) --
+    the shape at which the launch stops splitting segments (one workgroup per segment).  Through update() + the registered
+    attention, against fp32 softmax on sampled segments; a split launch of the same inputs must agree."""
+    from trimkv_amd import get_attention_interface
+    from trimkv_amd.attn.hip_attn import decode_attention
+    B, H, G = 16, 8, 2
+    cache, k, v, lb, gen = _fill_dense(B, H, n - 1, 3.0, 1.0, seed=n)
+    kn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    vn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    lbn = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) + 3.0)
+    K, V, _, _, kw = cache.update(kn, vn, lbn, torch.arange(n - 1, n, device=DEV), 0)
+    assert K.shape == (B, H, n, 128)
+    q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    out, _, _ = get_attention_interface("trimkv_hip")(_Mod(), q, K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)
+    segs = torch.arange(0, B * H, 8, device=DEV)
+    slab = cache._slabs[0]
+    want = _fp32_attention_on_segments(q, slab.k, slab.v, segs, G, n)
+    ok, err = attn_close(out.view(B * H, G, 128)[segs], want)
+    assert ok, err
+    assert torch.equal(slab.k[:, n - 1], kn.view(B * H, 128)) and torch.equal(slab.v[:, n - 1], vn.view(B * H, 128))
+    split = decode_attention(q.view(B * H * G, 128), slab.k, slab.v, B * H, G, slab.seg_len, None, slab.cap, n, 128 ** -0.5, chunk=1088)
+    assert (split.float() - out.view(-1, 128).float()).abs().max() < 4e-3
+
+
+@pytest.mark.parametrize("n", [8193, 8448, 8704])
+def test_config5_decode_attention_batch8_split_and_merge(n):
+    """BASELINE config 5's decode shape at its batch: 8 x 8 KV heads = 64 segments of 8193..8704 rows, 40 query heads
+    (G=5); with 64 segments every segment is cut into 4 pieces and merged by the second kernel."""
+    from trimkv_amd import _lib, get_attention_interface
+    B, H, G = 8, 8, 5
+    cache, k, v, lb, gen = _fill_dense(B, H, n, 2.0, 2.0, seed=n)
+    assert _lib.load().trimkv_decode_attn_workspace(B * H, G, 128, n, 0) > 0      # the library's own choice splits
+    K, V, _, _, kw = cache.update(None, None, None, None, 0)
+    q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    out, _, _ = get_attention_interface("trimkv_hip")(_Mod(), q, K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)
+    segs = torch.arange(0, B * H, 4, device=DEV)
+    slab = cache._slabs[0]
+    want = _fp32_attention_on_segments(q, slab.k, slab.v, segs, G, n)
+    ok, err = attn_close(out.view(B * H, G, 128)[segs], want)
+    assert ok, err
+
+
+def test_config3_all_36_layers_evicted_by_one_launch():
+    """BASELINE config 3 whole: 36 layers x 512 segments x 4224 rows (46 GB of slabs).  compress() evicts all layers with
+    ONE trimkv_evict_layers launch (grid 512 x 36, per-layer slabs from a device table); layers 0, 17 and 35 are
+    compared with torch.topk on scores snapshotted before it: retained rows, their order, K, V, log beta, positions."""
+    from trimkv_amd import TrimKVCache
+    L, B, H, M, buf = 36, 64, 8, 4096, 128
+    n = M + buf
+    gen = torch.Generator(device=DEV).manual_seed(33)
+    cache = TrimKVCache()
+    pos = torch.arange(n, device=DEV)
+    check = (0, 17, 35)
+    snaps = {}
+    for l in range(L):
+        k = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        v = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        lb = torch.nn.functional.logsigmoid(torch.randn(B, H, n, generator=gen, device=DEV) * 1.5 + 3.0)
+        cache.update(k, v, lb, pos, l)
+        if l in check:
+            snaps[l] = (k, v, lb)
+        del k, v, lb
+    launches = []
+    orig = cache._evict_layers
+    cache._evict_layers = lambda layers, *a, **kw: (launches.append(list(layers)), orig(layers, *a, **kw))[1]
+    cache.compress("alpha", M, buf)
+    assert launches == [list(range(L))], "every layer must go through the single layered launch"
+    for l in range(L):
+        assert cache.get_cache_length(l) == M
+    lens = torch.stack([cache._slabs[l].seg_len for l in range(L)])
+    assert (lens == M).all()
+    for l in check:
+        k, v, lb = snaps[l]
+        sc = lb.float() * (n + 1 - pos)                       # the reference's expression (cache_utils.py:172-174)
+        top = torch.topk(sc, M + 1, dim=-1)
+        tie = top.values[..., M - 1] == top.values[..., M]
+        assert int(tie.sum()) <= 2
+        want = torch.sort(top.indices[..., :M], dim=-1).values
+        K, V, LB, POS = cache[l]
+        ok = ~tie
+        assert torch.equal(POS[ok], want[ok]), f"layer {l}: retained indices differ from torch.topk"
+        assert torch.equal(LB[ok], lb.gather(2, want)[ok])
+        idx = want.unsqueeze(-1).expand(-1, -1, -1, 128)
+        assert torch.equal(K[ok], k.gather(2, idx)[ok]) and torch.equal(V[ok], v.gather(2, idx)[ok])
 
 
 def test_config4_ragged_lognormal_budgets():

@@ -385,3 +385,73 @@ def test_layers_of_different_capacity_share_a_budget(strategy):
     d.ref.compress(**kw); d.cache.compress(**kw)
     _assert_no_tie_at_a_cut(snap, d.ref)
     _same(d.cache, d.ref)
+
+
+@pytest.mark.parametrize("cls", ["batched", "single"])
+@pytest.mark.parametrize("alpha_threshold", [0.05, 0.6, 0.9, 0.45])
+def test_threshold_is_compared_in_the_score_dtype(cls, alpha_threshold):
+    """scores >= torch.log(torch.tensor(a)) with bf16 scores compares against the threshold ROUNDED to bf16
+    (cache_utils.py:462, 893): a token whose bf16 score equals bf16(log a) is kept even where bf16(log a) lies below the
+    fp32 logarithm (a = 0.05, 0.6, 0.9).  Such tokens are planted: the newest token has age 2, so log beta =
+    bf16(log a) / 2 gives exactly that score."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, DynamicBudgetTrimKVCache
+    B, H, L, n = (2, 3, 2, 60) if cls == "batched" else (1, 4, 2, 60)
+    cache, ref = (BatchedDynamicBudgetTrimKVCache(), BatchedRaggedCacheRef()) if cls == "batched" else (DynamicBudgetTrimKVCache(), SingleRaggedCacheRef())
+    gen = torch.Generator().manual_seed(int(alpha_threshold * 100))
+    thr16 = torch.log(torch.tensor(alpha_threshold)).to(torch.bfloat16)
+    pos = torch.arange(n)
+    planted = 0
+    for l in range(L):
+        k, v = draw_kv(gen, B, H, n)
+        lb = draw_log_beta(gen, B, H, n, mu=4.0, sigma=1.5, dtype=torch.bfloat16)
+        lb[:, ::2, -1] = thr16 / 2          # score of the newest token of every other head == bf16(log a) exactly
+        lb[:, 1::2, -2] = thr16 / 3         # age 3: 3 * (thr/3) rounds to thr or to a neighbour -- either side of the cut
+        planted += B * ((H + 1) // 2)
+        ref.update(k, v, lb, pos, l)
+        cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), l)
+    kw = dict(strategy="alpha_threshold", memory_size=8, buffer_size=2, alpha_threshold=alpha_threshold)
+    ref.compress(**kw)
+    cache.compress(**kw)
+    planted_segs = [b * H + h for b in range(B) for h in range(0, H, 2)]
+    kept_newest = sum(int(layer[seg][-1]) == n - 1 for layer in ref.segment_positions() for seg in planted_segs if layer[seg].numel())
+    assert kept_newest == planted, "the oracle itself must keep the planted boundary tokens"
+    _same(cache, ref)
+    assert 0 < ref.get_total_cached_tokens() < L * B * H * n
+
+
+def test_zero_budgets_keep_nothing():
+    """A per-head budget of 0 empties the head (topk with k = 0, cache_utils.py:508-521): lengths, the host mirror,
+    cu_seqlens and later appends must all agree; through the classes and through the raw C entry point with keep = 0."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, _lib as Lb
+    B, H, L, n = 2, 4, 2, 50
+    budgets = np.array([0, 7, 50, 0, 1, 0, 49, 12], dtype=np.int64)
+    d = _Driver(BatchedDynamicBudgetTrimKVCache(), BatchedRaggedCacheRef(), B, H, L, seed=13)
+    d.cache.set_budgets(budgets)
+    d.append(n)
+    q_idx = d.ref.get_seq_length() + 1
+    for l in range(L):
+        cu = d.ref.cu_seqlens_k[l]
+        mask = torch.ones(d.ref.key_cache[l].shape[0], dtype=torch.bool)
+        for seg in range(B * H):
+            lo, hi = int(cu[seg]), int(cu[seg + 1])
+            kb = int(budgets[seg])
+            if hi - lo > kb:
+                sc = (q_idx - d.ref.kv_positions[l][lo:hi, 0]) * d.ref.retention_weights[l][lo:hi, 0]
+                m = torch.zeros(hi - lo, dtype=torch.bool)
+                if kb:
+                    m[torch.topk(sc, kb).indices] = True
+                mask[lo:hi] = m
+        d.ref._apply_mask(l, mask, B * H)
+    d.cache.evict_to_budgets(buffer_size=0)
+    assert d.cache.head_lens[0].cpu().tolist() == budgets.tolist()
+    _same(d.cache, d.ref)
+    d.append(1)                      # an emptied head takes new rows at row 0
+    _same(d.cache, d.ref)
+    # raw entry point: keep = 0 for every segment
+    slab = d.cache._slabs[0]
+    lib = Lb.load()
+    rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                          slab.nseg, slab.cap, slab.D, Lb.BF16, Lb.F32, 0, None, 0, 1000, 0, 1, 0, slab.max_len, None, 0, None, 0,
+                          Lb.current_stream(torch.device(DEV)))
+    Lb.check(rc, "trimkv_evict")
+    assert slab.seg_len.cpu().tolist() == [0] * slab.nseg

@@ -281,3 +281,45 @@ def test_ragged_scores_stay_in_log_beta_dtype():
     age = bf16_round((70001 - pos.numpy()).astype(np.float32))
     want = bf16_round((age.astype(np.float64) * lb.float().numpy().astype(np.float64)).astype(np.float32))
     assert np.array_equal(got.float().numpy(), want)
+
+
+def _bf16_round(x):
+    """float -> nearest-even bf16, with integer arithmetic on the bit pattern (no torch)."""
+    u = np.float32(x).view(np.uint32)
+    u = np.uint32(u + np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1)))
+    return (u & np.uint32(0xFFFF0000)).view(np.float32)
+
+
+@pytest.mark.parametrize("alpha_threshold", [0.05, 0.6, 0.9, 0.45])
+@pytest.mark.parametrize("cls", [BatchedRaggedCacheRef, SingleRaggedCacheRef])
+def test_threshold_compares_in_the_score_dtype(cls, alpha_threshold):
+    """cache_utils.py:462, 893: `scores >= torch.log(torch.tensor(a))` on bf16 scores compares against bf16(log a) (a 0-dim
+    fp32 tensor does not promote a bf16 tensor).  Pinned with bit-level bf16 arithmetic in numpy: a token is kept iff
+    bf16(bf16(age) * log beta) >= bf16(log a); tokens with a score of exactly bf16(log a) are planted (age 2)."""
+    B = 2 if cls is BatchedRaggedCacheRef else 1
+    H, n = 3, 40
+    rng = np.random.default_rng(int(alpha_threshold * 1000))
+    thr16 = _bf16_round(np.log(np.float32(alpha_threshold)))
+    k = torch.from_numpy(rng.standard_normal((B, H, n, 8)).astype(np.float32)).to(torch.bfloat16)
+    lb = torch.nn.functional.logsigmoid(torch.from_numpy((rng.standard_normal((B, H, n)) * 1.5 + 4.0).astype(np.float32))).to(torch.bfloat16)
+    lb[:, :, -1] = float(thr16) / 2
+    assert float(lb[0, 0, -1]) * 2 == float(thr16)
+    ref = cls()
+    ref.update(k, k.clone(), lb, torch.arange(n), 0)
+    ref.compress("alpha_threshold", 4, 1, alpha_threshold=alpha_threshold)
+    got = ref.segment_positions()[0]
+    lbf = lb.float().numpy()
+    on_the_cut = 0
+    for b in range(B):
+        for h in range(H):
+            want = []
+            for i in range(n):
+                sc = _bf16_round(_bf16_round(np.float32(n + 1 - i)) * lbf[b, h, i])
+                on_the_cut += int(sc == thr16)
+                if sc >= thr16:
+                    want.append(i)
+            assert got[b * H + h].tolist() == want
+            assert want[-1] == n - 1
+    assert on_the_cut >= B * H
+    if alpha_threshold in (0.05, 0.6, 0.9):     # the cases where an fp32 comparison would drop the planted tokens
+        assert np.float32(thr16) < np.log(np.float32(alpha_threshold))

@@ -620,6 +620,13 @@ class _RaggedCache(_SlabBacked):
             return _lib.SCORE_KNORM_ALPHA
         raise ValueError(f"Unknown compression strategy: {strategy}")
 
+    @staticmethod
+    def _log_threshold(alpha_threshold: float, score_dtype) -> float:
+        """``log(alpha_threshold)`` as the reference's comparison sees it: ``scores >= torch.log(torch.tensor(a))``
+        (cache_utils.py:462, 893) compares in the scores' dtype (a 0-dim fp32 tensor does not promote a bf16/fp16
+        tensor), so the threshold is rounded to that dtype first."""
+        return float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)).to(score_dtype))
+
     def _ptr_table(self, tensors: List[torch.Tensor], device) -> torch.Tensor:
         return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64).to(device)
 
@@ -895,7 +902,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             layers = list(range(num_layers))
             threshold = None
             if "threshold" in strategy:
-                threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
+                threshold = self._log_threshold(alpha_threshold, self._slabs[layers[0]].lb.dtype)
             thr, take, tie_base, _ = self._group_select(layers, H, num_layers * H * memory_size, strategy, threshold)
             self._compact_layers(layers, H, thr, take, tie_base, strategy)
             self._refresh(layers)
@@ -951,7 +958,7 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
         if floor_budget_ratio == 0:
             threshold = None
             if "threshold" in strategy:
-                threshold = float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)))
+                threshold = self._log_threshold(alpha_threshold, self._slabs[layers[0]].lb.dtype)
             thr, take, tie_base, _ = self._group_select(layers, H, total_budget, strategy, threshold)
             self._compact_layers(layers, H, thr, take, tie_base, strategy)
             self._refresh(layers)

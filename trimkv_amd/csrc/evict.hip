@@ -238,7 +238,7 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
 
 struct EvictArgs {
     char* k_slab; char* v_slab; char* lb_slab; int64_t* pos_slab; int32_t* seg_len;
-    int nseg, cap, row_bytes, lpr_shift, kv_dtype, lb_dtype;
+    int nseg, cap, max_len, row_bytes, lpr_shift, kv_dtype, lb_dtype;
     int keep; const int32_t* keep_per_seg; int slack;
     int64_t q_idx; int strategy, rounding, sliding_window;
     int32_t* kept_idx; int kept_stride;
@@ -275,12 +275,17 @@ __global__ __launch_bounds__(EV_THREADS) void evict_kernel(EvictArgs a) {
     select_layer(a);
     const int seg = blockIdx.x;
     const int n = a.seg_len[seg];
-    if (n <= 0 || n > a.cap) return;  // nothing cached, or a corrupt length: touch nothing
+    // nothing cached, a corrupt length, or more rows than the caller's bound (which sized the key array): touch nothing
+    if (n <= 0 || n > a.cap || n > a.max_len) return;
     int want = 0;
     if (SELECT) {
         want = a.keep_per_seg ? a.keep_per_seg[seg] : a.keep;
         if (want < 0) want = 0;
         if (n <= want || n < want + a.slack) return;  // uniform across the workgroup
+        if (want == 0) {  // a budget of zero keeps nothing (topk with k = 0): no selection, no rows to move
+            if (threadIdx.x == 0) a.seg_len[seg] = 0;
+            return;
+        }
     }
     uint32_t* keys = LDS_KEYS ? lds_keys : a.ws_keys + (int64_t)seg * a.ws_stride;
 
@@ -643,6 +648,7 @@ static int lpr_shift_of(int row_bytes) {
 template <bool SELECT>
 static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st, int nlayers = 1) {
     const size_t key_bytes = (size_t)max_len * 4;
+    a.max_len = max_len;
     if (key_bytes <= (size_t)EV_LDS_KEY_BYTES) {
         // allow more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per workgroup): once per device and
         // instantiation; the flag is only ever set, so a race repeats the call at worst
