@@ -303,6 +303,22 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
                        int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * trimkv_decode_attn_static -- trimkv_decode_attn for callers that cannot allocate device memory (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as trimkv_decode_attn without `workspace`: the split-K partials go to a fixed array of
+ * TRIMKV_DECODE_ATTN_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process ends) and the
+ * call allocates nothing.  A call whose partials need more (trimkv_decode_attn_workspace(...) bytes) is refused with
+ * TRIMKV_ERR_WORKSPACE and launches nothing.  The first call on a device looks the array's address up (no
+ * allocation); make that call outside a graph capture.  All calls on one GPU share the array: calls that may overlap
+ * (different streams without ordering, several host threads) race on it and must be ordered by the caller.
+ */
+#define TRIMKV_DECODE_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
+int trimkv_decode_attn_static(const void* q, void* out, const void* k_slab, const void* v_slab,
+                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                              int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                              int max_len, int chunk, void* stream);
+
+/*
  * trimkv_prefill_attn -- GQA attention of a block of q_len queries (a prompt or prompt chunk)
  * over every segment's retained K/V, bottom-right causal: query t sees keys j <= n - q_len + t,
  * n = seg_len[seg] (the chunk's own tokens are already appended).  A query that sees no key
