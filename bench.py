@@ -278,6 +278,7 @@ def ragged_main(args):
 
     attn_fn = get_attention_interface("db_attn_flash_batched")
     cache = BatchedDynamicBudgetTrimKVCache()
+    cache.fuse_decode_append = not args.no_fuse
     S0 = int(start.max())
     cache.set_budgets(start)
     for l in range(L):   # ragged initial state: every head keeps its best min(budget, prompt) tokens of a synthetic prompt
@@ -302,7 +303,7 @@ def ragged_main(args):
         for l in range(L):
             kn, vn, lbn, q = pool[l][t % POOL]
             K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
-            n_l = int(cache._slabs[l].lens.sum())
+            n_l = cache._slabs[l].total
             rows += n_l
             if sample:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -349,7 +350,8 @@ def ragged_main(args):
     if events:
         avg_s = sum(e0.elapsed_time(e1) for e0, e1, _ in events) * 1e-3 / len(events)
         avg_b = sum(n * 2 * D * 2 + nseg * 2 * G * D * 2 for _, _, n in events) / len(events)
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false> + decode_attn_merge_kernel<{G}, 16, false>", "achieved": round(avg_b / avg_s / 1e9, 1),
+        targs = f"<{G}, 16, false, {'true' if cache.fuse_decode_append else 'false'}>"
+        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel{targs} + decode_attn_merge_kernel{targs}", "achieved": round(avg_b / avg_s / 1e9, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(avg_b / avg_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(events), "algorithmic_bytes_per_launch": int(avg_b)}
     out_json = {
@@ -379,7 +381,12 @@ def main():
     ap.add_argument("--chunk", type=int, default=0, help="split-K rows per workgroup for decode attention (0 = library default)")
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers (smoke runs only; makes the result invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--event-every", type=int, default=8, help="sample attention launches with HIP events every N steps")
+    ap.add_argument("--no-fuse", action="store_true",
+                    help="launch the append and the attention of a layer separately (trimkv_append + trimkv_decode_attn) instead of "
+                         "letting the attention launch carry the append out (trimkv_append_attend, the cache's fuse_decode_append)")
+    ap.add_argument("--event-every", type=int, default=-1,
+                    help="sample the attention launches of every N-th step with HIP events (0: none; default: about 16 sampled steps, "
+                         "at least every 8th -- recording events costs the host about as much as a launch at the small configs)")
     ap.add_argument("--gate", action="store_true",
                     help="produce log beta with the fused `rg` retention gate (MFMA first linear + epilogue inside the append "
                          "kernel) from a random hidden state per layer instead of appending drawn values; reported as a "
@@ -392,6 +399,8 @@ def main():
                     help="secondary workload: chunked prompt processing at config 5's shape (4096-token chunks); "
                          "with it --steps/--warmup count chunks (defaults 6/2)")
     args = ap.parse_args()
+    if args.event_every < 0:
+        args.event_every = max(8, args.steps // 16)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures ONE GPU: the path shards by batch or KV head without communication, "
               "so a multi-GPU figure is N independent copies of this run; --gpus must be 1.", file=sys.stderr)
@@ -430,6 +439,7 @@ def main():
     # Cycle of the steady state: an eviction takes every head to M rows, the next buf steps attend M+1 .. M+buf rows and the
     # last of them evicts again.  The cache starts one row short of the trigger, so the first warm-up step evicts.
     cache = TrimKVCache()
+    cache.fuse_decode_append = not args.no_fuse
     n0 = M + buf - 1
     pos0 = torch.arange(n0, device=dev)
     for l in range(L):
@@ -474,29 +484,32 @@ def main():
     append_bytes = nseg * (2 * D * 2 + 12)                                          # one K row, one V row, log beta, position
     evict_round_bytes = L * nseg * (12 * (M + buf) + 2 * 12 * M + 2 * 2 * M * D * 2)  # one eviction of every layer, M+buf -> M
 
+    scale = D ** -0.5
+    use_gate = bool(args.gate)
+
     def layers_pass(sample):
-        """Append + attend for every layer: one decode step without its eviction.  Returns the bytes it had to move."""
+        """Append + attend for every layer: one decode step without its eviction.  Returns the bytes it had to move.
+        (The loop body is kept lean: at the small configs the host's time per layer is comparable to the kernels'.)"""
         nonlocal T, tick
         pos = torch.full((1,), T, dtype=torch.int64, device=dev)
-        moved = 0
+        slot = tick % POOL
+        update = cache.update
         for l in range(L):
-            kn, vn, lbn, q = pool[l][tick % POOL]
-            if args.gate:
+            kn, vn, lbn, q = pool[l][slot]
+            if use_gate:
                 lbn = gates[l](hidden_pool[l]).transpose(1, 2)   # LazyLogBeta: finished inside the append kernel
-            K, V, _, _, kw = cache.update(kn, vn, lbn, pos, l)
-            n = cache.get_cache_length(l)
-            moved += attn_bytes(n) + append_bytes
+            K, V, _, _, kw = update(kn, vn, lbn, pos, l)
             if sample:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-                attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+                attn_fn(mod, q, K, V, None, scaling=scale, flash_attn_kwargs=kw)
                 e1.record()
-                events.append((e0, e1, n))
+                events.append((e0, e1, kw["max_len"]))
             else:
-                attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+                attn_fn(mod, q, K, V, None, scaling=scale, flash_attn_kwargs=kw)
         T += 1
         tick += 1
-        return moved
+        return L * (attn_bytes(cache.get_cache_length(0)) + append_bytes)     # every layer holds the same number of rows
 
     def step(sample=False):
         """One full decode step; returns (bytes moved, 1 if it evicted)."""
@@ -530,6 +543,7 @@ def main():
         b_, e_ = step(args.event_every > 0 and t % args.event_every == 0)
         moved_bytes += b_
         evictions += e_
+    enqueue_seconds = time.perf_counter() - t0     # host time to issue the steps; close to `seconds` means the host is the limit
     torch.cuda.synchronize()
     seconds = time.perf_counter() - t0
     window_last_n = window_first_n + args.steps - 1 if amortised else None
@@ -555,10 +569,12 @@ def main():
         durs = [e0.elapsed_time(e1) * 1e-3 for e0, e1, _ in events]
         lens = [n for _, _, n in events]
         avg_s = sum(durs) / len(durs)
-        avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens)
+        fused = cache.fuse_decode_append and not args.gate   # the sampled launch then also writes the new rows
+        avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens) + (append_bytes if fused else 0)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
-        roof = {"bound": "hbm", "kernel": f"decode_attn_kernel<{G}, 16, false>" + ("" if B * Hkv >= 128 else f" + decode_attn_merge_kernel<{G}, 16, false>"), "achieved": round(achieved, 1),
+        targs = f"<{G}, 16, false, {'true' if fused else 'false'}>"
+        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 128 else " + decode_attn_merge_kernel" + targs), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "traffic_measured_in_run": False,
@@ -569,7 +585,7 @@ def main():
                              "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
     parity = attention_gate(cache, c, attn_fn, mod)
     parity.update(evict_parity)
-    timing = {"ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}
+    timing = {"host_enqueue_ms_per_step": round(enqueue_seconds * 1e3 / args.steps, 4), "ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}
     if amortised:
         timing.update({"evictions_timed": "1 (amortised: ms_per_step = ms_append_attend + ms_evict_round / buffer_size)",
                        "window_attended_rows": [window_first_n, window_last_n], "cycle_mean_attended_rows": M + (buf + 1) / 2,
@@ -584,7 +600,10 @@ def main():
         "config": {"workload": f"BASELINE config {args.config} ({c['name']} shape): {L} layers, batch {B}, {Hkv} KV heads, {Hq} query heads, "
                                f"head_dim {D}, memory_size {M}, buffer_size {buf}, steady-state decode (append + attend per layer, "
                                f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
-                   "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(), **timing},
+                   "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(),
+                   "launches_per_layer_step": ("1: append + attend in one launch (trimkv_append_attend)" if cache.fuse_decode_append and not args.gate
+                                               else "2: trimkv_append, trimkv_decode_attn") + ("" if B * Hkv >= 128 else " + split-K merge"),
+                   **timing},
         "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
                      "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                      "cycle_mean_algorithmic_bytes_per_step": int(ab["step"]),

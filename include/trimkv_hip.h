@@ -303,6 +303,31 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
                        int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * trimkv_append_attend -- one decode step of one layer in a single launch: trimkv_append with s_new = 1 followed by
+ * trimkv_decode_attn over the slab rows including the new one.  Replaces, at Q_LEN == 1, TrimKVCache.update
+ * (src/trimkv/cache_utils.py:62-110; flat caches :596-689) plus the attention call that follows it for the same layer
+ * (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:353 -> :365; src/trimkv/attn/flash_attn.py:61-71, 135-145).
+ *
+ * Segment seg = b*kv_heads + h receives row seg_len[seg] from k_new / v_new / lb_new / pos_new at [b][h] (ELEMENT strides
+ * over batch and kv head; head_dim contiguous; pos strides may be 0) and is then attended by query rows seg*group ..
+ * seg*group+group-1 over seg_len[seg] + 1 rows; afterwards seg_len[seg] += 1 and, if cu_seqlens is given,
+ * cu_seqlens[i] += i (cache_utils.py:678-680).  Results are bit-identical to the two separate calls.  K/V rows are the
+ * slab layout only (segment seg starts at row seg*cap).  max_len_after: the caller's bound on the lengths after the
+ * append (<= cap); a segment whose slab is full is left as it is and attends its old rows.  chunk, workspace (size:
+ * trimkv_decode_attn_workspace(nseg, group, head_dim, max_len_after, chunk)) and seg_order as in trimkv_decode_attn; when
+ * segments are split the lengths are advanced by the merge launch.
+ */
+int trimkv_append_attend(const void* q, void* out,
+                         void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                         const int32_t* seg_order, int nseg, int kv_heads, int cap, int head_dim, int group,
+                         int kv_dtype, int lb_dtype,
+                         const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                         const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
+                         const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                         float scale, int max_len_after, int chunk,
+                         void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * trimkv_decode_attn_static -- trimkv_decode_attn for callers that cannot allocate device memory (code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
  * Same arguments and results as trimkv_decode_attn without `workspace`: the split-K partials go to a fixed array of

@@ -34,10 +34,11 @@ def _group_slice(group: int) -> int:
     return max(g for g in range(1, _MAX_GROUP + 1) if group % g == 0)
 
 
-def _workspace(device, nbytes: int) -> Optional[torch.Tensor]:
+def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
+    """Split-K scratch, one buffer per (device, stream): launches that share a buffer must be ordered."""
     if nbytes <= 0:
         return None
-    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    key = (device, _lib.current_stream(device) if stream is None else stream)
     ws = _WS.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -69,6 +70,44 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
                                 _lib.current_stream(query.device))
     _lib.check(rc, "trimkv_decode_attn")
     return out
+
+
+def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: int = 0,
+                  seg_order: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The deferred one-token append of ``slab`` (a cache layer whose ``update`` ran with ``fuse_decode_append``) and the
+    attention over the layer including that token, in one launch: ``trimkv_append_attend``.  ``query`` [nseg*group, D]
+    contiguous -> [nseg*group, D].  Clears the pending append."""
+    lib = _lib.load()
+    nseg, d = slab.B * slab.H, slab.D
+    out = torch.empty_like(query)
+    st = _lib.current_stream(query.device)
+    ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, slab.max_len, chunk)
+    ws = _workspace(query.device, ws_bytes, st) if ws_bytes else None
+    # slab.pending[0] = the new row's addresses and strides, in the order of the entry point's parameters
+    rc = lib.trimkv_append_attend(query.data_ptr(), out.data_ptr(), *slab.ptrs, None if seg_order is None else seg_order.data_ptr(),
+                                  nseg, slab.H, slab.cap, d, group, *slab.codes, *slab.pending[0],
+                                  scale, slab.max_len, chunk, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
+    if rc:
+        _lib.check(rc, "trimkv_append_attend")
+    slab.pending = None
+    return out
+
+
+def _take_pending(kw: Optional[dict], query: torch.Tensor, key: torch.Tensor, group: int, fusable: bool):
+    """The layer whose deferred append this attention call has to carry out, or None.  When the call cannot do it in
+    its own launch (``fusable`` False, a query of another dtype, K that is not the cache's slab) the append is
+    carried out here with the ordinary kernel, so that the rows are in place either way."""
+    pend = kw.get("pending_append") if kw else None
+    if pend is None:
+        return None
+    cache, slab = pend
+    if slab.pending is None:
+        return None
+    if (fusable and group <= _MAX_GROUP and query.is_cuda and query.dtype == slab.k.dtype and key.data_ptr() == slab.k.data_ptr()
+            and query.shape[-1] == slab.D):
+        return slab
+    cache._flush(slab)
+    return None
 
 
 def prefill_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, batch: int, kv_heads: int, group: int,
@@ -113,6 +152,12 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     Hkv, n = key.shape[1], key.shape[2]
     G = Hq // Hkv
     scale = D ** -0.5 if scaling is None else scaling
+    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None)
+    if slab is not None:
+        q2 = query.reshape(B * Hq, D)
+        if not q2.is_contiguous():
+            q2 = q2.contiguous()
+        return append_attend(slab, q2, G, scale).view(B, 1, Hq, D), None, None
     if Q == 1 and attention_mask is None:
         ks = key.stride()
         if not (ks[3] == 1 and ks[2] == D and ks[0] == Hkv * ks[1] and value.stride() == ks and ks[1] % D == 0):
@@ -161,6 +206,13 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
     if num_kv_heads is None:
         num_kv_heads = nseg // batch_size
     G = Hq // num_kv_heads
+    slab = _take_pending(kw, query, key, G, Q == 1 and kw.get("seg_start") is not None)
+    if slab is not None:
+        q2 = query.reshape(B * Hq, D)
+        if not q2.is_contiguous():
+            q2 = q2.contiguous()
+        out = append_attend(slab, q2, G, D ** -0.5, chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"))
+        return out.view(B, 1, Hq, D), None, None
     seg_start = kw.get("seg_start")
     if seg_start is None:  # packed rows, as the reference stores them
         seg_start = cu[:-1]

@@ -89,7 +89,8 @@ class LazyLogBeta:
 class _Slab:
     """Device storage of one layer."""
 
-    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order")
+    __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order",
+                 "pending", "codes", "total")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -102,7 +103,9 @@ class _Slab:
         self.cu = torch.zeros(nseg + 1, dtype=torch.int32, device=device) if ragged else None
         self.lens = np.zeros(nseg, dtype=np.int64)  # exact host mirror of seg_len
         self.max_len = 0
+        self.total = 0  # sum of lens (kept by the ragged caches, which size their split-K chunk from it)
         self.order = None  # ragged caches: segments by decreasing length/budget (dispatch order of the attention launch)
+        self.pending = None  # a one-token append that the next attention call will carry out (see _SlabBacked._defer)
         self._refresh_views()
 
     def _refresh_views(self) -> None:
@@ -113,6 +116,7 @@ class _Slab:
         self.lb3, self.pos3 = self.lb.view(B, H, cap), self.pos.view(B, H, cap)
         self.ptrs = (self.k.data_ptr(), self.v.data_ptr(), self.lb.data_ptr(), self.pos.data_ptr(), self.seg_len.data_ptr(),
                      None if self.cu is None else self.cu.data_ptr())
+        self.codes = (_lib.dtype_code(self.k.dtype), _lib.dtype_code(self.lb.dtype))
 
     @property
     def nseg(self) -> int:
@@ -159,6 +163,11 @@ class _SlabBacked(_CacheBase):
         self.sliding_window_size = 0
         self._budget_hint: Optional[int] = None  # memory_size + buffer_size of the last compress()
         self._ws: Dict[Any, torch.Tensor] = {}
+        # Opt-in: a decode-step update() (one token) leaves its rows to the attention call of the same layer, which then
+        # appends and attends in one launch.  Only for callers whose next reader of what update() returned is this
+        # package's HIP attention (the reference's own call order, modeling_trimkv_qwen3.py:353 -> :365) and who leave the
+        # tensors passed to update() untouched until then.
+        self.fuse_decode_append = False
 
     # ---- storage helpers -------------------------------------------------------------------
     def _workspace(self, nbytes: int, device) -> Optional[torch.Tensor]:
@@ -178,10 +187,65 @@ class _SlabBacked(_CacheBase):
             return need + max(128, need // 8)
         return max(need + max(128, s_new), int(slab.cap * 1.5))
 
+    # ---- one-token appends carried out by the attention launch ---------------------------------
+    def _defer(self, slab: _Slab, k, v, lb, pos) -> bool:
+        """Decode step with ``fuse_decode_append`` on: instead of launching the append, remember the new row; the attention
+        call that follows for this layer appends and attends in one launch (``trimkv_append_attend``).  Anything else that
+        touches the layer first -- another update, an eviction, reading ``key_cache`` -- carries the append out on its own
+        (``_flush``).  Returns False when this update cannot be deferred (the ordinary append runs then)."""
+        if slab.pending is not None:
+            self._flush(slab)
+        if isinstance(lb, LazyLogBeta) or not (k.is_cuda and lb.is_cuda):
+            return False
+        B, H, D = slab.B, slab.H, slab.D
+        if tuple(k.shape) != (B, H, 1, D) or v.shape != k.shape or v.dtype != k.dtype or k.dtype != slab.k.dtype:
+            return False
+        if tuple(lb.shape) != (B, H, 1) or lb.dtype != slab.lb.dtype:
+            return False
+        ks = k.stride()
+        if ks[3] != 1 or (ks[0] | ks[1]) % 8 or v.stride() != ks or (k.data_ptr() | v.data_ptr()) % 16:
+            return False
+        if pos.dtype != torch.int64 or pos.device != k.device:
+            return False
+        if pos.dim() == 1:
+            ps = (0, 0)
+        elif tuple(pos.shape) == (B, H, 1):
+            ps = pos.stride()[:2]
+        else:
+            return False
+        if slab.max_len + 1 > slab.cap:
+            slab.regrow(self._new_capacity(slab, slab.max_len + 1, 1))
+        # [0]: what trimkv_append_attend needs of the new row (addresses, element strides over batch and head);
+        # [1:]: the tensors themselves, kept alive and used by _flush
+        slab.pending = ((k.data_ptr(), v.data_ptr(), ks[0], ks[1], lb.data_ptr(), lb.stride(0), lb.stride(1), pos.data_ptr(), ps[0], ps[1]),
+                        k, v, lb, pos)
+        slab.lens += 1
+        slab.max_len += 1
+        slab.total += slab.lens.size
+        return True
+
+    def _flush(self, slab: Optional[_Slab]) -> None:
+        """Carry out a deferred append with the ordinary append kernel."""
+        if slab is None or slab.pending is None:
+            return
+        _, k, v, lb, pos = slab.pending
+        slab.pending = None
+        slab.lens -= 1
+        slab.max_len -= 1
+        slab.total -= slab.lens.size
+        self._append(self._slabs.index(slab), k, v, lb, pos)
+
+    def _flush_all(self) -> None:
+        for slab in self._slabs:
+            if slab is not None and slab.pending is not None:
+                self._flush(slab)
+
     def _append(self, layer: int, k, v, lb, pos) -> _Slab:
         B, H, S, D = k.shape
         _require_cuda(k, "key_states")
         slab = self._slabs[layer]
+        if slab is not None and slab.pending is not None:
+            self._flush(slab)
         lazy = isinstance(lb, LazyLogBeta)
         lb_dtype = lb.dtype
         if slab is None:
@@ -233,6 +297,7 @@ class _SlabBacked(_CacheBase):
             _lib.check(rc, "trimkv_append")
         slab.lens += S
         slab.max_len += S
+        slab.total += S * slab.lens.size
         return slab
 
     # ---- several layers in one launch ----------------------------------------------------------
@@ -315,6 +380,8 @@ class _DenseViews:
         s = self._c._slabs[layer]
         if s is None:
             return _EMPTY()
+        if s.pending is not None:
+            self._c._flush(s)
         return getattr(s, self._BASE[self._w]).narrow(2, 0, s.max_len)
 
     def __iter__(self):
@@ -347,10 +414,12 @@ class TrimKVCache(_SlabBacked):
     def kv_positions(self):
         return _DenseViews(self, "pos")
 
-    def _layer_tuple(self, layer: int):
+    def _layer_tuple(self, layer: int, flush: bool = True):
         s = self._slabs[layer]
         if s is None:
             return (self.key_cache[layer], self.value_cache[layer], self.retention_weights[layer], self.kv_positions[layer])
+        if flush and s.pending is not None:
+            self._flush(s)
         n = s.max_len
         return (s.k4.narrow(2, 0, n), s.v4.narrow(2, 0, n), s.lb3.narrow(2, 0, n), s.pos3.narrow(2, 0, n))
 
@@ -388,17 +457,26 @@ class TrimKVCache(_SlabBacked):
             if layer_idx == 0:
                 self._seen_tokens += seq_len
             self._ensure_layer(layer_idx)
-            slab = self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
+            slab = self._slabs[layer_idx]
+            if not (seq_len == 1 and self.fuse_decode_append and slab is not None
+                    and self._defer(slab, key_states, value_states, retention_weights, cache_positions)):
+                self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
             self.n_seen_tokens[layer_idx] += seq_len
         slab = self._slabs[layer_idx]
-        extra = {} if slab is None else {"seg_len": slab.seg_len, "max_len": slab.max_len, "seg_cap": slab.cap}
-        return (*self._layer_tuple(layer_idx), extra)
+        if slab is None:
+            return (*self._layer_tuple(layer_idx), {})
+        extra = {"seg_len": slab.seg_len, "max_len": slab.max_len, "seg_cap": slab.cap}
+        if slab.pending is not None:
+            # the last of the max_len rows is not in the slab yet: the attention call that receives this dictionary writes it
+            extra["pending_append"] = (self, slab)
+        return (*self._layer_tuple(layer_idx, flush=False), extra)
 
     def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
                  floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
                  num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
         """Evict every layer that holds ``memory_size + buffer_size`` tokens or more down to
         ``memory_size`` per head (cache_utils.py:140-158)."""
+        self._flush_all()
         num_layers = len(self._slabs) if num_layers is None else num_layers
         assert num_layers == len(self._slabs), "All caches must have the same number of layers"
         first = self._slabs[0] if self._slabs else None
@@ -435,6 +513,7 @@ class TrimKVCache(_SlabBacked):
         ``fp32(log beta) * (seen + 1 - position)`` in temporal order (cache_utils.py:160-198)."""
         strat = self._dense_strategy_code(comrpess_strategy)
         slab = self._slabs[layer_idx]
+        self._flush(slab)
         n = slab.max_len
         if memory_size > n:
             raise RuntimeError(f"selected index k out of range: k={memory_size} > cached tokens {n}")
@@ -455,6 +534,7 @@ class TrimKVCache(_SlabBacked):
     # ---- batch utilities used by HF generation modes (cache_utils.py:112-132) ---------------
     def batch_select_indices(self, indices: torch.Tensor):
         """Only keep ``indices`` along the batch axis (contrastive / beam search)."""
+        self._flush_all()
         for slab in self._slabs:
             if slab is None:
                 continue
@@ -469,6 +549,7 @@ class TrimKVCache(_SlabBacked):
             slab._refresh_views()
 
     def batch_split(self, full_batch_size: int, split_size: int) -> List["TrimKVCache"]:
+        self._flush_all()
         out = []
         for i in range(0, full_batch_size, split_size):
             part = TrimKVCache(max_seq_len=self.max_seq_len, device=self.device)
@@ -485,6 +566,7 @@ class TrimKVCache(_SlabBacked):
                 new.k, new.v, new.lb, new.pos = slab.k[lo:hi], slab.v[lo:hi], slab.lb[lo:hi], slab.pos[lo:hi]
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
                 new.lens, new.max_len, new.order = slab.lens[lo:hi].copy(), slab.max_len, None
+                new.pending, new.total = None, int(new.lens.sum())
                 new._refresh_views()
                 part._slabs.append(new)
             out.append(part)
@@ -492,6 +574,7 @@ class TrimKVCache(_SlabBacked):
 
     # ---- observability (cache_utils.py:200-223) ---------------------------------------------
     def log(self, layer_idx: int = None):
+        self._flush_all()
         logs = {}
         if layer_idx is None:
             for l in range(len(self._slabs)):
@@ -502,6 +585,7 @@ class TrimKVCache(_SlabBacked):
         return logs
 
     def copy_to_device(self, device: str):
+        self._flush_all()
         new = TrimKVCache(max_seq_len=self.max_seq_len, device=device)
         new._seen_tokens = self._seen_tokens
         new.offset = self.offset.to(device)
@@ -517,6 +601,7 @@ class TrimKVCache(_SlabBacked):
             c.k, c.v, c.lb, c.pos = (t.to(device, copy=True) for t in (slab.k, slab.v, slab.lb, slab.pos))
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
             c.lens, c.max_len, c.order = slab.lens.copy(), slab.max_len, None
+            c.pending, c.total = None, slab.total
             c._refresh_views()
             new._slabs.append(c)
         return new
@@ -539,6 +624,8 @@ class _PackedViews:
         s = self._c._slabs[layer]
         if s is None:
             return _EMPTY()
+        if s.pending is not None:
+            self._c._flush(s)
         valid = torch.arange(s.cap, device=s.k.device)[None, :] < s.seg_len[:, None]
         t = getattr(s, self._w)[valid]
         return t if self._w in ("k", "v") else t.unsqueeze(-1)
@@ -569,10 +656,12 @@ class _RaggedCache(_SlabBacked):
 
     @property
     def head_lens(self) -> List[torch.Tensor]:
+        self._flush_all()
         return [_EMPTY() if s is None else s.seg_len for s in self._slabs]
 
     @property
     def cu_seqlens_k(self) -> List[torch.Tensor]:
+        self._flush_all()
         return [_EMPTY() if s is None else s.cu for s in self._slabs]
 
     def get_total_cached_tokens(self) -> int:  # cache_utils.py:253-254, 593-594
@@ -588,17 +677,25 @@ class _RaggedCache(_SlabBacked):
             if layer_idx == 0:
                 self._seen_tokens += S
             self._ensure_layer(layer_idx)
-            slab = self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
+            slab = self._slabs[layer_idx]
+            if not (S == 1 and self.fuse_decode_append and slab is not None
+                    and self._defer(slab, key_states, value_states, retention_weights, cache_positions)):
+                self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
             # on the first call cu starts as zeros and the kernel's "cu[i] += i*S" yields
             # arange(0, nseg*S+1, S), what the reference builds at cache_utils.py:297, 643
             self.n_seen_tokens[layer_idx] += S
         slab = self._slabs[layer_idx]
-        # split-K chunk for ragged lengths: about 512 workgroups over the rows actually cached
-        # (the library's own default assumes every segment is max_len long)
-        chunk = max(512, ((int(slab.lens.sum()) // 512 + 63) // 64) * 64)
+        # split-K chunk for ragged lengths: about 384 pieces over the rows actually cached (the library's own default
+        # assumes every segment is max_len long); measured on 256 lognormal segments (128..8256 rows, 410 k rows): 1088-row pieces 52 us, 832 54.7, 1664 53 -- pieces
+        # long enough to stream, short enough that no compute unit ends up with much more than its share
+        chunk = max(512, ((slab.total // 384 + 63) // 64) * 64)
         kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu,
               "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len, "chunk": chunk,
               "seg_order": slab.order}
+        if slab.pending is not None:
+            # head_lens / cu_seqlens_k still hold the values before this token: the attention call that receives this
+            # dictionary appends the row and advances them in the same launch
+            kw["pending_append"] = (self, slab)
         flat = (slab.k.view(-1, slab.D), slab.v.view(-1, slab.D), slab.lb.view(-1, 1), slab.pos.view(-1, 1))
         return flat, kw
 
@@ -759,6 +856,7 @@ class _RaggedCache(_SlabBacked):
             for i, l in enumerate(layers):
                 self._slabs[l].lens = lens[i].copy()
                 self._slabs[l].max_len = int(lens[i].max())
+                self._slabs[l].total = int(lens[i].sum())
                 if getattr(self, "_budgets_host", None) is None:
                     self._set_dispatch_order(self._slabs[l], lens[i])
 
@@ -788,6 +886,7 @@ class _RaggedCache(_SlabBacked):
         variable-k select the reference reaches through its floor branch
         (cache_utils.py:508-521).  The trigger is evaluated on the host mirror of the lengths and
         again per segment on the device; no host synchronisation happens here."""
+        self._flush_all()
         layers = [l for l in range(len(self._slabs)) if self._slabs[l] is not None] if layers is None else layers
         lib = _lib.load()
         code = self._strategy_code(strategy)
@@ -825,9 +924,11 @@ class _RaggedCache(_SlabBacked):
             _lib.check(rc, "trimkv_build_cu_seqlens")
             slab.lens = np.where(hit, kh, slab.lens)
             slab.max_len = int(slab.lens.max())
+            slab.total = int(slab.lens.sum())
 
     def segment_positions(self):
         """Per layer, per segment: retained absolute positions (host tensors)."""
+        self._flush_all()
         out = []
         for s in self._slabs:
             pos = s.pos.cpu()
@@ -863,6 +964,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
     def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
                  floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
                  num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
+        self._flush_all()
         num_layers = len(self._slabs) if num_layers is None else num_layers
         H = self.num_kv_heads if num_key_value_heads is None else num_key_value_heads
         B = self.batch_size
@@ -934,6 +1036,7 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
     def compress(self, strategy: str = "alpha", memory_size: int = 2048, buffer_size: int = 512,
                  floor_budget_ratio: float = 0., alpha_threshold: float = 0.0, num_layers: Optional[int] = None,
                  num_key_value_heads: Optional[int] = None, skip_layers: int = 0):
+        self._flush_all()
         num_layers = len(self._slabs) if num_layers is None else num_layers
         H = self._slabs[0].nseg if num_key_value_heads is None else num_key_value_heads
         if "layer_wise" in strategy:  # cache_utils.py:356-369, 371-416: one top-k over the whole layer

@@ -1,0 +1,589 @@
+// Single-query GQA attention over ragged per-segment K/V (split-K + merge), gfx950.
+//
+// Replaces flash_attn_varlen_func at Q_LEN == 1 (src/trimkv/attn/flash_attn.py:61-71, 135-145),
+// HF flash_attention_2 on the dense cache (src/trimkv/attn/__init__.py:15-26) and
+// eager_attention_forward (src/trimkv/attn/eager_attn.py:48-73) at decode time.
+//
+// The op is HBM-bound (about 4 flop per byte of K/V), so the kernel is built around the stream:
+//   * a wavefront reads whole 256-byte rows, 16 lanes x 16 bytes per row, 4 rows per load
+//     instruction (1 KiB contiguous), with a ring of register buffers that keeps several tiles of
+//     its K/V stream in flight (the kernel is bound by bytes in flight over latency, not by ALU);
+//   * q.K uses v_dot2_f32_bf16 on the bytes as loaded; the 16-lane partial sums of one tile are
+//     reduced with a transposing DPP butterfly that leaves ONE (row, head) score per lane, so the
+//     softmax costs one exp per lane per tile;
+//   * a wavefront takes 128 rows at a time: all their scores first, one running-max update, then
+//     the V rows; probabilities reach the lanes that hold the matching V rows through LDS as
+//     packed bf16 pairs, and P.V is v_dot2_f32_bf16 over two rows at a time (v_perm_b32
+//     interleaves the rows);
+//   * the four wavefronts of a workgroup own disjoint quarters of the workgroup's rows and merge
+//     (max, sum, accumulator) in LDS; with 128 segments or more (or when the caller's chunk covers
+//     the longest segment) one workgroup covers a whole segment and writes the output itself,
+//     otherwise segments are split and a second, tiny kernel merges the partials;
+//   * rows of 96 or 64 features keep their length in memory: the 16-lane row group then has 12 or 8
+//     loading lanes, the others repeat the last piece against q = 0.
+#pragma once
+#include "common.hip.h"
+
+#include <atomic>
+#include <type_traits>
+
+namespace trimkv {
+
+typedef uint32_t at_u32x4 __attribute__((ext_vector_type(4)));
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+#ifndef TRIMKV_AT_WPE
+#define TRIMKV_AT_WPE 2
+#endif
+#ifndef TRIMKV_AT_WAVES
+#define TRIMKV_AT_WAVES 4
+#endif
+constexpr int AT_WAVES = TRIMKV_AT_WAVES;
+constexpr int AT_THREADS = AT_WAVES * 64;
+constexpr int AT_D = 128;            // head_dim the lane layout is built for; 64 and 96 run zero-padded to it
+constexpr int AT_BLOCK_ROWS = 128;   // rows one wavefront scores before it touches V
+constexpr float AT_NEG = -1.0e30f;   // "minus infinity" that stays finite under subtraction
+
+template <int G>
+struct AttnCfg {
+    static constexpr int NJ = G <= 4 ? 4 : 2;                  // load instructions (of 4 rows) per tile
+    static constexpr int NV = NJ * G;                          // scores per tile per 16-lane row group (<= 16)
+    static constexpr int TILE_ROWS = NJ * 4;
+    static constexpr int NT = AT_BLOCK_ROWS / TILE_ROWS;       // tiles per block
+    static constexpr int PSTRIDE = NV <= 8 ? 8 : 16;           // bf16 slots per (tile, row group) in LDS
+#ifndef TRIMKV_AT_RING
+    static constexpr int RING = (NJ >= 4 || G >= 6) ? 4 : 8;   // register tile buffers: RING-1 tiles in flight per wavefront
+#else
+    static constexpr int RING = TRIMKV_AT_RING;
+#endif
+};
+
+typedef uint32_t __attribute__((may_alias)) u32_alias;  // LDS words written as bf16 halves, read as pairs
+typedef uint16_t __attribute__((may_alias)) u16_alias;
+#define DPP_MOV(v, ctrl) __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, (v)), (ctrl), 0xf, 0xf, false))
+constexpr int DPP_QUAD_XOR1 = 0xB1;       // quad_perm [1,0,3,2]
+constexpr int DPP_QUAD_XOR2 = 0x4E;       // quad_perm [2,3,0,1]
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;
+constexpr int DPP_ROW_ROR8 = 0x128;
+
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+// c + a.lo * b.lo + a.hi * b.hi on packed bf16 (v_dot2_f32_bf16) or fp16 (v_dot2_f32_f16) pairs
+template <bool F16>
+__device__ __forceinline__ float dot2_kv(uint32_t a, uint32_t b, float c) {
+    if constexpr (F16) return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, a), __builtin_bit_cast(f16x2_t, b), c, false);
+    else return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+template <bool F16>
+__device__ __forceinline__ uint16_t to_kv_bits(float f) { return F16 ? f32_to_f16_bits(f) : f32_to_bf16_bits(f); }
+
+// Sum 16 per-lane values over the 16 lanes of a row group, leaving value x(c) in lane c, where
+// x(c) = bit2(c)<<3 | bit0(c)<<2 | bit1(c)<<1 | bit3(c).  Each step halves the values a lane
+// carries: the lane keeps the half its lane bit names and adds the partner's copy of that half.
+__device__ __forceinline__ float reduce16_transposed(float (&v)[16], int c) {
+    const bool b0 = c & 1, b1 = c & 2, b2 = c & 4, b3 = c & 8;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float keep = b2 ? v[i + 8] : v[i], send = b2 ? v[i] : v[i + 8];
+        v[i] = keep + DPP_MOV(send, DPP_ROW_HALF_MIRROR);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float keep = b0 ? v[i + 4] : v[i], send = b0 ? v[i] : v[i + 4];
+        v[i] = keep + DPP_MOV(send, DPP_QUAD_XOR1);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const float keep = b1 ? v[i + 2] : v[i], send = b1 ? v[i] : v[i + 2];
+        v[i] = keep + DPP_MOV(send, DPP_QUAD_XOR2);
+    }
+    const float keep = b3 ? v[1] : v[0], send = b3 ? v[0] : v[1];
+    return keep + DPP_MOV(send, DPP_ROW_ROR8);
+}
+
+// The new token of every segment, for the kernels that append before they attend (APPEND = true): one row per
+// (batch, kv head) of strided [batch][kv_heads][1][...] tensors, the slabs' metadata arrays and the length counters.
+struct AppendPart {
+    const char* k_new; const char* v_new; int64_t kv_sb, kv_sh;   // BYTE strides
+    const void* lb_new; int64_t lb_sb, lb_sh;                     // element strides
+    const int64_t* pos_new; int64_t pos_sb, pos_sh;
+    void* lb_slab; int64_t* pos_slab; int32_t* seg_len; int32_t* cu;
+    int kv_heads, lb_dtype;
+};
+
+struct AttnArgs {
+    const uint4* q; void* out; const uint4* k; const uint4* v;
+    const int32_t* seg_len; const int32_t* seg_start; const int32_t* seg_order;
+    int nseg, cap, max_len, chunk, nsplit, direct;
+    float scale_log2;
+    float* ws_o; float* ws_ml;
+    AppendPart ap;   // read by APPEND kernels only
+};
+
+// Length of segment `seg` as the launch sees it.  APPEND: the stored length is the one before this step's token; the token
+// lands in row n_old (returned through *new_row) unless the slab is full, in which case nothing is appended (-1).
+template <bool APPEND>
+__device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new_row) {
+    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
+    *new_row = -1;
+    if (APPEND) {
+        n = max(n, 0);
+        if (n + 1 <= a.cap && n + 1 <= a.max_len) { *new_row = n; n += 1; }
+    }
+    return max(0, min(n, a.max_len));
+}
+
+// Attention of the G query heads of segment `seg` over its rows [t0, t1): the body shared by both kernels.
+// `direct`: normalise and write the output; otherwise the unnormalised accumulator and (max, sum) go to partial
+// slot `slot` of the workspace.  All 256 threads of the workgroup must call it together (it uses barriers).
+// ROW16: 16-byte pieces per K/V/q row (head_dim / 8).  With fewer than 16, lanes c >= ROW16 of each 16-lane row group
+// re-read the row's last piece and hold q = 0, so they add nothing to the scores; what they accumulate is not stored.
+// APPEND: row `new_row` of the segment (-1: none) is this step's token.  It is read from a.ap.k_new / v_new wherever the
+// stream reaches it, and the wavefront that owns it writes it into the slabs (K, V, log beta, position).
+template <int G, int ROW16, bool F16, bool APPEND>
+__device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base, int new_row) {
+    constexpr int D_REAL = ROW16 * 8;
+    using C = AttnCfg<G>;
+    constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
+
+    __shared__ u32_alias p_lds[AT_WAVES][NT][4][PS / 2];
+    __shared__ uint32_t smax[AT_WAVES][8];
+    __shared__ float so[AT_WAVES][G][AT_D];
+    __shared__ float sm[AT_WAVES][8];
+    __shared__ float sl[AT_WAVES][8];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int c = lane & 15, r = lane >> 4;
+    const int pw = (t1 - t0 + AT_WAVES - 1) / AT_WAVES;
+    const int w0 = t0 + w * pw, w1 = min(t1, w0 + pw);
+
+    const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
+    const int cc = ROW16 == 16 ? c : min(c, ROW16 - 1);
+    const uint4* kp = a.k + row0 * ROW16 + cc;  // ROW16 uint4 per row; this lane's 16-byte column
+    const uint4* vp = a.v + row0 * ROW16 + cc;
+
+    // q is loaded first and waited for right after the first K/V prefetches have been issued (loads return in order, so
+    // that wait leaves the prefetches in flight): q's round trip overlaps the first tiles', and no later wait can be for q.
+    // Were q still outstanding when the block loop starts, the wait at the first q.K (static code, executed by every
+    // block) would have to drain the whole prefetch ring each time.
+    uint4 qv[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        qv[g] = a.q[((int64_t)seg * G + g) * ROW16 + cc];
+        if (ROW16 < 16 && c >= ROW16) qv[g] = make_uint4(0u, 0u, 0u, 0u);
+    }
+    const uint4* knew = nullptr;
+    const uint4* vnew = nullptr;
+    if (APPEND) {
+        const int b = seg / a.ap.kv_heads, h = seg - b * a.ap.kv_heads;
+        const int64_t off = (int64_t)b * a.ap.kv_sb + (int64_t)h * a.ap.kv_sh + ((int64_t)cc << 4);
+        knew = (const uint4*)(a.ap.k_new + off);
+        vnew = (const uint4*)(a.ap.v_new + off);
+        if (new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and stores it
+            // its loads are issued here, behind q and ahead of the first K/V prefetch, so that the wait below covers them
+            const uint4 kn = *knew, vn = *vnew;
+            float lbn = 0.0f;
+            int64_t pn = 0;
+            if (lane == 0) {
+                lbn = load_as_f32(a.ap.lb_new, (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh, a.ap.lb_dtype);
+                pn = a.ap.pos_new[(int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh];
+            }
+            const int64_t dst = row0 + new_row;
+            if (r == 0 && c < ROW16) {
+                ((uint4*)a.k)[dst * ROW16 + c] = kn;
+                ((uint4*)a.v)[dst * ROW16 + c] = vn;
+            }
+            if (lane == 0) {
+                store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
+                a.ap.pos_slab[dst] = pn;
+            }
+        }
+    }
+
+    // which (row-in-tile, head) this lane owns after the transposing reduction
+    const int my_x = ((c & 4) << 1) | ((c & 1) << 2) | (c & 2) | ((c & 8) >> 3);
+    const bool my_valid = my_x < NV;
+    const int my_j = my_x / G, my_g = my_x - my_j * G;
+
+    float o[G][8];
+    float m_run[G];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m_run[g] = AT_NEG;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = 0.0f;
+    }
+    float l_lane = 0.0f;
+
+    auto load_tile = [&](const uint4* base, const uint4* fresh, int row_begin, uint4 (&dst)[NJ]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) {
+            const int row = min(row_begin + j * 4 + r, w1 - 1);  // rows past the end re-read the last one (weight 0)
+            const uint4* src = base + (int64_t)row * ROW16;
+            if (APPEND) src = row == new_row ? fresh : src;      // this step's token comes from the caller's tensor (a select, not a branch)
+            // K/V are read once per step and never again before they have left every cache: a non-temporal load
+            // (streaming hint) moves them about 13 % faster than a plain one on this part
+            const at_u32x4 t = __builtin_nontemporal_load((const at_u32x4*)src);
+            dst[j] = make_uint4(t.x, t.y, t.z, t.w);
+        }
+    };
+
+    if (w0 < w1) {
+        // The wavefront consumes one stream of tiles: for every block of up to 128 rows, its K tiles
+        // (slots 0..NT-1) and then its V tiles (slots NT..2NT-1).  A ring of RING register buffers,
+        // indexed by slot % RING (static: the slot loop is fully unrolled and 2*NT is a multiple of
+        // RING), keeps the next RING-1 tiles of that stream in flight while one is consumed -- K and
+        // V alike, across the softmax and across block boundaries.  Bandwidth here is bytes in
+        // flight over latency, and registers are the cheapest place to park them.
+        constexpr int RING = C::RING, PD = RING - 1;
+        uint4 ring[RING][NJ];
+        float s[NT];
+        float m_mine = AT_NEG;
+        u16_alias* pw16 = (u16_alias*)&p_lds[w][0][0][0];
+
+        auto scores_of_tile = [&](int t, int blk, const uint4 (&kt)[NJ]) __attribute__((always_inline)) {
+            float part[16];
+#pragma unroll
+            for (int x = 0; x < 16; ++x) part[x] = 0.0f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                for (int g = 0; g < G; ++g) {
+                    float acc = dot2_kv<F16>(kt[j].x, qv[g].x, 0.0f);
+                    acc = dot2_kv<F16>(kt[j].y, qv[g].y, acc);
+                    acc = dot2_kv<F16>(kt[j].z, qv[g].z, acc);
+                    acc = dot2_kv<F16>(kt[j].w, qv[g].w, acc);
+                    part[j * G + g] = acc;
+                }
+            }
+            const float val = reduce16_transposed(part, c);
+            const int row = blk + t * TILE_ROWS + my_j * 4 + r;
+            return (my_valid && row < w1) ? val * a.scale_log2 : AT_NEG;
+        };
+        // ntiles: tiles of this block that were scored (the rest of s[] is not read)
+        auto softmax_of_block = [&](auto ntb_c, int nrows) __attribute__((always_inline)) {
+            constexpr int NTB = decltype(ntb_c)::value;
+            float lmax = AT_NEG;
+#pragma unroll
+            for (int t = 0; t < NTB; ++t) lmax = fmaxf(lmax, s[t]);
+            if (lane < 8) smax[w][lane] = float_key(AT_NEG);
+            if (my_valid) atomicMax(&smax[w][my_g], float_key(lmax));
+            float alpha_mine = 1.0f;
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const float mb = key_float(smax[w][g]);
+                const float m_new = fmaxf(m_run[g], mb);
+                const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_new);
+                m_run[g] = m_new;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[g][e] *= alpha;
+                if (g == my_g) { alpha_mine = alpha; m_mine = m_new; }
+            }
+            l_lane *= alpha_mine;
+#pragma unroll
+            for (int t = 0; t < NTB; ++t) {
+                if (t * TILE_ROWS < nrows) {
+                    const float p = my_valid ? __builtin_amdgcn_exp2f(s[t] - m_mine) : 0.0f;
+                    l_lane += p;
+                    if (my_valid) pw16[(t * 4 + r) * PS + my_g * NJ + my_j] = to_kv_bits<F16>(p);
+                }
+            }
+        };
+        auto accumulate_tile = [&](int t, const uint4 (&vt)[NJ]) __attribute__((always_inline)) {
+            uint32_t pd[NV / 2];
+#pragma unroll
+            for (int i = 0; i < NV / 2; ++i) pd[i] = p_lds[w][t][r][i];
+#pragma unroll
+            for (int u = 0; u < NJ / 2; ++u) {
+                const uint4 ra = vt[2 * u], rb = vt[2 * u + 1];
+                const uint32_t va[4] = {ra.x, ra.y, ra.z, ra.w};
+                const uint32_t vv[4] = {rb.x, rb.y, rb.z, rb.w};
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t lo = __builtin_amdgcn_perm(vv[i], va[i], 0x05040100u);  // rows (2u, 2u+1), element 2i
+                    const uint32_t hi = __builtin_amdgcn_perm(vv[i], va[i], 0x07060302u);  // rows (2u, 2u+1), element 2i+1
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const uint32_t pp = pd[(g * NJ) / 2 + u];
+                        o[g][2 * i] = dot2_kv<F16>(lo, pp, o[g][2 * i]);
+                        o[g][2 * i + 1] = dot2_kv<F16>(hi, pp, o[g][2 * i + 1]);
+                    }
+                }
+            }
+        };
+
+        // One block of NTB tiles (NTB*TILE_ROWS rows, `nrows` of them real) as straight-line code:
+        // slots 0..NTB-1 are its K tiles, NTB..2NTB-1 its V tiles.  Loads are never placed under a
+        // branch: the compiler can count outstanding loads exactly (s_waitcnt vmcnt(N), N > 0:
+        // "wait for this tile, leave the prefetched ones in flight") only when every path issues
+        // the same loads.  Rows are clamped to the wavefront's last row, so a load past the end is
+        // legal and re-reads cached bytes; its scores are masked.
+        // CHAINED: the first PD slots are already in flight and the block prefetches the first PD
+        // slots of the block that follows it (the steady-state loop over full blocks).
+        auto run_block = [&](auto ntb_c, auto chained_c, int blk, int nrows) __attribute__((always_inline)) {
+            constexpr int NTB = decltype(ntb_c)::value;
+            constexpr bool CHAINED = decltype(chained_c)::value;
+            constexpr int SL = 2 * NTB;
+            static_assert(!CHAINED || (SL % RING == 0 && PD <= NTB), "chained blocks need ring-aligned slots");
+            auto load_slot = [&](int slot, int base_row, uint4 (&dst)[NJ]) __attribute__((always_inline)) {
+                if (slot < NTB) load_tile(kp, knew, base_row + slot * TILE_ROWS, dst);
+                else load_tile(vp, vnew, base_row + (slot - NTB) * TILE_ROWS, dst);
+            };
+            if (!CHAINED) {
+#pragma unroll
+                for (int sl = 0; sl < (PD < SL ? PD : SL); ++sl) load_slot(sl, blk, ring[sl % RING]);
+            }
+#pragma unroll
+            for (int sl = 0; sl < SL; ++sl) {
+                const int ahead = sl + PD;
+                if (ahead < SL) load_slot(ahead, blk, ring[ahead % RING]);
+                else if (CHAINED) load_slot(ahead - SL, blk + NTB * TILE_ROWS, ring[ahead % RING]);
+                // keep the prefetch where it is: left alone, the scheduler sinks these loads past
+                // the arithmetic to shorten live ranges, which empties the pipeline
+                __builtin_amdgcn_sched_barrier(0);
+                if (sl == NTB) softmax_of_block(ntb_c, nrows);
+                if (sl < NTB) {
+                    s[sl] = scores_of_tile(sl, blk, ring[sl % RING]);
+                } else if (CHAINED || (sl - NTB) * TILE_ROWS < nrows) {
+                    accumulate_tile(sl - NTB, ring[sl % RING]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        using std::integral_constant;
+        using std::true_type;
+        using std::false_type;
+
+#pragma unroll
+        for (int sl = 0; sl < PD; ++sl) load_tile(kp, knew, w0 + sl * TILE_ROWS, ring[sl % RING]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
+        int blk = w0;
+#pragma unroll 1
+        for (; blk + AT_BLOCK_ROWS <= w1; blk += AT_BLOCK_ROWS)
+            run_block(integral_constant<int, NT>{}, true_type{}, blk, AT_BLOCK_ROWS);
+        // the tail (< 128 rows): the smallest power-of-two block that covers it, one pipelined pass
+        const int rest = w1 - blk;
+        if (rest > 0) {
+            const int need = (rest + TILE_ROWS - 1) / TILE_ROWS;  // 1 .. NT tiles
+            if (need <= 1) run_block(integral_constant<int, 1>{}, false_type{}, blk, rest);
+            else if (need <= 2) run_block(integral_constant<int, 2>{}, false_type{}, blk, rest);
+            else if (need <= 4) run_block(integral_constant<int, 4>{}, false_type{}, blk, rest);
+            else if (need <= 8) run_block(integral_constant<int, (NT >= 8 ? 8 : NT)>{}, false_type{}, blk, rest);
+            else run_block(integral_constant<int, NT>{}, false_type{}, blk, rest);
+        }
+    }
+
+    // ---- merge the four row groups of a wavefront, then the four wavefronts ----
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float x = o[g][e];
+            x += __shfl_xor(x, 16, 64);
+            x += __shfl_xor(x, 32, 64);
+            o[g][e] = x;
+        }
+    }
+    if (lane < 8) sl[w][lane] = 0.0f;
+    if (my_valid && l_lane != 0.0f) atomicAdd(&sl[w][my_g], l_lane);
+    if (r == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) so[w][g][c * 8 + e] = o[g][e];
+        }
+    }
+    if (lane == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) sm[w][g] = m_run[g];
+    }
+    __syncthreads();
+    if (APPEND && direct && tid == 0 && new_row >= 0) {
+        // one workgroup per segment: every wavefront read the old length before the barrier above, nobody else reads it
+        a.ap.seg_len[seg] = new_row + 1;
+        if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;     // cu[i] += i per appended token (cache_utils.py:678-680)
+    }
+    for (int i = tid; i < G * AT_D; i += AT_THREADS) {
+        const int g = i / AT_D, d = i - g * AT_D;
+        float mx = AT_NEG;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) mx = fmaxf(mx, sm[ww][g]);
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) {
+            const float f = __builtin_amdgcn_exp2f(sm[ww][g] - mx);
+            acc += f * so[ww][g][d];
+            lsum += f * sl[ww][g];
+        }
+        if (direct) {
+            const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = to_kv_bits<F16>(y);
+        } else {
+            const int64_t slot = slot_base * G + g;
+            a.ws_o[slot * AT_D + d] = acc;
+            if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
+        }
+    }
+}
+
+template <int G, int ROW16, bool F16, bool APPEND>
+__global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_kernel(AttnArgs a) {
+    // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
+    // axis so that consecutive ids are different segments: with the split as the fast axis and 8
+    // splits, every "split 0" workgroup would land on the same XCD, and ragged lengths (most
+    // segments need one or two splits) would leave most of the chip idle.
+    // High splits exist only for the longest segments; they are dispatched first so that the few
+    // long segments do not form the tail of the launch.
+    // seg_order (optional): the segment each grid column works on, longest first, so that with very uneven lengths
+    // the long segments are dispatched first instead of forming the tail of the launch.
+    int seg = blockIdx.x;
+    if (a.seg_order) seg = min(max(a.seg_order[seg], 0), a.nseg - 1);
+    const int split = (int)gridDim.y - 1 - (int)blockIdx.y;
+    int new_row;
+    const int n = segment_rows<APPEND>(a, seg, &new_row);
+    const int nsp = (n + a.chunk - 1) / a.chunk;
+    if (split >= nsp) {
+        if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
+            for (int i = threadIdx.x; i < G * ROW16 * 8; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * (ROW16 * 8) + i] = 0;
+        }
+        return;
+    }
+    const int rps = (n + nsp - 1) / nsp;
+    const int t0 = split * rps, t1 = min(n, t0 + rps);
+    attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split, new_row);
+}
+
+// Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
+// splits first (independent loads), then the accumulators.  A separate launch on purpose: the
+// kernel boundary is what makes partials written on one XCD visible on another; doing the same
+// inside one kernel needs device-scope fences (an L2 write-back and invalidate per workgroup on
+// this part), which costs far more than the launch.
+template <int G, int ROW16, bool F16, bool APPEND>
+__global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
+    const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
+    int new_row;
+    const int n = segment_rows<APPEND>(a, seg, &new_row);
+    if (APPEND) {
+        // The split workgroups of the main launch all read the old length, so it is advanced here, by the only workgroup of
+        // this launch that reads it, once all of its threads have.
+        __syncthreads();
+        if (threadIdx.x == 0 && new_row >= 0) {
+            a.ap.seg_len[seg] = new_row + 1;
+            if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;
+        }
+    }
+    const int nsp = (n + a.chunk - 1) / a.chunk;
+    const int64_t slot0 = ((int64_t)seg * a.nsplit) * G + g;
+    // every load of a batch of 8 splits is issued before anything is used: one memory round trip per batch
+    float mx = AT_NEG, acc = 0.0f, lsum = 0.0f;
+    for (int sp0 = 0; sp0 < nsp; sp0 += 8) {
+        float m8[8], l8[8], o8[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int64_t slot = slot0 + (int64_t)min(sp0 + u, nsp - 1) * G;   // past the end: the last split again (weight 0 below)
+            m8[u] = a.ws_ml[slot * 2];
+            l8[u] = a.ws_ml[slot * 2 + 1];
+            o8[u] = a.ws_o[slot * AT_D + d];
+        }
+        float bm = AT_NEG;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) bm = fmaxf(bm, sp0 + u < nsp ? m8[u] : AT_NEG);
+        const float m_new = fmaxf(mx, bm);
+        const float rescale = __builtin_amdgcn_exp2f(mx - m_new);
+        acc *= rescale;
+        lsum *= rescale;
+        mx = m_new;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float f = sp0 + u < nsp ? __builtin_amdgcn_exp2f(m8[u] - mx) : 0.0f;
+            acc += f * o8[u];
+            lsum += f * l8[u];
+        }
+    }
+    const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+    if (d < ROW16 * 8) ((uint16_t*)a.out)[((int64_t)seg * G + g) * (ROW16 * 8) + d] = to_kv_bits<F16>(y);
+}
+
+static int pick_chunk(int nseg, int max_len) {
+    // One workgroup per segment streams at full rate already with 128 segments (a workgroup keeps 12 tiles in flight).  In a
+    // decode step over 28 layers (nothing of a layer survives in the last-level cache until its next turn) two splits plus
+    // the merge launch took 25.6 + 3.9 us per layer at 128 segments x 2112 rows against 28.6 us for whole segments; a
+    // single layer replayed from the last-level cache had suggested the opposite.  With fewer segments they are cut so
+    // that about 256 workgroups exist, but not below 512 rows each (one full block per wavefront).
+    const int whole = ((max_len + 63) / 64) * 64;
+    if (nseg >= 128) return whole;
+    const int nsplit = (256 + nseg - 1) / nseg;
+    int chunk = (((max_len + nsplit - 1) / nsplit + 63) / 64) * 64;
+    if (chunk < 512) chunk = 512;
+    return chunk < whole ? chunk : whole;
+}
+
+template <int G, int ROW16, bool F16, bool APPEND>
+static void launch_attn_rows(const AttnArgs& a, hipStream_t st) {
+    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16, F16, APPEND>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
+    if (!a.direct) hipLaunchKernelGGL((decode_attn_merge_kernel<G, ROW16, F16, APPEND>), dim3(a.nseg), dim3(G * AT_D), 0, st, a);
+}
+
+template <int G, bool F16, bool APPEND>
+static void launch_attn_dtype(const AttnArgs& a, int head_dim, hipStream_t st) {
+    if (head_dim == 128) launch_attn_rows<G, 16, F16, APPEND>(a, st);
+    else if (head_dim == 96) launch_attn_rows<G, 12, F16, APPEND>(a, st);
+    else launch_attn_rows<G, 8, F16, APPEND>(a, st);
+}
+
+template <int G, bool APPEND>
+static void launch_attn(const AttnArgs& a, int head_dim, int dtype, hipStream_t st) {
+    if (dtype == TRIMKV_F16) launch_attn_dtype<G, true, APPEND>(a, head_dim, st);
+    else launch_attn_dtype<G, false, APPEND>(a, head_dim, st);
+}
+
+// group = 1..8 -> the matching instantiation
+template <bool APPEND>
+static void launch_attn_group(const AttnArgs& a, int group, int head_dim, int dtype, hipStream_t st) {
+    switch (group) {
+        case 1: launch_attn<1, APPEND>(a, head_dim, dtype, st); break;
+        case 2: launch_attn<2, APPEND>(a, head_dim, dtype, st); break;
+        case 3: launch_attn<3, APPEND>(a, head_dim, dtype, st); break;
+        case 4: launch_attn<4, APPEND>(a, head_dim, dtype, st); break;
+        case 5: launch_attn<5, APPEND>(a, head_dim, dtype, st); break;
+        case 6: launch_attn<6, APPEND>(a, head_dim, dtype, st); break;
+        case 7: launch_attn<7, APPEND>(a, head_dim, dtype, st); break;
+        default: launch_attn<8, APPEND>(a, head_dim, dtype, st); break;
+    }
+}
+
+// Argument checks and split-K set-up shared by the entry points; fills `a` except for a.ap.
+static int prepare_attn(const char* fn, AttnArgs& a, const void* q, void* out, const void* k_slab, const void* v_slab,
+                        const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                        int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                        int max_len, int chunk, void* workspace, size_t workspace_bytes) {
+    if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if (dtype != TRIMKV_BF16 && dtype != TRIMKV_F16) return fail(TRIMKV_ERR_DTYPE, "%s: K/V/q must be bf16 or fp16 (dtype=%d)", fn, dtype);
+    if (head_dim != 128 && head_dim != 96 && head_dim != 64) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: head_dim must be 64, 96 or 128 (got %d)", fn, head_dim);
+    if (group < 1 || group > 8) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: group must be in [1, 8] (got %d)", fn, group);
+    if (nseg <= 0 || cap <= 0 || max_len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d cap=%d max_len=%d", fn, nseg, cap, max_len);
+    if (!seg_start && max_len > cap) return fail(TRIMKV_ERR_CAPACITY, "%s: max_len %d exceeds capacity %d", fn, max_len, cap);
+    if (((uintptr_t)q | (uintptr_t)out | (uintptr_t)k_slab | (uintptr_t)v_slab) & 15) return fail(TRIMKV_ERR_SHAPE, "%s: q/out/K/V must be 16-byte aligned", fn);
+    if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
+    if (chunk % 64) return fail(TRIMKV_ERR_SHAPE, "%s: chunk must be a multiple of 64 (got %d)", fn, chunk);
+    a.q = (const uint4*)q; a.out = out; a.k = (const uint4*)k_slab; a.v = (const uint4*)v_slab;
+    a.seg_len = seg_len; a.seg_start = seg_start; a.seg_order = seg_order; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
+    a.nsplit = (max_len + chunk - 1) / chunk;
+    if (a.nsplit > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: max_len/chunk = %d splits exceeds the grid limit 65535", fn, a.nsplit);
+    a.direct = a.nsplit <= 1;
+    a.scale_log2 = scale * 1.4426950408889634f;
+    a.ws_o = nullptr; a.ws_ml = nullptr;
+    a.ap = AppendPart{};
+    if (!a.direct) {
+        const size_t need = (size_t)nseg * a.nsplit * group * (AT_D + 2) * sizeof(float);   // partial rows are padded to 128 features
+        if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+        if ((uintptr_t)workspace & 15) return fail(TRIMKV_ERR_SHAPE, "%s: workspace must be 16-byte aligned", fn);
+        a.ws_o = (float*)workspace;
+        a.ws_ml = a.ws_o + (size_t)nseg * a.nsplit * group * AT_D;
+    }
+    return TRIMKV_OK;
+}
+
+}  // namespace trimkv
