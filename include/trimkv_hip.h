@@ -166,13 +166,16 @@ int trimkv_evict(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, i
  * [nlayers*nseg] receives how many equal-to-cut tokens precede each segment in that order.
  * With use_threshold != 0 no selection is done: a token is kept iff score >= threshold_score
  * (cache_utils.py:462, 893; -inf keeps everything) and budget is ignored.
+ * first_kept (optional, [nlayers*nseg]) receives 1 where the segment's oldest token (row 0) is among the kept ones and 0
+ * elsewhere: what the single-sequence floor branch needs to reproduce bucketize(right=False) against the inclusive
+ * cumulative lengths (cache_utils.py:496), which credits a chosen first row to the previous head.
  */
 int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
                            const void* const* k_slabs, const int32_t* const* seg_lens,
                            int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                            int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                            int64_t q_idx, int strategy, int rounding,
-                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept,
                            void* stream);
 
 /*
@@ -180,14 +183,14 @@ int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* po
  * instead of one per group across the layers: the layer-wise strategies of the flat caches
  * (cache_utils.py:356-416, 719-834), every layer of one `compress` in one launch of
  * ngroups x nlayers workgroups.  Same arguments; thr_key and tie_take are [nlayers][ngroups],
- * tie_base and new_len [nlayers][nseg], ties counted inside each layer.
+ * tie_base, new_len and first_kept [nlayers][nseg], ties counted inside each layer.
  */
 int trimkv_group_threshold_each_layer(const void* const* lb_slabs, const int64_t* const* pos_slabs,
                                       const void* const* k_slabs, const int32_t* const* seg_lens,
                                       int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                                       int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                                       int64_t q_idx, int strategy, int rounding,
-                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept,
                                       void* stream);
 
 /*
@@ -205,7 +208,7 @@ int trimkv_group_threshold_wide(const void* const* lb_slabs, const int64_t* cons
                                 int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                                 int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                                 int64_t q_idx, int strategy, int rounding,
-                                uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
@@ -232,7 +235,7 @@ typedef struct trimkv_layer_slabs {
     void* lb_slab;       /* [nseg][cap] log beta */
     int64_t* pos_slab;   /* [nseg][cap] */
     int32_t* seg_len;    /* [nseg], updated */
-    int64_t q_idx;       /* tokens seen by this layer + 1 (cache_utils.py:173) */
+    int64_t q_idx;       /* tokens seen by this layer + 1 (cache_utils.py:173); see trimkv_evict_layers for the overrides */
     int32_t cap;         /* rows per segment in this layer's slabs */
     int32_t reserved;
 } trimkv_layer_slabs;
@@ -245,9 +248,14 @@ typedef struct trimkv_layer_slabs {
  * (keep_layer_stride = 0: the same budgets for every layer) or [nlayers][nseg]
  * (keep_layer_stride = nseg).  max_len bounds every layer's segment lengths and must not exceed any
  * layer's cap; workspace: nlayers * trimkv_evict_workspace(nseg, max_len) bytes.
+ * Query index (tokens seen + 1) of the scores: *q_idx_dev (a device int64 that the caller advances on the device -- the
+ * form a captured graph can replay step after step) if q_idx_dev is given; else q_idx if it is positive (one value for
+ * every layer: the table then only holds addresses and can be kept for as long as the slabs live); else each layer's
+ * own layers[l].q_idx.
  */
 int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
                         int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                        int64_t q_idx, const int64_t* q_idx_dev,
                         int strategy, int rounding, int sliding_window, int max_len,
                         void* workspace, size_t workspace_bytes, void* stream);
 
@@ -256,12 +264,12 @@ int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg,
  * (the per-layer rebuild loops at cache_utils.py:466-482, 912-943).  thr_key / tie_take are
  * [ngroups] shared by all layers (thr_layer_stride = 0: one budget across layers) or
  * [nlayers][ngroups] (thr_layer_stride = ngroups: layer-wise budgets); tie_base is [nlayers][nseg]
- * as trimkv_group_threshold writes it.
+ * as trimkv_group_threshold writes it.  q_idx > 0 replaces every layer's layers[l].q_idx.
  */
 int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int segs_per_group, int head_dim,
                                     int kv_dtype, int lb_dtype,
                                     const uint32_t* thr_key, const int32_t* tie_take, int thr_layer_stride,
-                                    const int32_t* tie_base, int strategy, int rounding, int max_len,
+                                    const int32_t* tie_base, int64_t q_idx, int strategy, int rounding, int max_len,
                                     void* workspace, size_t workspace_bytes, void* stream);
 
 /*

@@ -82,23 +82,23 @@ def test_bad_arguments_are_refused_without_a_launch():
     assert lib.trimkv_gate_hidden_swiglu(one, one, one, one, one, 8, 2048, 500, 8, _lib.BF16, None) == -6
     # group selection
     assert lib.trimkv_group_threshold(one, one, None, one, 1, 8, 3, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 0, 1,
-                                      one, one, one, one, None) == -2  # 3 does not divide 8
+                                      one, one, one, one, None, None) == -2  # 3 does not divide 8
     assert lib.trimkv_group_threshold(one, one, None, one, 1, 8, 4, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 1, 1,
-                                      one, one, one, one, None) == -1  # knorm without K
+                                      one, one, one, one, None, None) == -1  # knorm without K
     assert lib.trimkv_group_threshold_each_layer(one, one, None, one, 3, 8, 3, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 0, 1,
-                                                 one, one, one, one, None) == -2
+                                                 one, one, one, one, one, None) == -2
     wide = lambda spg, ws, wsb, strat=0: lib.trimkv_group_threshold_wide(one, one, None, one, 2, 8, spg, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0,
-                                                                         5, strat, 1, one, one, one, one, ws, wsb, None)
+                                                                         5, strat, 1, one, one, one, one, None, ws, wsb, None)
     need = lib.trimkv_group_threshold_workspace(2, 8, 4)
-    assert need == (2 * 4 * 256 + 2 * 8 * 2) * 4
+    assert need == (2 * 4 * 256 + 2 * 8 * 3) * 4
     assert wide(3, one, need) == -2 and wide(4, None, 0) == -5 and wide(4, one, need - 1) == -5 and wide(4, one, need, strat=1) == -1
     # several layers in one launch
     layers = lambda **kw: lib.trimkv_evict_layers(kw.get("table", one), kw.get("nl", 3), 4, kw.get("D", 128), _lib.BF16, _lib.F32, kw.get("keep", 8),
-                                                  kw.get("kps"), kw.get("stride", 0), 0, kw.get("strat", 0), 0, 0, 64, None, 0, None)
+                                                  kw.get("kps"), kw.get("stride", 0), 0, 77, None, kw.get("strat", 0), 0, 0, 64, None, 0, None)
     assert layers(table=None) == -1 and layers(nl=0) == -2 and layers(D=100) == -2 and layers(keep=-1) == -2 and layers(strat=5) == -6
     assert layers(kps=one, stride=3) == -2
     compact = lambda **kw: lib.trimkv_compact_threshold_layers(one, 3, 8, kw.get("spg", 4), 128, _lib.BF16, _lib.F32, kw.get("thr", one), one,
-                                                               kw.get("stride", 0), one, 0, 1, 64, None, 0, None)
+                                                               kw.get("stride", 0), one, 77, 0, 1, 64, None, 0, None)
     assert compact(spg=3) == -2 and compact(thr=None) == -1 and compact(stride=5) == -2
 
 

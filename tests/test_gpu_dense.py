@@ -138,11 +138,23 @@ def test_knorm_alpha_and_sliding_window():
     pos = torch.arange(n)
     ref = DenseCacheRef(); ref.update(k, v, lb, pos, 0)
     cache = TrimKVCache(); cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), 0)
+    # the oracle's scores (cache_utils.py:172-180): fp32(log beta) * age + log||k|| with norm and log rounded to bf16
+    sc = lb.float() * (n + 1 - pos) + torch.log(k.norm(dim=-1))
     want = ref.compress_layer(0, M, "knorm_alpha")
     got = cache.compress_layer(0, M, "knorm_alpha", return_indices=True).cpu().long()
-    # log||k|| is rounded to bf16 on both sides but summed in a different order: allow the rare flip at the cut
-    diff = sum(len(set(got[0, h].tolist()) ^ set(want[0, h].tolist())) for h in range(H))
-    assert diff <= 2 * H, f"{diff} differing indices"
+    # The GPU sums the squares in another order than torch, so a row's bf16 log||k|| can differ by one unit u; every score is
+    # then within u of the oracle's and so is the cut (an order statistic), hence the kept sets can differ only on tokens
+    # whose oracle score is within 2u of the oracle's cut.  Everything else must match exactly.
+    u = 2.0 ** (np.floor(np.log2(float(torch.log(k.float().norm(dim=-1)).abs().max()))) - 7)
+    flips = 0
+    for h in range(H):
+        cut = float(sc[0, h][want[0, h]].min())
+        moved = set(got[0, h].tolist()) ^ set(want[0, h].tolist())
+        flips += len(moved)
+        assert got[0, h].numel() == M and all(abs(float(sc[0, h, i]) - cut) <= 2 * u for i in moved), (h, sorted(moved))
+    if flips == 0:
+        assert torch.equal(got, want)
+        assert torch.equal(cache.key_cache[0].cpu(), ref.key_cache[0]) and torch.equal(cache.kv_positions[0].cpu(), ref.kv_positions[0])
     # sliding window: the newest w tokens survive whatever their score
     ref2 = DenseCacheRef(); ref2.update(k, v, lb - 30.0 * (pos >= n - 16), pos, 0)
     c2 = TrimKVCache(); c2.update(k.to(DEV), v.to(DEV), (lb - 30.0 * (pos >= n - 16)).to(DEV), pos.to(DEV), 0)
@@ -203,3 +215,36 @@ def test_skipped_layers_getitem_iter_log_copy_and_batch_utils():
     assert torch.equal(cache.kv_positions[0].cpu(), ref.kv_positions[0][[3, 1]])
     with pytest.raises(NotImplementedError):
         TrimKVCache(_distributed_cache_data=[1])
+
+
+def test_knorm_alpha_all_layers_in_one_launch():
+    """compress("knorm_alpha") over three layers (the layered launch): per layer and head the kept set equals the oracle's
+    except, at most, for tokens within two bf16 units of log||k|| of the oracle's cut (see the single-layer test)."""
+    from trimkv_amd import TrimKVCache
+    gen = torch.Generator().manual_seed(15)
+    B, H, L, n, M, buf = 2, 4, 3, 400, 256, 64
+    cache, ref = TrimKVCache(), DenseCacheRef()
+    pos = torch.arange(n)
+    snap = []
+    for l in range(L):
+        k, v = draw_kv(gen, B, H, n)
+        lb = draw_log_beta(gen, B, H, n, sigma=1.5)
+        ref.update(k, v, lb, pos, l)
+        cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), l)
+        snap.append((lb.float() * (n + 1 - pos) + torch.log(k.norm(dim=-1)), k))
+    ref.compress("knorm_alpha", M, buf)
+    cache.compress("knorm_alpha", M, buf)
+    exact = 0
+    for l, (sc, k) in enumerate(snap):
+        assert cache.get_cache_length(l) == ref.get_cache_length(l) == M
+        u = 2.0 ** (np.floor(np.log2(float(torch.log(k.float().norm(dim=-1)).abs().max()))) - 7)
+        got, want = cache.kv_positions[l].cpu(), ref.kv_positions[l]
+        for b in range(B):
+            for h in range(H):
+                cut = float(sc[b, h][want[b, h]].min())
+                moved = set(got[b, h].tolist()) ^ set(want[b, h].tolist())
+                assert all(abs(float(sc[b, h, i]) - cut) <= 2 * u for i in moved), (l, b, h, sorted(moved))
+                exact += not moved
+        if torch.equal(got, want):
+            assert torch.equal(cache.key_cache[l].cpu(), ref.key_cache[l]) and torch.equal(cache.retention_weights[l].cpu(), ref.retention_weights[l])
+    assert exact >= B * H * L - 2

@@ -37,16 +37,16 @@ SIGNATURES = {
     "trimkv_evict": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _i, _i64, _i, _i, _i, _i,
                           _p, _i, _p, _sz, _p]),
     "trimkv_group_threshold": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
-                                    _p, _p, _p, _p, _p]),
+                                    _p, _p, _p, _p, _p, _p]),
     "trimkv_group_threshold_each_layer": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
-                                    _p, _p, _p, _p, _p]),
+                                    _p, _p, _p, _p, _p, _p]),
     "trimkv_group_threshold_workspace": (_sz, [_i, _i, _i]),
     "trimkv_group_threshold_wide": (_i, [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i64, _i, _f, _i64, _i, _i,
-                                         _p, _p, _p, _p, _p, _sz, _p]),
+                                         _p, _p, _p, _p, _p, _p, _sz, _p]),
     "trimkv_compact_threshold": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i, _i, _i,
                                       _p, _sz, _p]),
-    "trimkv_evict_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _i, _i, _i, _i, _p, _sz, _p]),
-    "trimkv_compact_threshold_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p, _i, _i, _i, _p, _sz, _p]),
+    "trimkv_evict_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _i64, _p, _i, _i, _i, _i, _p, _sz, _p]),
+    "trimkv_compact_threshold_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p, _i64, _i, _i, _i, _p, _sz, _p]),
     "trimkv_build_cu_seqlens": (_i, [_p, _i, _p, _p]),
     "trimkv_decode_attn_workspace": (_sz, [_i, _i, _i, _i, _i]),
     "trimkv_decode_attn": (_i, [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p]),

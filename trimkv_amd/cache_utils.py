@@ -163,6 +163,7 @@ class _SlabBacked(_CacheBase):
         self.sliding_window_size = 0
         self._budget_hint: Optional[int] = None  # memory_size + buffer_size of the last compress()
         self._ws: Dict[Any, torch.Tensor] = {}
+        self._table_cache: Dict[Any, Any] = {}
         # Opt-in: a decode-step update() (one token) leaves its rows to the attention call of the same layer, which then
         # appends and attends in one launch.  Only for callers whose next reader of what update() returned is this
         # package's HIP attention (the reference's own call order, modeling_trimkv_qwen3.py:353 -> :365) and who leave the
@@ -309,31 +310,60 @@ class _SlabBacked(_CacheBase):
         return all((s.nseg, s.D, s.k.dtype, s.lb.dtype, s.k.device) == (s0.nseg, s0.D, s0.k.dtype, s0.lb.dtype, s0.k.device)
                    for s in (self._slabs[l] for l in layers))
 
-    def _layer_table(self, layers: List[int], q_idx) -> torch.Tensor:
-        """Device table of ``trimkv_layer_slabs`` for ``layers``; ``q_idx`` maps a layer to its tokens seen + 1."""
+    def _device_tables(self, layers: List[int]) -> Dict[str, torch.Tensor]:
+        """Device-resident address tables of ``layers``: ``"slabs"`` (an array of ``trimkv_layer_slabs`` with q_idx = 0: the
+        launches get the query index as an argument) and the plain pointer tables ``"lb"``, ``"pos"``, ``"k"``, ``"len"`` of the
+        group-selection kernels.  Built and uploaded once; rebuilt only when a slab of the set has moved (regrow, batch
+        reordering), so that an eviction in steady state enqueues without any host-to-device copy."""
+        key = tuple(layers)
+        slabs = [self._slabs[l] for l in layers]
+        hit = self._table_cache.get(key)
+        if hit is not None and all(a is s.ptrs for a, s in zip(hit[0], slabs)) and hit[1] == [s.cap for s in slabs]:
+            return hit[2]
+        dev = slabs[0].k.device
+        arr = np.zeros(len(layers), dtype=self._LAYER_DT)
+        for i, s in enumerate(slabs):
+            arr[i] = (s.ptrs[0], s.ptrs[1], s.ptrs[2], s.ptrs[3], s.ptrs[4], 0, s.cap, 0)
+        tables = {"slabs": torch.from_numpy(arr.view(np.uint8)).to(dev)}
+        for name, idx in (("k", 0), ("lb", 2), ("pos", 3), ("len", 4)):
+            tables[name] = torch.tensor([s.ptrs[idx] for s in slabs], dtype=torch.int64).to(dev)
+        self._table_cache[key] = ([s.ptrs for s in slabs], [s.cap for s in slabs], tables)
+        return tables
+
+    def _layer_table_with_q(self, layers: List[int], q_of_layer) -> torch.Tensor:
+        """A one-off ``trimkv_layer_slabs`` table that carries a different query index per layer (layers that have seen
+        different numbers of tokens); uploaded for this launch."""
         arr = np.zeros(len(layers), dtype=self._LAYER_DT)
         for i, l in enumerate(layers):
             s = self._slabs[l]
-            arr[i] = (s.ptrs[0], s.ptrs[1], s.ptrs[2], s.ptrs[3], s.ptrs[4], int(q_idx(l)), s.cap, 0)
+            arr[i] = (s.ptrs[0], s.ptrs[1], s.ptrs[2], s.ptrs[3], s.ptrs[4], int(q_of_layer[i]), s.cap, 0)
         return torch.from_numpy(arr.view(np.uint8)).to(self._slabs[layers[0]].k.device)
 
-    def _evict_layers(self, layers: List[int], keep: int, keep_per_seg: Optional[np.ndarray], slack: int, strategy_code: int,
+    def _evict_layers(self, layers: List[int], keep: int, keep_per_seg, slack: int, strategy_code: int,
                       rounding: int, sliding_window: int, q_idx) -> None:
-        """``trimkv_evict_layers`` over ``layers`` (all of one shape): one launch of nseg x len(layers) workgroups."""
+        """``trimkv_evict_layers`` over ``layers`` (all of one shape): one launch of nseg x len(layers) workgroups.
+        ``q_idx``: the query index, one int or one per layer.  ``keep_per_seg``: None, a host array (uploaded) or a device
+        int32 tensor, ``[nseg]`` or ``[len(layers), nseg]``."""
         s0 = self._slabs[layers[0]]
         dev = s0.k.device
         max_len = max(self._slabs[l].max_len for l in layers)
-        table = self._layer_table(layers, q_idx)
+        qs = [int(q_idx)] * len(layers) if np.isscalar(q_idx) else [int(q) for q in q_idx]
+        if all(q == qs[0] for q in qs) and qs[0] > 0:
+            table, q_all = self._device_tables(layers)["slabs"], qs[0]
+        else:
+            table, q_all = self._layer_table_with_q(layers, qs), 0
         kdev, stride = None, 0
         if keep_per_seg is not None:
-            kp = np.ascontiguousarray(keep_per_seg, dtype=np.int32)
-            stride = 0 if kp.ndim == 1 else s0.nseg
-            kdev = torch.from_numpy(kp.reshape(-1)).to(dev)
+            if torch.is_tensor(keep_per_seg):
+                kdev = keep_per_seg.to(device=dev, dtype=torch.int32).contiguous()
+            else:
+                kdev = torch.from_numpy(np.ascontiguousarray(keep_per_seg, dtype=np.int32)).to(dev)
+            stride = 0 if kdev.dim() == 1 else s0.nseg
         lib = _lib.load()
         ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
         rc = lib.trimkv_evict_layers(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
-                                     int(keep), _lib.ptr(kdev), stride, int(slack), strategy_code, rounding, int(sliding_window), max_len,
-                                     _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
+                                     int(keep), _lib.ptr(kdev), stride, int(slack), q_all, None, strategy_code, rounding, int(sliding_window),
+                                     max_len, _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
         _lib.check(rc, "trimkv_evict_layers")
         self._keepalive_layers = (table, kdev)   # read asynchronously by the launch
 
@@ -487,7 +517,7 @@ class TrimKVCache(_SlabBacked):
         todo = [l for l in range(skip_layers, num_layers) if memory_size + buffer_size <= self.get_cache_length(l)]
         if len(todo) > 1 and self._layers_alike(todo):   # the usual case: every layer is due at the same step -> one launch
             self._evict_layers(todo, memory_size, None, 0, self._dense_strategy_code(strategy), _lib.ROUND_UPCAST,
-                               self.sliding_window_size, lambda l: self.get_seq_length(l) + 1)
+                               self.sliding_window_size, [self.get_seq_length(l) + 1 for l in todo])
             for l in todo:
                 self._slabs[l].lens[:] = memory_size
                 self._slabs[l].max_len = memory_size
@@ -724,9 +754,6 @@ class _RaggedCache(_SlabBacked):
         tensor), so the threshold is rounded to that dtype first."""
         return float(torch.log(torch.tensor(alpha_threshold, dtype=torch.float32)).to(score_dtype))
 
-    def _ptr_table(self, tensors: List[torch.Tensor], device) -> torch.Tensor:
-        return torch.tensor([t.data_ptr() for t in tensors], dtype=torch.int64).to(device)
-
     @staticmethod
     def _equalise_capacity(slabs: List[_Slab]) -> None:
         """The cross-layer selection kernels address every layer with one row capacity.  Layers grow on their own (their
@@ -737,9 +764,9 @@ class _RaggedCache(_SlabBacked):
                 s.regrow(cap)
 
     def _group_select(self, layers: List[int], segs_per_group: int, budget: int, strategy: str,
-                      threshold: Optional[float] = None):
+                      threshold: Optional[float] = None, want_first_kept: bool = False):
         """Run ``trimkv_group_threshold`` over ``layers`` (all of one shape); returns the device
-        tensors (thr_key, tie_take, tie_base [L,nseg], new_len [L,nseg])."""
+        tensors (thr_key, tie_take, tie_base [L,nseg], new_len [L,nseg]) and, on request, first_kept [L,nseg]."""
         slabs = [self._slabs[l] for l in layers]
         s0 = slabs[0]
         for s in slabs:
@@ -753,16 +780,14 @@ class _RaggedCache(_SlabBacked):
         take = torch.empty(ngroups, dtype=torch.int32, device=dev)
         tie_base = torch.empty(L, s0.nseg, dtype=torch.int32, device=dev)
         new_len = torch.empty(L, s0.nseg, dtype=torch.int32, device=dev)
-        lb_t = self._ptr_table([s.lb for s in slabs], dev)
-        pos_t = self._ptr_table([s.pos for s in slabs], dev)
-        k_t = self._ptr_table([s.k for s in slabs], dev)
-        len_t = self._ptr_table([s.seg_len for s in slabs], dev)
+        first = torch.empty(L, s0.nseg, dtype=torch.int32, device=dev) if want_first_kept else None
+        t = self._device_tables(layers)
         lib = _lib.load()
-        args = (lb_t.data_ptr(), pos_t.data_ptr(), k_t.data_ptr(), len_t.data_ptr(),
+        args = (t["lb"].data_ptr(), t["pos"].data_ptr(), t["k"].data_ptr(), t["len"].data_ptr(),
                 L, s0.nseg, segs_per_group, s0.cap, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
                 int(budget), 0 if threshold is None else 1, 0.0 if threshold is None else float(threshold),
                 self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE,
-                thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr())
+                thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(), _lib.ptr(first))
         if L * segs_per_group >= 16:   # a large group (a budget shared by all layers): one workgroup per (layer, segment)
             ws = self._workspace(lib.trimkv_group_threshold_workspace(L, s0.nseg, segs_per_group), dev)
             rc = lib.trimkv_group_threshold_wide(*args, ws.data_ptr(), ws.numel(), _lib.current_stream(dev))
@@ -770,7 +795,8 @@ class _RaggedCache(_SlabBacked):
         else:
             rc = lib.trimkv_group_threshold(*args, _lib.current_stream(dev))
             _lib.check(rc, "trimkv_group_threshold")
-        self._keepalive = (lb_t, pos_t, k_t, len_t)  # the launch reads these tables asynchronously
+        if want_first_kept:
+            return thr, take, tie_base, new_len, first
         return thr, take, tie_base, new_len
 
     def _group_select_each(self, layers: List[int], segs_per_group: int, budget: int, strategy: str):
@@ -787,14 +813,13 @@ class _RaggedCache(_SlabBacked):
         take = torch.empty(L, ngroups, dtype=torch.int32, device=dev)
         tie_base = torch.empty(L, nseg, dtype=torch.int32, device=dev)
         new_len = torch.empty(L, nseg, dtype=torch.int32, device=dev)
-        tables = [self._ptr_table([getattr(s, name) for s in slabs], dev) for name in ("lb", "pos", "k", "seg_len")]
+        t = self._device_tables(layers)
         rc = _lib.load().trimkv_group_threshold_each_layer(
-            tables[0].data_ptr(), tables[1].data_ptr(), tables[2].data_ptr(), tables[3].data_ptr(), L, nseg, segs_per_group, s0.cap, s0.D,
+            t["lb"].data_ptr(), t["pos"].data_ptr(), t["k"].data_ptr(), t["len"].data_ptr(), L, nseg, segs_per_group, s0.cap, s0.D,
             _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype), int(budget), 0, 0.0, self.get_seq_length() + 1,
-            self._strategy_code(strategy), _lib.ROUND_NATIVE, thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(),
+            self._strategy_code(strategy), _lib.ROUND_NATIVE, thr.data_ptr(), take.data_ptr(), tie_base.data_ptr(), new_len.data_ptr(), None,
             _lib.current_stream(dev))
         _lib.check(rc, "trimkv_group_threshold_each_layer")
-        self._keepalive = tuple(tables)  # the launch reads these tables asynchronously
         return thr, take, tie_base, new_len
 
     def _compact(self, layer: int, segs_per_group: int, thr, take, tie_base_l, strategy: str) -> None:
@@ -819,21 +844,24 @@ class _RaggedCache(_SlabBacked):
         s0 = self._slabs[layers[0]]
         dev = s0.k.device
         max_len = max(self._slabs[l].max_len for l in layers)
-        q = self.get_seq_length() + 1
-        table = self._layer_table(layers, lambda l: q)
+        table = self._device_tables(layers)["slabs"]
         lib = _lib.load()
         ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
         rc = lib.trimkv_compact_threshold_layers(table.data_ptr(), len(layers), s0.nseg, segs_per_group, s0.D,
                                                  _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
                                                  thr.data_ptr(), take.data_ptr(), thr.shape[1] if per_layer else 0, tie_base.data_ptr(),
-                                                 self._strategy_code(strategy), _lib.ROUND_NATIVE, max_len,
+                                                 self.get_seq_length() + 1, self._strategy_code(strategy), _lib.ROUND_NATIVE, max_len,
                                                  _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
         _lib.check(rc, "trimkv_compact_threshold_layers")
         self._keepalive_layers = (table, None)
 
-    def _evict_per_segment(self, layer: int, keep: np.ndarray, strategy: str) -> None:
+    def _evict_per_segment(self, layer: int, keep, strategy: str) -> None:
+        """``keep``: per-segment budgets of one layer, a host array or a device int32 tensor."""
         slab = self._slabs[layer]
-        keep_dev = torch.from_numpy(np.ascontiguousarray(keep, dtype=np.int32)).to(slab.k.device)
+        if torch.is_tensor(keep):
+            keep_dev = keep.to(device=slab.k.device, dtype=torch.int32).contiguous()
+        else:
+            keep_dev = torch.from_numpy(np.ascontiguousarray(keep, dtype=np.int32)).to(slab.k.device)
         lib = _lib.load()
         ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
         rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
@@ -899,10 +927,20 @@ class _RaggedCache(_SlabBacked):
                 due.append((l, kh, hit))
         if not due:
             return
-        if len(due) > 1 and self._layers_alike([l for l, _, _ in due]):   # the layers that are due: one launch
-            q = self.get_seq_length() + 1
+        every = [l for l in range(len(self._slabs)) if self._slabs[l] is not None]
+        if len(due) > 1 and list(layers) == every and self._layers_alike(every):
+            # One launch over every layer, whichever of them are due: the kernel re-checks the trigger per segment, so the
+            # launch -- address table and budgets resident on the device -- is the same at every step and nothing is uploaded.
+            key = ("all", str(self._slabs[every[0]].k.device))
+            keep = self._budgets_dev.get(key)
+            if keep is None:
+                kh_all = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[every]
+                keep = torch.from_numpy(np.ascontiguousarray(kh_all, dtype=np.int32)).to(self._slabs[every[0]].k.device)
+                self._budgets_dev[key] = keep
+            self._evict_layers(every, 0, keep, buffer_size, code, _lib.ROUND_NATIVE, 0, self.get_seq_length() + 1)
+        elif len(due) > 1 and self._layers_alike([l for l, _, _ in due]):   # a subset of the layers: its budgets are uploaded
             self._evict_layers([l for l, _, _ in due], 0, np.stack([kh for _, kh, _ in due]), buffer_size, code, _lib.ROUND_NATIVE, 0,
-                               lambda l: q)
+                               self.get_seq_length() + 1)
         else:
             for l, kh, _ in due:
                 slab = self._slabs[l]
@@ -981,14 +1019,13 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             for part in ([todo] if alike else [[l] for l in todo]):   # layers of one shape go through together
                 if floor_budget_ratio > 0:
                     budget = int(memory_size * H * (1 - floor_budget_ratio))
-                    _, _, _, new_len = self._group_select_each(part, H, budget, base)
-                    chosen = new_len.cpu().numpy().astype(np.int64)
+                    _, _, _, chosen = self._group_select_each(part, H, budget, base)
                     floor_per_head = int(memory_size * floor_budget_ratio)
-                    # top-up (:789-806): a head keeps its best max(chosen, floor) tokens, at most all of them
-                    keep = np.minimum(np.maximum(chosen, floor_per_head), np.stack([self._slabs[l].lens for l in part]))
+                    # top-up (:789-806): a head keeps its best max(chosen, floor) tokens, at most all of them (on the device)
+                    lens_dev = torch.stack([self._slabs[l].seg_len for l in part])
+                    keep = torch.minimum(chosen.clamp_min(floor_per_head), lens_dev)
                     if len(part) > 1:
-                        q = self.get_seq_length() + 1
-                        self._evict_layers(part, 0, keep, 0, self._strategy_code(base), _lib.ROUND_NATIVE, 0, lambda l: q)
+                        self._evict_layers(part, 0, keep, 0, self._strategy_code(base), _lib.ROUND_NATIVE, 0, self.get_seq_length() + 1)
                     else:
                         self._evict_per_segment(part[0], keep[0], base)
                 else:
@@ -1068,48 +1105,23 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             return
         assert "threshold" not in strategy, "Thresholding strategy is not compatible with floor_budget_ratio > 0"
         adaptive = int(total_budget * (1 - floor_budget_ratio))
-        thr, take, tie_base, new_len = self._group_select(layers, H, adaptive, strategy)
-        chosen = new_len.cpu().numpy().astype(np.int64).reshape(-1)          # per (layer, head), flattened
-        first_sel = self._first_token_selected(layers, thr, take, tie_base, strategy).reshape(-1)
-        lens = np.concatenate([self._slabs[l].lens for l in layers])
-        # bucketize against the inclusive cumsum with right=False (cache_utils.py:496): a chosen
-        # token that is the FIRST row of head j >= 1 is counted for head j-1.
-        credited = chosen.copy()
-        moved = first_sel.copy()
+        _, _, _, chosen, first = self._group_select(layers, H, adaptive, strategy, want_first_kept=True)
+        # bucketize against the inclusive cumsum with right=False (cache_utils.py:496): a chosen token that is the FIRST row
+        # of head j >= 1 is counted for head j-1.  first[j] says whether head j's first row was chosen (0 for an empty head);
+        # all of it stays on the device.
+        chosen = chosen.reshape(-1).to(torch.int64)          # per (layer, head), flattened in the reference's order
+        moved = first.reshape(-1).to(torch.int64)
         moved[0] = 0
-        moved[lens == 0] = 0
-        credited -= moved
+        credited = chosen - moved
         credited[:-1] += moved[1:]
-        head_cnt = credited + int(memory_size * floor_budget_ratio)
+        head_cnt = (credited + int(memory_size * floor_budget_ratio)).to(torch.int32)
         if len(layers) > 1 and self._layers_alike(layers):   # k >= len keeps all (:514-516)
-            q = self.get_seq_length() + 1
-            self._evict_layers(layers, 0, head_cnt.reshape(len(layers), H), 0, self._strategy_code(strategy), _lib.ROUND_NATIVE, 0,
-                               lambda l: q)
+            self._evict_layers(layers, 0, head_cnt.view(len(layers), H), 0, self._strategy_code(strategy), _lib.ROUND_NATIVE, 0,
+                               self.get_seq_length() + 1)
         else:
             for i, l in enumerate(layers):
                 self._evict_per_segment(l, head_cnt[i * H:(i + 1) * H], strategy)
         self._refresh(layers)
-
-    def _first_token_selected(self, layers, thr, take, tie_base, strategy) -> np.ndarray:
-        """For every (layer, head): is its oldest token among the globally chosen ones?"""
-        thr_key = int(thr.cpu().numpy().astype(np.uint32)[0])
-        take_n = int(take.cpu()[0])
-        tb = tie_base.cpu().numpy()
-        q_idx = self.get_seq_length() + 1
-        out = np.zeros((len(layers), self._slabs[layers[0]].nseg), dtype=np.int64)
-        for i, l in enumerate(layers):
-            s = self._slabs[l]
-            lb0, pos0 = s.lb[:, 0], s.pos[:, 0]
-            score = (q_idx - pos0) * lb0  # the ragged classes' own expression (cache_utils.py:441)
-            if "knorm" in strategy:
-                score = score + torch.log(s.k[:, 0].norm(dim=-1).clamp_min(1e-12))
-            f = score.float().cpu().numpy().astype(np.float32)
-            f = np.where(f == 0, np.float32(0), f)
-            u = f.view(np.uint32)
-            key = np.where(u & np.uint32(0x80000000), ~u, u | np.uint32(0x80000000)).astype(np.uint64)
-            sel = (key > thr_key) | ((key == thr_key) & (tb[i] < take_n))
-            out[i] = sel & (s.lens > 0)
-        return out
 
     def log(self):
         positions = self.segment_positions()

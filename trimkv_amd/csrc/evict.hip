@@ -31,34 +31,72 @@ struct ScoreArgs {
     int64_t q_idx;
 };
 
-// ||k_row|| and its log, rounded as torch rounds them for a 16-bit K (norm -> K dtype, log -> K dtype).
-__device__ __forceinline__ float knorm_term(const ScoreArgs& s, int i) {
-    const uint16_t* row = (const uint16_t*)(s.k + (int64_t)i * s.row_bytes);
-    const int d = s.row_bytes >> 1;
-    float acc = 0.0f;
-    for (int e = 0; e < d; ++e) {
-        const float x = s.kv_dtype == TRIMKV_BF16 ? bf16_bits_to_f32(row[e]) : f16_bits_to_f32(row[e]);
-        acc = __fmaf_rn(x, x, acc);
+// log ||k_row|| for the 64 rows base .. base+63 of a segment, one per lane (lane l gets row base + l; rows past n-1 repeat
+// row n-1), rounded as torch rounds it for a 16-bit K: norm -> K dtype, log -> K dtype (cache_utils.py:176-180); NATIVE
+// clamps the norm at 1e-12 first (:390, 759).  The whole wavefront works on it: 16 lanes read one row as 16-byte pieces
+// (4 rows per step, 16 steps), square-sum their 8 elements in fp32 and add across the 16 lanes with a fixed butterfly, so
+// the value of a row depends on nothing but the row -- every pass and every kernel that scores a token gets the same bits.
+// The fp32 sum is formed in another order than torch forms it; after the two roundings to 16 bits the results agree
+// except for rows whose norm sits on a rounding boundary, where they may differ by one unit of the 16-bit logarithm.
+__device__ __forceinline__ float knorm_terms_of_wave(const ScoreArgs& s, int base, int n) {
+    const int lane = threadIdx.x & 63, grp = lane >> 4, c = lane & 15;
+    const int pieces = s.row_bytes >> 4;
+    float mine = 0.0f;
+#pragma unroll 4
+    for (int j = 0; j < 16; ++j) {   // four rows' loads in flight per lane group at a time
+        const int row = min(base + j * 4 + grp, n - 1);
+        const char* rp = s.k + (int64_t)row * s.row_bytes;
+        float acc = 0.0f;
+        for (int p = c; p < pieces; p += 16) {
+            const uint4 w = *(const uint4*)(rp + (p << 4));
+            const uint32_t words[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float lo, hi;
+                if (s.kv_dtype == TRIMKV_BF16) { lo = __uint_as_float(words[e] << 16); hi = __uint_as_float(words[e] & 0xffff0000u); }
+                else { lo = f16_bits_to_f32((uint16_t)(words[e] & 0xffffu)); hi = f16_bits_to_f32((uint16_t)(words[e] >> 16)); }
+                acc = __fmaf_rn(lo, lo, acc);
+                acc = __fmaf_rn(hi, hi, acc);
+            }
+        }
+#pragma unroll
+        for (int d = 1; d < 16; d <<= 1) acc = __fadd_rn(acc, __shfl_xor(acc, d, 64));
+        float nrm = round_to_dtype(__fsqrt_rn(acc), s.kv_dtype);
+        if (s.rounding == TRIMKV_ROUND_NATIVE) nrm = fmaxf(nrm, round_to_dtype(1e-12f, s.kv_dtype));
+        const float term = round_to_dtype(logf(nrm), s.kv_dtype);
+        const float got = __shfl(term, (lane & 3) << 4, 64);   // row base + l was handled in step l / 4 by lane group l % 4
+        if ((lane >> 2) == j) mine = got;
     }
-    float nrm = round_to_dtype(__fsqrt_rn(acc), s.kv_dtype);
-    if (s.rounding == TRIMKV_ROUND_NATIVE) nrm = fmaxf(nrm, round_to_dtype(1e-12f, s.kv_dtype));
-    return round_to_dtype(logf(nrm), s.kv_dtype);
+    return mine;
 }
 
-// Order-preserving key of token i's score; n = segment length (for the sliding window).
-__device__ __forceinline__ uint32_t score_key(const ScoreArgs& s, int i, int n) {
+// Order-preserving key of token i's score; n = segment length (for the sliding window); knorm = the token's log ||k||
+// (read only by the knorm strategy).
+__device__ __forceinline__ uint32_t score_key(const ScoreArgs& s, int i, int n, float knorm) {
     if (s.sliding_window > 0 && i >= n - s.sliding_window) return float_key(__builtin_inff());
     const float lb = load_as_f32(s.lb, i, s.lb_dtype);
     const float age = (float)(s.q_idx - s.pos[i]);  // int64 -> fp32, round to nearest even
     float sc;
     if (s.rounding == TRIMKV_ROUND_NATIVE && s.lb_dtype != TRIMKV_F32) {
         sc = round_to_dtype(__fmul_rn(round_to_dtype(age, s.lb_dtype), lb), s.lb_dtype);
-        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = round_to_dtype(__fadd_rn(sc, knorm_term(s, i)), s.lb_dtype);
+        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = round_to_dtype(__fadd_rn(sc, knorm), s.lb_dtype);
     } else {
         sc = __fmul_rn(lb, age);
-        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = __fadd_rn(sc, knorm_term(s, i));
+        if (s.strategy == TRIMKV_SCORE_KNORM_ALPHA) sc = __fadd_rn(sc, knorm);
     }
     return float_key(sc);
+}
+
+// f(i, key) for every token i of the segment that this thread owns (i = threadIdx.x, + THREADS, ...).  Whole wavefronts
+// walk the segment together (the loop bound is wave-uniform), because the knorm term is computed by the wavefront.
+template <int THREADS, class F>
+__device__ __forceinline__ void for_each_key(const ScoreArgs& s, int n, F&& f) {
+    const int lane = threadIdx.x & 63;
+    for (int base = (int)(threadIdx.x & ~63u); base < n; base += THREADS) {
+        const float knorm = s.strategy == TRIMKV_SCORE_KNORM_ALPHA ? knorm_terms_of_wave(s, base, n) : 0.0f;
+        const int i = base + lane;
+        if (i < n) f(i, score_key(s, i, n, knorm));
+    }
 }
 
 // ---- 4-pass radix select: the `want`-th largest of keys[0..n) -------------------------------
@@ -247,6 +285,8 @@ struct EvictArgs {
     const uint32_t* thr_key; const int32_t* tie_take; const int32_t* tie_base; int segs_per_group;
     // several layers in one launch (blockIdx.y = layer): per-layer slabs come from this device table
     const trimkv_layer_slabs* layers; int keep_layer_stride, thr_layer_stride;
+    // query index of a layered launch: *q_idx_dev if given, else q_idx_all if positive, else the table's per-layer value
+    const int64_t* q_idx_dev; int64_t q_idx_all;
 };
 
 // blockIdx.y selects a layer: its slab addresses, capacity and query index replace the scalar fields, and the
@@ -256,7 +296,8 @@ __device__ __forceinline__ void select_layer(EvictArgs& a) {
     const int layer = blockIdx.y;
     const trimkv_layer_slabs L = a.layers[layer];
     a.k_slab = (char*)L.k_slab; a.v_slab = (char*)L.v_slab; a.lb_slab = (char*)L.lb_slab; a.pos_slab = L.pos_slab; a.seg_len = L.seg_len;
-    a.q_idx = L.q_idx; a.cap = L.cap;
+    a.q_idx = a.q_idx_dev ? *a.q_idx_dev : (a.q_idx_all > 0 ? a.q_idx_all : L.q_idx);
+    a.cap = L.cap;
     if (a.keep_per_seg) a.keep_per_seg += (int64_t)layer * a.keep_layer_stride;
     if (a.tie_base) a.tie_base += (int64_t)layer * a.nseg;
     if (a.thr_key) { a.thr_key += (int64_t)layer * a.thr_layer_stride; a.tie_take += (int64_t)layer * a.thr_layer_stride; }
@@ -298,7 +339,7 @@ __global__ __launch_bounds__(EV_THREADS) void evict_kernel(EvictArgs a) {
     ScoreArgs s;
     s.lb = lbseg; s.pos = posseg; s.k = kseg; s.lb_dtype = a.lb_dtype; s.kv_dtype = a.kv_dtype; s.row_bytes = a.row_bytes;
     s.strategy = a.strategy; s.rounding = a.rounding; s.sliding_window = a.sliding_window; s.q_idx = a.q_idx;
-    for (int i = threadIdx.x; i < n; i += EV_THREADS) keys[i] = score_key(s, i, n);
+    for_each_key<EV_THREADS>(s, n, [&](int i, uint32_t key) { keys[i] = key; });
     __syncthreads();
 
     uint32_t thr;
@@ -329,6 +370,7 @@ struct GroupArgs {
     int64_t budget; int use_threshold; float threshold_score;
     int64_t q_idx; int strategy, rounding;
     uint32_t* thr_key; int32_t* tie_take; int32_t* tie_base; int32_t* new_len;
+    int32_t* first_kept;   // optional [nlayers][nseg]: 1 if the segment's oldest token (row 0) is among the kept ones
     int per_layer;   // one budget per (layer, group): blockIdx.y = layer, results are [nlayers][groups]
 };
 
@@ -364,6 +406,7 @@ __global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a
         if (a.k_slabs) a.k_slabs += layer;
         a.thr_key += (int64_t)layer * gridDim.x; a.tie_take += (int64_t)layer * gridDim.x;
         a.tie_base += (int64_t)layer * a.nseg; a.new_len += (int64_t)layer * a.nseg;
+        if (a.first_kept) a.first_kept += (int64_t)layer * a.nseg;
         a.nlayers = 1;
     }
     const int g = blockIdx.x;
@@ -396,10 +439,9 @@ __global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a
                     for (int s = 0; s < a.segs_per_group; ++s) {
                         const int n = max(0, min(a.seg_lens[l][seg0 + s], a.cap));
                         const ScoreArgs sa = group_segment(a, l, seg0 + s);
-                        for (int i = threadIdx.x; i < n; i += GT_THREADS) {
-                            const uint32_t key = score_key(sa, i, n);
+                        for_each_key<GT_THREADS>(sa, n, [&](int, uint32_t key) {
                             if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1ull);
-                        }
+                        });
                     }
                 __syncthreads();
                 if (threadIdx.x == 0) {  // 256 bins, walked from the largest down
@@ -428,16 +470,19 @@ __global__ __launch_bounds__(GT_THREADS) void group_threshold_kernel(GroupArgs a
             const int n = max(0, min(a.seg_lens[l][seg0 + s], a.cap));
             const ScoreArgs sa = group_segment(a, l, seg0 + s);
             uint64_t cnt = 0;  // low 32 bits: greater, high 32 bits: equal
-            for (int i = threadIdx.x; i < n; i += GT_THREADS) {
-                const uint32_t key = score_key(sa, i, n);
+            uint32_t key0 = 0;  // thread 0 owns row 0
+            for_each_key<GT_THREADS>(sa, n, [&](int i, uint32_t key) {
                 cnt += (key > thr ? 1ull : 0ull) + (key == thr ? (1ull << 32) : 0ull);
-            }
+                if (i == 0) key0 = key;
+            });
             cnt = block_sum_u64(cnt, red);
             const int64_t gt = (int64_t)(cnt & 0xffffffffull), eq = (int64_t)(cnt >> 32);
             const int64_t eq_kept = max((int64_t)0, min(eq, take - eq_seen));
             if (threadIdx.x == 0) {
                 a.new_len[(int64_t)l * a.nseg + seg0 + s] = (int32_t)(gt + eq_kept);
                 a.tie_base[(int64_t)l * a.nseg + seg0 + s] = (int32_t)min(eq_seen, (int64_t)INT32_MAX);
+                // row 0 is the first of its segment's equal-to-cut tokens, so its rank among them is the segment's tie base
+                if (a.first_kept) a.first_kept[(int64_t)l * a.nseg + seg0 + s] = n > 0 && (key0 > thr || (key0 == thr && eq_seen < take));
             }
             eq_seen += eq;
         }
@@ -457,7 +502,7 @@ constexpr int GW_THREADS = 256;
 struct WideArgs {
     GroupArgs g;
     uint32_t* hist;   // [ngroups][4][256]
-    uint32_t* cnt;    // [nlayers][nseg][2]: tokens above the cut, tokens equal to it
+    uint32_t* cnt;    // [nlayers][nseg][3]: tokens above the cut, tokens equal to it, row 0 (bit 0: above, bit 1: equal)
 };
 
 // digit and remaining rank chosen in a pass, from that pass's 256-bin histogram (in LDS), largest bin first
@@ -518,10 +563,9 @@ __global__ __launch_bounds__(GW_THREADS) void group_hist_kernel(WideArgs w, int 
     __syncthreads();
     const int n = max(0, min(a.seg_lens[l][seg], a.cap));
     const ScoreArgs sa = group_segment(a, l, seg);
-    for (int i = threadIdx.x; i < n; i += GW_THREADS) {
-        const uint32_t key = score_key(sa, i, n);
+    for_each_key<GW_THREADS>(sa, n, [&](int, uint32_t key) {
         if ((key & hi_mask) == prefix) atomicAdd(&lh[(key >> shift) & 255u], 1u);
-    }
+    });
     __syncthreads();
     if (lh[threadIdx.x]) atomicAdd(&w.hist[((int64_t)g * 4 + pass) * 256 + threadIdx.x], lh[threadIdx.x]);
 }
@@ -558,19 +602,21 @@ __global__ __launch_bounds__(GW_THREADS) void group_count_kernel(WideArgs w) {
     const int n = max(0, min(a.seg_lens[l][seg], a.cap));
     const ScoreArgs sa = group_segment(a, l, seg);
     uint64_t cnt = 0;  // low 32 bits: greater, high 32 bits: equal
-    for (int i = threadIdx.x; i < n; i += GW_THREADS) {
-        const uint32_t key = score_key(sa, i, n);
+    uint32_t row0 = 0;  // thread 0 owns row 0
+    for_each_key<GW_THREADS>(sa, n, [&](int i, uint32_t key) {
         cnt += (key > thr ? 1ull : 0ull) + (key == thr ? (1ull << 32) : 0ull);
-    }
+        if (i == 0) row0 = (key > thr ? 1u : 0u) | (key == thr ? 2u : 0u);
+    });
     for (int d = 32; d > 0; d >>= 1) cnt += __shfl_down(cnt, d, 64);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = cnt;
     __syncthreads();
     if (threadIdx.x == 0) {
         uint64_t t = 0;
         for (int i = 0; i < GW_THREADS / 64; ++i) t += red[i];
-        const int64_t e = ((int64_t)l * a.nseg + seg) * 2;
+        const int64_t e = ((int64_t)l * a.nseg + seg) * 3;
         w.cnt[e] = (uint32_t)(t & 0xffffffffull);
         w.cnt[e + 1] = (uint32_t)(t >> 32);
+        w.cnt[e + 2] = row0;
         if (s == 0 && l == 0) {
             a.thr_key[g] = thr;
             a.tie_take[g] = (int32_t)min(take, (int64_t)INT32_MAX);
@@ -581,6 +627,7 @@ __global__ __launch_bounds__(GW_THREADS) void group_count_kernel(WideArgs w) {
 __global__ __launch_bounds__(GW_THREADS) void group_scan_kernel(WideArgs w) {
     __shared__ uint32_t gt_l[GW_THREADS], eq_l[GW_THREADS];
     __shared__ int32_t len_l[GW_THREADS], base_l[GW_THREADS];
+    uint32_t row0 = 0;
     __shared__ long long carry;
     const GroupArgs& a = w.g;
     const int g = blockIdx.x;
@@ -594,8 +641,9 @@ __global__ __launch_bounds__(GW_THREADS) void group_scan_kernel(WideArgs w) {
         if (e < entries) {
             const int l = e / a.segs_per_group, s = e - l * a.segs_per_group;
             idx = (int64_t)l * a.nseg + g * a.segs_per_group + s;
-            gt_l[threadIdx.x] = w.cnt[idx * 2];
-            eq_l[threadIdx.x] = w.cnt[idx * 2 + 1];
+            gt_l[threadIdx.x] = w.cnt[idx * 3];
+            eq_l[threadIdx.x] = w.cnt[idx * 3 + 1];
+            row0 = w.cnt[idx * 3 + 2];
         }
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -614,6 +662,7 @@ __global__ __launch_bounds__(GW_THREADS) void group_scan_kernel(WideArgs w) {
         if (e < entries) {
             a.new_len[idx] = len_l[threadIdx.x];
             a.tie_base[idx] = base_l[threadIdx.x];
+            if (a.first_kept) a.first_kept[idx] = (row0 & 1u) || ((row0 & 2u) && (int64_t)base_l[threadIdx.x] < take);
         }
     }
 }
@@ -752,6 +801,7 @@ static int check_layer_args(const char* fn, const trimkv_layer_slabs* layers, in
 
 extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
                                    int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                                   int64_t q_idx, const int64_t* q_idx_dev,
                                    int strategy, int rounding, int sliding_window, int max_len,
                                    void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_evict_layers";
@@ -764,7 +814,7 @@ extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers
     if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
     if (rounding != TRIMKV_ROUND_UPCAST && rounding != TRIMKV_ROUND_NATIVE) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown rounding %d", fn, rounding);
     EvictArgs a = {};
-    a.layers = layers; a.keep_layer_stride = keep_layer_stride;
+    a.layers = layers; a.keep_layer_stride = keep_layer_stride; a.q_idx_all = q_idx; a.q_idx_dev = q_idx_dev;
     a.nseg = nseg; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
     a.keep = keep; a.keep_per_seg = keep_per_seg; a.slack = slack < 0 ? 0 : slack;
     a.strategy = strategy; a.rounding = rounding; a.sliding_window = sliding_window < 0 ? 0 : sliding_window;
@@ -775,7 +825,7 @@ extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers
 extern "C" int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int segs_per_group, int head_dim,
                                                int kv_dtype, int lb_dtype,
                                                const uint32_t* thr_key, const int32_t* tie_take, int thr_layer_stride,
-                                               const int32_t* tie_base, int strategy, int rounding, int max_len,
+                                               const int32_t* tie_base, int64_t q_idx, int strategy, int rounding, int max_len,
                                                void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_compact_threshold_layers";
     int lpr_shift;
@@ -787,7 +837,7 @@ extern "C" int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers,
         return fail(TRIMKV_ERR_SHAPE, "%s: thr_layer_stride must be 0 or nseg/segs_per_group (got %d)", fn, thr_layer_stride);
     if (strategy != TRIMKV_SCORE_ALPHA && strategy != TRIMKV_SCORE_KNORM_ALPHA) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: unknown strategy %d", fn, strategy);
     EvictArgs a = {};
-    a.layers = layers; a.thr_layer_stride = thr_layer_stride;
+    a.layers = layers; a.thr_layer_stride = thr_layer_stride; a.q_idx_all = q_idx;
     a.nseg = nseg; a.row_bytes = head_dim * 2; a.lpr_shift = lpr_shift; a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype;
     a.strategy = strategy; a.rounding = rounding; a.sliding_window = 0;
     a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.segs_per_group = segs_per_group;
@@ -799,7 +849,7 @@ static int group_threshold_common(const char* fn, int per_layer, const void* con
                                       int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                                       int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                                       int64_t q_idx, int strategy, int rounding,
-                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                      uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept,
                                       void* stream) {
     if (!lb_slabs || !pos_slabs || !seg_lens || !thr_key || !tie_take || !tie_base || !new_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if (strategy == TRIMKV_SCORE_KNORM_ALPHA && !k_slabs) return fail(TRIMKV_ERR_NULL, "%s: knorm_alpha needs k_slabs", fn);
@@ -812,7 +862,7 @@ static int group_threshold_common(const char* fn, int per_layer, const void* con
     a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
     a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
     a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
-    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.per_layer = per_layer;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.first_kept = first_kept; a.per_layer = per_layer;
     if (per_layer && nlayers > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nlayers=%d exceeds the grid limit 65535", fn, nlayers);
     hipLaunchKernelGGL(group_threshold_kernel, dim3(nseg / segs_per_group, per_layer ? nlayers : 1), dim3(GT_THREADS), 0, (hipStream_t)stream, a);
     return launch_status(fn);
@@ -822,9 +872,9 @@ static int group_threshold_common(const char* fn, int per_layer, const void* con
 #define TRIMKV_GROUP_PARAMS const void* const* lb_slabs, const int64_t* const* pos_slabs, const void* const* k_slabs, \
     const int32_t* const* seg_lens, int nlayers, int nseg, int segs_per_group, int cap, int head_dim, int kv_dtype, int lb_dtype, \
     int64_t budget, int use_threshold, float threshold_score, int64_t q_idx, int strategy, int rounding, \
-    uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, void* stream
+    uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept, void* stream
 #define TRIMKV_GROUP_ARGS lb_slabs, pos_slabs, k_slabs, seg_lens, nlayers, nseg, segs_per_group, cap, head_dim, kv_dtype, lb_dtype, budget, \
-    use_threshold, threshold_score, q_idx, strategy, rounding, thr_key, tie_take, tie_base, new_len, stream
+    use_threshold, threshold_score, q_idx, strategy, rounding, thr_key, tie_take, tie_base, new_len, first_kept, stream
 
 extern "C" int trimkv_group_threshold(TRIMKV_GROUP_PARAMS) { return group_threshold_common("trimkv_group_threshold", 0, TRIMKV_GROUP_ARGS); }
 
@@ -834,7 +884,7 @@ extern "C" int trimkv_group_threshold_each_layer(TRIMKV_GROUP_PARAMS) {
 
 extern "C" size_t trimkv_group_threshold_workspace(int nlayers, int nseg, int segs_per_group) {
     if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0) return 0;
-    return ((size_t)(nseg / segs_per_group) * 4 * 256 + (size_t)nlayers * nseg * 2) * sizeof(uint32_t);
+    return ((size_t)(nseg / segs_per_group) * 4 * 256 + (size_t)nlayers * nseg * 3) * sizeof(uint32_t);
 }
 
 extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const int64_t* const* pos_slabs,
@@ -842,7 +892,7 @@ extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const in
                                            int nlayers, int nseg, int segs_per_group, int cap, int head_dim,
                                            int kv_dtype, int lb_dtype, int64_t budget, int use_threshold, float threshold_score,
                                            int64_t q_idx, int strategy, int rounding,
-                                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len,
+                                           uint32_t* thr_key, int32_t* tie_take, int32_t* tie_base, int32_t* new_len, int32_t* first_kept,
                                            void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_group_threshold_wide";
     if (!lb_slabs || !pos_slabs || !seg_lens || !thr_key || !tie_take || !tie_base || !new_len) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
@@ -862,7 +912,7 @@ extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const in
     a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
     a.kv_dtype = kv_dtype; a.lb_dtype = lb_dtype; a.budget = budget; a.use_threshold = use_threshold; a.threshold_score = threshold_score;
     a.q_idx = q_idx; a.strategy = strategy; a.rounding = rounding;
-    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.per_layer = 0;
+    a.thr_key = thr_key; a.tie_take = tie_take; a.tie_base = tie_base; a.new_len = new_len; a.first_kept = first_kept; a.per_layer = 0;
     w.hist = (uint32_t*)workspace;
     w.cnt = w.hist + (size_t)ngroups * 4 * 256;
     hipStream_t st = (hipStream_t)stream;
