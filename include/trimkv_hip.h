@@ -301,12 +301,15 @@ int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlen
  * the order their workgroups should be dispatched -- longest first when lengths are very uneven, so
  * that the long segments do not form the tail of the launch (about 15 % at lognormal lengths).  It
  * changes scheduling only; entries are clamped to [0, nseg).
+ * seg_first (optional, may be NULL): int32 [nseg]; segment seg attends rows [seg_first[seg], seg_len[seg]) only (clamped to the
+ * segment).  This is how a left-padding attention_mask reaches the kernel at decode time: the padded prefix of a batch
+ * element is skipped for each of its heads (HF flash_attention_2 drops the same columns, src/trimkv/attn/__init__.py:15-26).
  * head_dim must be 128, 96 or 64 (the kernel is laid out for 128; shorter rows run zero-padded to
  * it); group in [1, 8]; dtype bf16 or fp16 (q, K, V and out alike).
  */
 size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim, int max_len, int chunk);
 int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
-                       const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                       const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                        int nseg, int cap, int head_dim, int group, int dtype, float scale,
                        int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream);
 
@@ -347,7 +350,7 @@ int trimkv_append_attend(const void* q, void* out,
  */
 #define TRIMKV_DECODE_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
 int trimkv_decode_attn_static(const void* q, void* out, const void* k_slab, const void* v_slab,
-                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                               int nseg, int cap, int head_dim, int group, int dtype, float scale,
                               int max_len, int chunk, void* stream);
 

@@ -159,7 +159,7 @@ int main() {
     void* dWS = nullptr;
     HIP_OK(hipMalloc(&dWS, ws_bytes ? ws_bytes : 16));
     const float scale = 1.0f / std::sqrt((float)D);
-    TRIMKV_OK(trimkv_decode_attn(dQ, dO, dK, dV, dLEN, nullptr, nullptr, nseg, cap, D, G, TRIMKV_BF16, scale, keep, 64, dWS, ws_bytes, stream));
+    TRIMKV_OK(trimkv_decode_attn(dQ, dO, dK, dV, dLEN, nullptr, nullptr, nullptr, nseg, cap, D, G, TRIMKV_BF16, scale, keep, 64, dWS, ws_bytes, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::vector<uint16_t> gO((size_t)nseg * G * D);
     if (!to_host(gO, dO)) return 2;
@@ -186,7 +186,7 @@ int main() {
         }
 
     // ---- argument errors come back as negative codes with a message, and nothing is launched ----
-    if (trimkv_decode_attn(dQ, dO, dK, dV, dLEN, nullptr, nullptr, nseg, cap, 80, G, TRIMKV_BF16, scale, keep, 0, nullptr, 0, stream) != TRIMKV_ERR_UNSUPPORTED ||
+    if (trimkv_decode_attn(dQ, dO, dK, dV, dLEN, nullptr, nullptr, nullptr, nseg, cap, 80, G, TRIMKV_BF16, scale, keep, 0, nullptr, 0, stream) != TRIMKV_ERR_UNSUPPORTED ||
         std::strlen(trimkv_last_error()) == 0) {
         std::printf("a head_dim of 80 should be refused with a message\n");
         return 1;

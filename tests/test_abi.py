@@ -54,13 +54,13 @@ def test_bad_arguments_are_refused_without_a_launch():
     base = dict(nseg=4, cap=64, D=128, G=4, dt=_lib.BF16, max_len=64, chunk=0)
     def attn(**kw):
         a = dict(base); a.update(kw)
-        return lib.trimkv_decode_attn(one, one, one, one, one, None, None, a["nseg"], a["cap"], a["D"], a["G"], a["dt"], 0.1,
+        return lib.trimkv_decode_attn(one, one, one, one, one, None, None, None, a["nseg"], a["cap"], a["D"], a["G"], a["dt"], 0.1,
                                       a["max_len"], a["chunk"], None, 0, None)
     assert attn(D=80) == -6 and attn(D=256) == -6 and attn(G=9) == -6 and attn(dt=_lib.F32) == -3
     assert attn(max_len=128) == -4            # longer than the slab
     assert attn(cap=4096, max_len=4096, chunk=256) == -5  # split-K needs a workspace
     assert attn(chunk=100) == -2
-    assert lib.trimkv_decode_attn(None, one, one, one, one, None, None, 4, 64, 128, 4, _lib.BF16, 0.1, 64, 0, None, 0, None) == -1
+    assert lib.trimkv_decode_attn(None, one, one, one, one, None, None, None, 4, 64, 128, 4, _lib.BF16, 0.1, 64, 0, None, 0, None) == -1
     # eviction: capacity, strategy, alignment of head_dim
     def evict(cap=64, D=128, keep=8, strat=0, rnd=0, max_len=64):
         return lib.trimkv_evict(one, one, one, one, one, 4, cap, D, _lib.BF16, _lib.F32, keep, None, 0, 100, strat, rnd, 0,

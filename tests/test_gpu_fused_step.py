@@ -207,7 +207,7 @@ def test_c_abi_append_attend_other_shapes_full_slabs_and_cu(D, dtype, lb_dtype):
         L.check(lib.trimkv_append(a["k"].data_ptr(), a["v"].data_ptr(), a["lb"].data_ptr(), a["pos"].data_ptr(), a["seg_len"].data_ptr(),
                                   a["cu"].data_ptr(), nseg, H, cap, D, code, lcode, kn.data_ptr(), vn.data_ptr(), *kn.stride()[:3],
                                   lbn.data_ptr(), *lbn.stride(), posn.data_ptr(), 0, 0, 1, 1, cap, st), "append")
-        L.check(lib.trimkv_decode_attn(q.data_ptr(), want.data_ptr(), a["k"].data_ptr(), a["v"].data_ptr(), a["seg_len"].data_ptr(), None, None,
+        L.check(lib.trimkv_decode_attn(q.data_ptr(), want.data_ptr(), a["k"].data_ptr(), a["v"].data_ptr(), a["seg_len"].data_ptr(), None, None, None,
                                        nseg, cap, D, G, code, scale, cap, chunk, ws.data_ptr(), ws.numel(), st), "attn")
         L.check(lib.trimkv_append_attend(q.data_ptr(), got.data_ptr(), b["k"].data_ptr(), b["v"].data_ptr(), b["lb"].data_ptr(), b["pos"].data_ptr(),
                                          b["seg_len"].data_ptr(), b["cu"].data_ptr(), None, nseg, H, cap, D, G, code, lcode,

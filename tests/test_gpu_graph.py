@@ -47,7 +47,7 @@ def test_decode_step_replays_from_a_hip_graph():
             L.check(lib.trimkv_append(s["K"].data_ptr(), s["V"].data_ptr(), s["LB"].data_ptr(), s["POS"].data_ptr(), s["LEN"].data_ptr(), None,
                                       nseg, H, cap, D, L.BF16, L.F32, k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), k.stride(2),
                                       lb.data_ptr(), lb.stride(0), lb.stride(1), lb.stride(2), posin.data_ptr(), 0, 0, 1, 1, cap, stream), "append")
-            L.check(lib.trimkv_decode_attn(qin[l].data_ptr(), out[l].data_ptr(), s["K"].data_ptr(), s["V"].data_ptr(), s["LEN"].data_ptr(), None, None,
+            L.check(lib.trimkv_decode_attn(qin[l].data_ptr(), out[l].data_ptr(), s["K"].data_ptr(), s["V"].data_ptr(), s["LEN"].data_ptr(), None, None, None,
                                            nseg, cap, D, G, L.BF16, D ** -0.5, cap, 0, ws.data_ptr(), ws.numel(), stream), "attn")
 
     side = torch.cuda.Stream()

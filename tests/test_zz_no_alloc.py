@@ -32,11 +32,11 @@ def _run_both(lib, L, c):
     got = torch.full_like(c["q"], -7.0)
     print(f"decode_attn vs decode_attn_static: nseg={c['nseg']} cap={c['cap']} G={c['G']} max_len={c['max_len']} chunk={c['chunk']} "
           f"partials={need} bytes", flush=True)
-    rc = lib.trimkv_decode_attn(c["q"].data_ptr(), want.data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["seg_len"].data_ptr(), None, None,
+    rc = lib.trimkv_decode_attn(c["q"].data_ptr(), want.data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["seg_len"].data_ptr(), None, None, None,
                                 c["nseg"], c["cap"], c["D"], c["G"], L.BF16, scale, c["max_len"], c["chunk"], ws.data_ptr(), ws.numel(), st)
     L.check(rc, "trimkv_decode_attn")
     before = torch.cuda.memory_allocated()
-    rc = lib.trimkv_decode_attn_static(c["q"].data_ptr(), got.data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["seg_len"].data_ptr(), None, None,
+    rc = lib.trimkv_decode_attn_static(c["q"].data_ptr(), got.data_ptr(), c["k"].data_ptr(), c["v"].data_ptr(), c["seg_len"].data_ptr(), None, None, None,
                                        c["nseg"], c["cap"], c["D"], c["G"], L.BF16, scale, c["max_len"], c["chunk"], st)
     L.check(rc, "trimkv_decode_attn_static")
     assert torch.cuda.memory_allocated() == before
@@ -71,7 +71,7 @@ def test_static_entry_point_refuses_what_does_not_fit():
     nseg, G, max_len, chunk = 4096, 8, 8192, 64
     need = lib.trimkv_decode_attn_workspace(nseg, G, 128, max_len, chunk)
     assert need > STATIC_BYTES
-    rc = lib.trimkv_decode_attn_static(one, one, one, one, one, None, None, nseg, max_len, 128, G, L.BF16, 0.1, max_len, chunk, None)
+    rc = lib.trimkv_decode_attn_static(one, one, one, one, one, None, None, None, nseg, max_len, 128, G, L.BF16, 0.1, max_len, chunk, None)
     assert rc == -5   # TRIMKV_ERR_WORKSPACE
     msg = lib.trimkv_last_error().decode()
     assert "scratch" in msg and str(need) in msg

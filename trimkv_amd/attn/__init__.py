@@ -42,6 +42,30 @@ def _adapt_hf_attention(name: str):
 get_trimkv_wrapper = _adapt_hf_attention   # the reference's name for the same adapter
 
 
+def register_with_transformers() -> bool:
+    """Make ``"trimkv_hip"`` a key that HF's own machinery accepts (``config._attn_implementation = "trimkv_hip"``): the
+    attention function in ``AttentionInterface`` (HF's two-value return) and, for the mask preparation of HF model code
+    (``create_causal_mask`` looks the key up), the mask builder of ``flash_attention_2`` -- None without padding, else the
+    2-D keep-mask, which ``dense_attention_forward`` turns into per-segment first rows.  Returns False when the installed
+    transformers has no such registries."""
+    try:
+        from transformers import AttentionInterface, AttentionMaskInterface
+        from transformers.masking_utils import ALL_MASK_ATTENTION_FUNCTIONS
+    except Exception:
+        return False
+
+    def hf_trimkv_hip(module, query, key, value, attention_mask=None, **kwargs):
+        out, weights, _ = hip_attn.dense_attention_forward(module, query, key, value, attention_mask, **kwargs)
+        return out, weights
+
+    AttentionInterface.register("trimkv_hip", hf_trimkv_hip)
+    AttentionMaskInterface.register("trimkv_hip", ALL_MASK_ATTENTION_FUNCTIONS["flash_attention_2"])
+    return True
+
+
+register_with_transformers()
+
+
 def get_attention_interface(attn_impl: str, compile: bool = False):
     """Name -> callable.  ``compile`` wraps an HF fallback in ``torch.compile`` as the reference does; the entries backed
     by libtrimkv_hip.so are ctypes launches of hand-written kernels and are returned as they are."""

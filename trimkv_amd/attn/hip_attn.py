@@ -18,6 +18,8 @@ ragged entry points ignore ``attention_mask`` and ``scaling`` (flash_attn.py:15,
 """
 from __future__ import annotations
 
+import os
+import warnings
 from typing import Dict, Optional, Tuple
 
 import torch
@@ -27,6 +29,18 @@ from .. import _lib
 
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
 _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
+_WARNED = set()
+
+
+def slow_path(what: str) -> None:
+    """A call is about to run on torch ops instead of the HIP kernels: say so once per cause, or refuse when the
+    environment asks for strictness (``TRIMKV_STRICT=1``)."""
+    if os.environ.get("TRIMKV_STRICT", "0") not in ("", "0"):
+        raise _lib.TrimKVLibraryError(f"{what}: this call would leave the HIP kernels for torch ops (TRIMKV_STRICT is set)")
+    if what not in _WARNED:
+        _WARNED.add(what)
+        warnings.warn(f"trimkv_amd: {what}: running on torch ops, not on the HIP kernels (set TRIMKV_STRICT=1 to make this an error)",
+                      RuntimeWarning, stacklevel=3)
 
 
 def _group_slice(group: int) -> int:
@@ -48,16 +62,18 @@ def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[to
 
 def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, nseg: int, group: int,
                      seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
-                     scale: float, chunk: int = 0, seg_order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     scale: float, chunk: int = 0, seg_order: Optional[torch.Tensor] = None,
+                     seg_first: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``.
-    ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only)."""
+    ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only).
+    ``seg_first``: optional int32 [nseg], the first attended row of every segment (rows before it are masked)."""
     if not query.is_cuda:
         raise _lib.TrimKVLibraryError("decode attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
     if group > _MAX_GROUP:   # more query heads per KV head than one launch takes: several launches over slices of the group
         g1 = _group_slice(group)
         q3 = query.view(nseg, group, -1)
         outs = [decode_attention(q3[:, a:a + g1].reshape(nseg * g1, -1), k_rows, v_rows, nseg, g1, seg_len, seg_start, cap, max_len,
-                                 scale, chunk, seg_order).view(nseg, g1, -1) for a in range(0, group, g1)]
+                                 scale, chunk, seg_order, seg_first).view(nseg, g1, -1) for a in range(0, group, g1)]
         return torch.cat(outs, dim=1).view(nseg * group, -1)
     lib = _lib.load()
     d = query.shape[-1]
@@ -65,7 +81,8 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
     ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, max_len, chunk)
     ws = _workspace(query.device, ws_bytes)
     rc = lib.trimkv_decode_attn(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(),
-                                _lib.ptr(seg_len), _lib.ptr(seg_start), _lib.ptr(seg_order), nseg, cap, d, group, _lib.dtype_code(query.dtype),
+                                _lib.ptr(seg_len), _lib.ptr(seg_start), _lib.ptr(seg_order), _lib.ptr(seg_first), nseg, cap, d, group,
+                                _lib.dtype_code(query.dtype),
                                 float(scale), max_len, chunk, _lib.ptr(ws), 0 if ws is None else ws.numel(),
                                 _lib.current_stream(query.device))
     _lib.check(rc, "trimkv_decode_attn")
@@ -144,6 +161,32 @@ def _causal_bottom_right(qlen: int, n: int, device) -> torch.Tensor:
     return j <= (n - qlen + t)
 
 
+_PAD_CACHE: Dict[str, tuple] = {}
+
+
+def _left_padding_offsets(attention_mask: torch.Tensor, batch: int, n: int, kv_heads: int) -> Optional[torch.Tensor]:
+    """If ``attention_mask`` only hides a prefix of every batch element's keys -- left padding, the layout batched
+    generation uses -- return the per-segment first visible row (int32 [batch*kv_heads]); otherwise None.
+    Accepted forms: the 2-D ``[B, n]`` keep-mask (1/True = attend) that HF hands to flash_attention_2, and the 4-D
+    additive ``[B, 1, 1, n]`` mask of the sdpa/eager paths (0 = attend).  Whether the mask really is a prefix is checked
+    on the device and read back once per mask tensor (all layers of a step pass the same tensor)."""
+    if attention_mask.dim() == 2 and tuple(attention_mask.shape) == (batch, n):
+        keep = attention_mask != 0
+    elif attention_mask.dim() == 4 and tuple(attention_mask.shape[:3]) == (batch, 1, 1) and attention_mask.shape[3] >= n:
+        keep = attention_mask[:, 0, 0, :n] == 0
+    else:
+        return None
+    key = (attention_mask.data_ptr(), tuple(attention_mask.shape), attention_mask._version, kv_heads)
+    hit = _PAD_CACHE.get("last")
+    if hit is not None and hit[0] == key:
+        return hit[1]
+    first = n - keep.sum(dim=-1, dtype=torch.int32)                                   # rows hidden per batch element
+    is_prefix = bool((keep == (torch.arange(n, device=keep.device)[None, :] >= first[:, None])).all())   # one read-back per new mask
+    seg_first = first.to(torch.int32).repeat_interleave(kv_heads).contiguous() if is_prefix else None
+    _PAD_CACHE["last"] = (key, seg_first)
+    return seg_first
+
+
 def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                             attention_mask: Optional[torch.Tensor] = None, scaling: Optional[float] = None,
                             dropout: float = 0.0, flash_attn_kwargs: Optional[dict] = None, **kwargs):
@@ -158,7 +201,10 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         if not q2.is_contiguous():
             q2 = q2.contiguous()
         return append_attend(slab, q2, G, scale).view(B, 1, Hq, D), None, None
-    if Q == 1 and attention_mask is None:
+    seg_first = None
+    if attention_mask is not None and Q == 1 and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
+        seg_first = _left_padding_offsets(attention_mask, B, n, Hkv)   # a left-padding mask is a per-segment first row
+    if Q == 1 and (attention_mask is None or seg_first is not None):
         ks = key.stride()
         if not (ks[3] == 1 and ks[2] == D and ks[0] == Hkv * ks[1] and value.stride() == ks and ks[1] % D == 0):
             key, value = key.contiguous(), value.contiguous()
@@ -170,7 +216,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
-        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale)
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, seg_first=seg_first)
         return out.view(B, 1, Hq, D), None, None
     if attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
@@ -182,7 +228,13 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             seg_len = None
         out = prefill_attention(query, key, value, B, Hkv, G, seg_len, None, key.stride(1) // D, n, scale)
         return out, None, None
-    # masked batches (padding): torch ops
+    # what is left: masks that are not a left-padding prefix at Q_LEN == 1, any mask with a query block, fp32 tensors,
+    # other head dims -- torch ops, announced
+    slow_path("dense attention with " + ("an attention_mask that is not plain left padding at decode time" if attention_mask is not None and Q == 1
+                                         else "an attention_mask on a query block" if attention_mask is not None
+                                         else f"dtype {query.dtype} / head_dim {D}"))
+    if attention_mask is not None and attention_mask.dim() == 2:   # HF's 2-D keep-mask -> additive
+        attention_mask = torch.zeros(B, 1, 1, n, dtype=torch.float32, device=query.device).masked_fill(attention_mask[:, None, None, :n] == 0, float("-inf"))
     k = key.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
     v = value.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
     w = torch.matmul(query, k.transpose(2, 3)).float() * scale

@@ -674,6 +674,9 @@ class _RaggedCache(_SlabBacked):
         self.batch_size: Optional[int] = None
         self.num_kv_heads: Optional[int] = None
         self._tables: Dict[Any, torch.Tensor] = {}
+        # update() normally hands the attention call the slab rows plus ``seg_start`` (no copy).  With this flag, or with
+        # ``cache_kwargs={"packed": True}`` on a call, it returns the reference's packed ``[sum(n), D]`` tensors instead.
+        self.return_packed = False
 
     # plain attributes in the reference; a property here because newer HF Cache classes define a
     # read-only `batch_size` of their own
@@ -701,20 +704,38 @@ class _RaggedCache(_SlabBacked):
         s = self._slabs[layer]
         return 0 if s is None else int(s.lens.sum())
 
-    def _update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int):
+    def _packed(self, slab: _Slab):
+        """The layer in the reference's own layout (cache_utils.py:682-689): ``[sum(n), D]`` rows packed segment after
+        segment, indexed by ``cu_seqlens_k``.  A copy, gathered on the device without a host synchronisation (the row
+        count comes from the host mirror of the lengths); for readers that index the returned K with the returned
+        ``cu_seqlens_k`` themselves, as flash_attn_varlen_func does (attn/flash_attn.py:135-145)."""
+        dev = slab.k.device
+        r = torch.arange(slab.total, device=dev, dtype=torch.int32)
+        seg = torch.searchsorted(slab.cu[1:], r, right=True)
+        src = seg * slab.cap + (r - slab.cu[seg])
+        flat = (slab.k.view(-1, slab.D).index_select(0, src), slab.v.view(-1, slab.D).index_select(0, src),
+                slab.lb.view(-1).index_select(0, src).unsqueeze(-1), slab.pos.view(-1).index_select(0, src).unsqueeze(-1))
+        kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu, "max_len": slab.max_len}
+        return flat, kw
+
+    def _update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int, packed: bool = False):
+        packed = packed or self.return_packed
         if key_states is not None:
             S = key_states.shape[2]
             if layer_idx == 0:
                 self._seen_tokens += S
             self._ensure_layer(layer_idx)
             slab = self._slabs[layer_idx]
-            if not (S == 1 and self.fuse_decode_append and slab is not None
+            if not (S == 1 and self.fuse_decode_append and not packed and slab is not None
                     and self._defer(slab, key_states, value_states, retention_weights, cache_positions)):
                 self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
             # on the first call cu starts as zeros and the kernel's "cu[i] += i*S" yields
             # arange(0, nseg*S+1, S), what the reference builds at cache_utils.py:297, 643
             self.n_seen_tokens[layer_idx] += S
         slab = self._slabs[layer_idx]
+        if packed:
+            self._flush(slab)
+            return self._packed(slab)
         # split-K chunk for ragged lengths: about 384 pieces over the rows actually cached (the library's own default
         # assumes every segment is max_len long); measured on 256 lognormal segments (128..8256 rows, 410 k rows): 1088-row pieces 52 us, 832 54.7, 1664 53 -- pieces
         # long enough to stream, short enough that no compute unit ends up with much more than its share
@@ -989,7 +1010,8 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             else:
                 assert B == self.batch_size, f"Batch size changed: {self.batch_size} -> {B}"
                 assert H == self.num_kv_heads, f"Num KV heads changed: {self.num_kv_heads} -> {H}"
-        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx)
+        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx,
+                                bool(cache_kwargs and cache_kwargs.get("packed")))
         kw["batch_size"], kw["num_kv_heads"] = self.batch_size, self.num_kv_heads
         return (*flat, kw)
 
@@ -1061,7 +1083,8 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
         if key_states is not None:
             assert key_states.shape[0] == 1, "Batch size greater than 1 is not supported for DynamicBudgetTrimKVCache"
             self.batch_size, self.num_kv_heads = 1, key_states.shape[1]
-        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx)
+        flat, kw = self._update(key_states, value_states, retention_weights, cache_positions, layer_idx,
+                                bool(cache_kwargs and cache_kwargs.get("packed")))
         return (*flat, kw)
 
     def get_cache_length(self, layer_idx: int = 0, head_idx: int = 0) -> int:

@@ -11,11 +11,11 @@ extern "C" size_t trimkv_decode_attn_workspace(int nseg, int group, int head_dim
 }
 
 static int decode_attn_common(const char* fn, const void* q, void* out, const void* k_slab, const void* v_slab,
-                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                               int nseg, int cap, int head_dim, int group, int dtype, float scale,
                               int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
     AttnArgs a;
-    const int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, seg_start, seg_order, nseg, cap, head_dim, group, dtype, scale,
+    const int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, seg_start, seg_order, seg_first, nseg, cap, head_dim, group, dtype, scale,
                                 max_len, chunk, workspace, workspace_bytes);
     if (rc) return rc;
     launch_attn_group<false>(a, group, head_dim, dtype, (hipStream_t)stream);
@@ -23,10 +23,10 @@ static int decode_attn_common(const char* fn, const void* q, void* out, const vo
 }
 
 extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void* v_slab,
-                                  const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                                  const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                                   int nseg, int cap, int head_dim, int group, int dtype, float scale,
                                   int max_len, int chunk, void* workspace, size_t workspace_bytes, void* stream) {
-    return decode_attn_common("trimkv_decode_attn", q, out, k_slab, v_slab, seg_len, seg_start, seg_order, nseg, cap, head_dim, group,
+    return decode_attn_common("trimkv_decode_attn", q, out, k_slab, v_slab, seg_len, seg_start, seg_order, seg_first, nseg, cap, head_dim, group,
                               dtype, scale, max_len, chunk, workspace, workspace_bytes, stream);
 }
 
@@ -54,7 +54,7 @@ static int static_scratch(const char* fn, void** out_ptr) {
 }
 
 extern "C" int trimkv_decode_attn_static(const void* q, void* out, const void* k_slab, const void* v_slab,
-                                         const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                                         const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                                          int nseg, int cap, int head_dim, int group, int dtype, float scale,
                                          int max_len, int chunk, void* stream) {
     const char* fn = "trimkv_decode_attn_static";
@@ -67,6 +67,6 @@ extern "C" int trimkv_decode_attn_static(const void* q, void* out, const void* k
         const int rc = static_scratch(fn, &ws);
         if (rc) return rc;
     }
-    return decode_attn_common(fn, q, out, k_slab, v_slab, seg_len, seg_start, seg_order, nseg, cap, head_dim, group, dtype, scale,
+    return decode_attn_common(fn, q, out, k_slab, v_slab, seg_len, seg_start, seg_order, seg_first, nseg, cap, head_dim, group, dtype, scale,
                               max_len, chunk, ws, need ? (size_t)TRIMKV_DECODE_ATTN_STATIC_SCRATCH_BYTES : 0, stream);
 }

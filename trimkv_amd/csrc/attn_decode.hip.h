@@ -115,6 +115,7 @@ struct AppendPart {
 struct AttnArgs {
     const uint4* q; void* out; const uint4* k; const uint4* v;
     const int32_t* seg_len; const int32_t* seg_start; const int32_t* seg_order;
+    const int32_t* seg_first;   // optional: rows before seg_first[seg] are not attended (left padding)
     int nseg, cap, max_len, chunk, nsplit, direct;
     float scale_log2;
     float* ws_o; float* ws_ml;
@@ -123,15 +124,18 @@ struct AttnArgs {
 
 // Length of segment `seg` as the launch sees it.  APPEND: the stored length is the one before this step's token; the token
 // lands in row n_old (returned through *new_row) unless the slab is full, in which case nothing is appended (-1).
+// *first: the first attended row (0 unless the caller masks a prefix of the segment).
 template <bool APPEND>
-__device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new_row) {
+__device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new_row, int* first) {
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     *new_row = -1;
     if (APPEND) {
         n = max(n, 0);
         if (n + 1 <= a.cap && n + 1 <= a.max_len) { *new_row = n; n += 1; }
     }
-    return max(0, min(n, a.max_len));
+    n = max(0, min(n, a.max_len));
+    *first = a.seg_first ? min(max(a.seg_first[seg], 0), n) : 0;
+    return n;
 }
 
 // Attention of the G query heads of segment `seg` over its rows [t0, t1): the body shared by both kernels.
@@ -441,17 +445,18 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     int seg = blockIdx.x;
     if (a.seg_order) seg = min(max(a.seg_order[seg], 0), a.nseg - 1);
     const int split = (int)gridDim.y - 1 - (int)blockIdx.y;
-    int new_row;
-    const int n = segment_rows<APPEND>(a, seg, &new_row);
-    const int nsp = (n + a.chunk - 1) / a.chunk;
+    int new_row, first;
+    const int n = segment_rows<APPEND>(a, seg, &new_row, &first);
+    const int live = n - first;
+    const int nsp = (live + a.chunk - 1) / a.chunk;
     if (split >= nsp) {
-        if (n == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
+        if (live == 0 && split == 0 && a.direct) {  // an empty segment attends to nothing: zeros
             for (int i = threadIdx.x; i < G * ROW16 * 8; i += AT_THREADS) ((uint16_t*)a.out)[((int64_t)seg * G) * (ROW16 * 8) + i] = 0;
         }
         return;
     }
-    const int rps = (n + nsp - 1) / nsp;
-    const int t0 = split * rps, t1 = min(n, t0 + rps);
+    const int rps = (live + nsp - 1) / nsp;
+    const int t0 = first + split * rps, t1 = min(n, t0 + rps);
     attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split, new_row);
 }
 
@@ -463,8 +468,8 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
 template <int G, int ROW16, bool F16, bool APPEND>
 __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
     const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
-    int new_row;
-    const int n = segment_rows<APPEND>(a, seg, &new_row);
+    int new_row, first;
+    const int n = segment_rows<APPEND>(a, seg, &new_row, &first);
     if (APPEND) {
         // The split workgroups of the main launch all read the old length, so it is advanced here, by the only workgroup of
         // this launch that reads it, once all of its threads have.
@@ -474,7 +479,7 @@ __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a)
             if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;
         }
     }
-    const int nsp = (n + a.chunk - 1) / a.chunk;
+    const int nsp = (n - first + a.chunk - 1) / a.chunk;
     const int64_t slot0 = ((int64_t)seg * a.nsplit) * G + g;
     // every load of a batch of 8 splits is issued before anything is used: one memory round trip per batch
     float mx = AT_NEG, acc = 0.0f, lsum = 0.0f;
@@ -556,7 +561,7 @@ static void launch_attn_group(const AttnArgs& a, int group, int head_dim, int dt
 
 // Argument checks and split-K set-up shared by the entry points; fills `a` except for a.ap.
 static int prepare_attn(const char* fn, AttnArgs& a, const void* q, void* out, const void* k_slab, const void* v_slab,
-                        const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order,
+                        const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_order, const int32_t* seg_first,
                         int nseg, int cap, int head_dim, int group, int dtype, float scale,
                         int max_len, int chunk, void* workspace, size_t workspace_bytes) {
     if (!q || !out || !k_slab || !v_slab) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
@@ -569,7 +574,7 @@ static int prepare_attn(const char* fn, AttnArgs& a, const void* q, void* out, c
     if (chunk <= 0) chunk = pick_chunk(nseg, max_len);
     if (chunk % 64) return fail(TRIMKV_ERR_SHAPE, "%s: chunk must be a multiple of 64 (got %d)", fn, chunk);
     a.q = (const uint4*)q; a.out = out; a.k = (const uint4*)k_slab; a.v = (const uint4*)v_slab;
-    a.seg_len = seg_len; a.seg_start = seg_start; a.seg_order = seg_order; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
+    a.seg_len = seg_len; a.seg_start = seg_start; a.seg_order = seg_order; a.seg_first = seg_first; a.nseg = nseg; a.cap = cap; a.max_len = max_len; a.chunk = chunk;
     a.nsplit = (max_len + chunk - 1) / chunk;
     if (a.nsplit > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: max_len/chunk = %d splits exceeds the grid limit 65535", fn, a.nsplit);
     a.direct = a.nsplit <= 1;

@@ -26,7 +26,7 @@ extern "C" int trimkv_append_attend(const void* q, void* out,
     if (((kv_stride_b * 2) | (kv_stride_h * 2)) & 15 || ((uintptr_t)k_new & 15) || ((uintptr_t)v_new & 15))
         return fail(TRIMKV_ERR_SHAPE, "%s: new K/V rows must be 16-byte aligned (strides %lld,%lld elements)", fn, (long long)kv_stride_b, (long long)kv_stride_h);
     AttnArgs a;
-    const int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, seg_order, nseg, cap, head_dim, group, kv_dtype, scale,
+    const int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, seg_order, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
                                 max_len_after, chunk, workspace, workspace_bytes);
     if (rc) return rc;
     a.ap.k_new = (const char*)k_new; a.ap.v_new = (const char*)v_new; a.ap.kv_sb = kv_stride_b * 2; a.ap.kv_sh = kv_stride_h * 2;

@@ -70,6 +70,12 @@ class RetentionGate(nn.Module):
     def forward(self, x: torch.Tensor):
         """x [B, S, hidden] -> log beta [B, S, Hkv] (a LazyLogBeta on the fused path)."""
         if not self._use_hip(x):
+            if self.fused and not self.training and x.is_cuda and x.dtype in (torch.bfloat16, torch.float16):
+                # an inference call on the GPU that the fused kernels cannot take (shape or activation): say so
+                from .attn.hip_attn import slow_path
+                slow_path(f"retention gate with hidden size {x.shape[-1]} (needs a multiple of 512), intermediate size "
+                          f"{self.retention_gate_intermediate_size} (a multiple of 16), activation {self.hidden_act} (silu) "
+                          f"or a bias of another dtype than the input")
             return self._torch_forward(x)
         B, S, hidden = x.shape
         lib = _lib.load()
