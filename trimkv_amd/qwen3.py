@@ -229,6 +229,9 @@ class TrimKVQwen3Model(nn.Module):
             inputs_embeds = self.embed_tokens(input_ids)
         if past_key_values is None:   # qwen3:648-652
             past_key_values = TrimKVCache(max_seq_len=self.config.max_seq_len, device=inputs_embeds.device)
+            # this model reads what update() returns only through the registered attention of the same layer: a decode
+            # step's append can ride on that launch
+            past_key_values.fuse_decode_append = self.config._attn_implementation == "trimkv_hip"
         if cache_position is None:
             seen = past_key_values.get_seq_length()
             cache_position = torch.arange(seen, seen + inputs_embeds.shape[1], device=inputs_embeds.device)
