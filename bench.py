@@ -433,8 +433,7 @@ def main():
     mod = Mod()
     attn_fn = get_attention_interface("trimkv_hip")
     if args.chunk:
-        _orig = hip_attn.decode_attention
-        hip_attn.decode_attention = lambda *a, **k: _orig(*a, **{**k, "chunk": args.chunk})
+        hip_attn.dense_chunk = args.chunk
 
     # Cycle of the steady state: an eviction takes every head to M rows, the next buf steps attend M+1 .. M+buf rows and the
     # last of them evicts again.  The cache starts one row short of the trigger, so the first warm-up step evicts.
@@ -574,7 +573,7 @@ def main():
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
         targs = f"<{G}, 16, false, {'true' if fused else 'false'}>"
-        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 128 else " + decode_attn_merge_kernel" + targs), "achieved": round(achieved, 1),
+        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 256 else " + decode_attn_merge_kernel" + targs), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "traffic_measured_in_run": False,
@@ -602,7 +601,7 @@ def main():
                                f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
                    "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(),
                    "launches_per_layer_step": ("1: append + attend in one launch (trimkv_append_attend)" if cache.fuse_decode_append and not args.gate
-                                               else "2: trimkv_append, trimkv_decode_attn") + ("" if B * Hkv >= 128 else " + split-K merge"),
+                                               else "2: trimkv_append, trimkv_decode_attn") + ("" if B * Hkv >= 256 else " + split-K merge"),
                    **timing},
         "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
                      "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

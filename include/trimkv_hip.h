@@ -291,7 +291,7 @@ int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlen
  * rows (a dense cache).  max_len is the caller's upper bound on seg_len (longer segments are
  * truncated to it).  A segment of length 0 yields zeros.
  * Split-K: every segment is cut into chunks of `chunk` rows (a multiple of 64).  0 lets the library
- * choose from nseg and max_len alone -- one chunk per segment from 128 segments on, which is right
+ * choose from nseg and max_len alone -- one chunk per segment from 256 segments on, which is right
  * for near-equal lengths; a caller that knows its lengths are very uneven should pass about
  * total_rows / 512 (at least 512) so that a few long segments do not run on one workgroup each
  * (the Python ragged caches do).  Partial (max, sum, accumulator)

@@ -126,9 +126,9 @@ def _fp32_attention_on_segments(q, K, V, segs, G, n):
 
 @pytest.mark.parametrize("n", [2049, 2112, 2176])
 def test_config2_decode_attention_full_shape(n):
-    """BASELINE config 2's decode shape: batch 16 x 8 KV heads = 128 segments of 2049..2176 rows, 16 query heads (G=2) --
-    the shape at which the launch stops splitting segments (one workgroup per segment).  Through update() + the registered
-    attention, against fp32 softmax on sampled segments; a split launch of the same inputs must agree."""
+    """BASELINE config 2's decode shape: batch 16 x 8 KV heads = 128 segments of 2049..2176 rows, 16 query heads (G=2); the
+    library cuts every segment in two here (256 workgroups) and merges.  Through update() + the registered attention,
+    against fp32 softmax on sampled segments; launches with whole segments and with other piece sizes must agree."""
     from trimkv_amd import get_attention_interface
     from trimkv_amd.attn.hip_attn import decode_attention
     B, H, G = 16, 8, 2
@@ -146,8 +146,9 @@ def test_config2_decode_attention_full_shape(n):
     ok, err = attn_close(out.view(B * H, G, 128)[segs], want)
     assert ok, err
     assert torch.equal(slab.k[:, n - 1], kn.view(B * H, 128)) and torch.equal(slab.v[:, n - 1], vn.view(B * H, 128))
-    split = decode_attention(q.view(B * H * G, 128), slab.k, slab.v, B * H, G, slab.seg_len, None, slab.cap, n, 128 ** -0.5, chunk=1088)
-    assert (split.float() - out.view(-1, 128).float()).abs().max() < 4e-3
+    for chunk in (4096, 704):      # whole segments; four pieces
+        other = decode_attention(q.view(B * H * G, 128), slab.k, slab.v, B * H, G, slab.seg_len, None, slab.cap, n, 128 ** -0.5, chunk=chunk)
+        assert (other.float() - out.view(-1, 128).float()).abs().max() < 4e-3
 
 
 @pytest.mark.parametrize("n", [8193, 8448, 8704])

@@ -30,6 +30,7 @@ from .. import _lib
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
 _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
 _WARNED = set()
+dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)
 
 
 def slow_path(what: str) -> None:
@@ -200,7 +201,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        return append_attend(slab, q2, G, scale).view(B, 1, Hq, D), None, None
+        return append_attend(slab, q2, G, scale, chunk=dense_chunk).view(B, 1, Hq, D), None, None
     seg_first = None
     if attention_mask is not None and Q == 1 and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         seg_first = _left_padding_offsets(attention_mask, B, n, Hkv)   # a left-padding mask is a per-segment first row
@@ -216,7 +217,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
-        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, seg_first=seg_first)
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first)
         return out.view(B, 1, Hq, D), None, None
     if attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)

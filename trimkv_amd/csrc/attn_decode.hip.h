@@ -177,32 +177,23 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         qv[g] = a.q[((int64_t)seg * G + g) * ROW16 + cc];
         if (ROW16 < 16 && c >= ROW16) qv[g] = make_uint4(0u, 0u, 0u, 0u);
     }
+    // APPEND: the new row is fetched by every wavefront right behind q (the same 512 bytes per segment; unconditional
+    // loads keep the compiler's count of outstanding loads exact) and stored by the wavefront that owns it once q's wait
+    // below has covered these loads too -- no round trip of its own.
     const uint4* knew = nullptr;
     const uint4* vnew = nullptr;
+    uint4 kn = make_uint4(0u, 0u, 0u, 0u), vn = kn;
+    float lbn = 0.0f;
+    int64_t pn = 0;
     if (APPEND) {
         const int b = seg / a.ap.kv_heads, h = seg - b * a.ap.kv_heads;
         const int64_t off = (int64_t)b * a.ap.kv_sb + (int64_t)h * a.ap.kv_sh + ((int64_t)cc << 4);
         knew = (const uint4*)(a.ap.k_new + off);
         vnew = (const uint4*)(a.ap.v_new + off);
-        if (new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and stores it
-            // its loads are issued here, behind q and ahead of the first K/V prefetch, so that the wait below covers them
-            const uint4 kn = *knew, vn = *vnew;
-            float lbn = 0.0f;
-            int64_t pn = 0;
-            if (lane == 0) {
-                lbn = load_as_f32(a.ap.lb_new, (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh, a.ap.lb_dtype);
-                pn = a.ap.pos_new[(int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh];
-            }
-            const int64_t dst = row0 + new_row;
-            if (r == 0 && c < ROW16) {
-                ((uint4*)a.k)[dst * ROW16 + c] = kn;
-                ((uint4*)a.v)[dst * ROW16 + c] = vn;
-            }
-            if (lane == 0) {
-                store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
-                a.ap.pos_slab[dst] = pn;
-            }
-        }
+        kn = *knew;
+        vn = *vnew;
+        lbn = load_as_f32(a.ap.lb_new, (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh, a.ap.lb_dtype);
+        pn = a.ap.pos_new[(int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh];
     }
 
     // which (row-in-tile, head) this lane owns after the transposing reduction
@@ -363,6 +354,17 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         for (int sl = 0; sl < PD; ++sl) load_tile(kp, knew, w0 + sl * TILE_ROWS, ring[sl % RING]);
 #pragma unroll
         for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
+        if (APPEND && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
+            const int64_t dst = row0 + new_row;
+            if (r == 0 && c < ROW16) {
+                ((uint4*)a.k)[dst * ROW16 + c] = kn;
+                ((uint4*)a.v)[dst * ROW16 + c] = vn;
+            }
+            if (lane == 0) {
+                store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
+                a.ap.pos_slab[dst] = pn;
+            }
+        }
         int blk = w0;
 #pragma unroll 1
         for (; blk + AT_BLOCK_ROWS <= w1; blk += AT_BLOCK_ROWS)
@@ -512,13 +514,13 @@ __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a)
 }
 
 static int pick_chunk(int nseg, int max_len) {
-    // One workgroup per segment streams at full rate already with 128 segments (a workgroup keeps 12 tiles in flight).  In a
-    // decode step over 28 layers (nothing of a layer survives in the last-level cache until its next turn) two splits plus
-    // the merge launch took 25.6 + 3.9 us per layer at 128 segments x 2112 rows against 28.6 us for whole segments; a
-    // single layer replayed from the last-level cache had suggested the opposite.  With fewer segments they are cut so
-    // that about 256 workgroups exist, but not below 512 rows each (one full block per wavefront).
+    // A compute unit pulls about 50 GB/s however many wavefronts it runs (measured: 8 workgroups of 4096 rows take 43 us, with
+    // 8 wavefronts each 39 us), so the launch needs all 256 of them: with fewer than 256 segments each is cut so that
+    // about 256 workgroups exist, but not below 512 rows apiece (one full block per wavefront), and a second, tiny launch
+    // merges the pieces.  At 128 segments x 2112 rows (28 layers, append fused into the launch) two pieces per segment plus
+    // the merge make the step 0.815 ms against 0.837 ms for whole segments; from 256 segments on nothing is split.
     const int whole = ((max_len + 63) / 64) * 64;
-    if (nseg >= 128) return whole;
+    if (nseg >= 256) return whole;
     const int nsplit = (256 + nseg - 1) / nseg;
     int chunk = (((max_len + nsplit - 1) / nsplit + 63) / 64) * 64;
     if (chunk < 512) chunk = 512;
