@@ -279,6 +279,12 @@ int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayer
 int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlens, void* stream);
 
 /*
+ * trimkv_build_cu_seqlens_layers -- the same for nlayers layers in one launch (the per-layer rebuilds of
+ * cache_utils.py:466-482, 912-943): seg_lens and cu_seqlens are device tables of nlayers pointers.
+ */
+int trimkv_build_cu_seqlens_layers(const int32_t* const* seg_lens, int32_t* const* cu_seqlens, int nlayers, int nseg, void* stream);
+
+/*
  * trimkv_decode_attn -- single-query GQA attention over every segment's retained K/V:
  *     out[seg*group + g][:] = softmax( q[seg*group + g] . K_seg^T * scale ) V_seg
  * Replaces flash_attn_varlen_func as called at src/trimkv/attn/flash_attn.py:61-71 and 135-145
@@ -337,6 +343,40 @@ int trimkv_append_attend(const void* q, void* out,
                          const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
                          float scale, int max_len_after, int chunk,
                          void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Piece-list launches -- trimkv_decode_attn and trimkv_append_attend for very uneven segment lengths (per-head budgets,
+ * src/trimkv/cache_utils.py:485-536, 789-806), in ONE launch even when segments are cut into pieces.
+ *
+ * `pieces` is a device array of npieces entries of four int32 {segment, piece, pieces_of_segment, first_slot}: the
+ * workgroup of entry i attends rows [first + piece*r, first + (piece+1)*r) of its segment, r = ceil(rows /
+ * pieces_of_segment) computed from the segment's length on the device (so the list stays valid while lengths drift; a
+ * piece may turn out empty), and the pieces of one segment use partial slots first_slot .. first_slot +
+ * pieces_of_segment - 1 (distinct segments: disjoint slot ranges below npieces).  Every segment must appear with all of
+ * its pieces exactly once.  Workgroups are dispatched in list order: sort it so that consecutive entries carry
+ * comparable row counts and long pieces come first.  A segment in one piece writes its output directly; otherwise the
+ * workgroup that finishes last merges the partials inside the same launch (no second kernel).
+ *
+ * workspace: trimkv_decode_attn_pieces_workspace(npieces, group) bytes, 16-byte aligned.  Its first 32 KiB hold one
+ * counter per segment and MUST be zero when the workspace is first used; every launch leaves them zero again.  At most
+ * 8192 segments.  Launches that share a workspace must be ordered (same stream).  Other arguments as in
+ * trimkv_decode_attn / trimkv_append_attend (no chunk, no seg_order: the list replaces both).
+ */
+size_t trimkv_decode_attn_pieces_workspace(int npieces, int group);
+int trimkv_decode_attn_pieces(const void* q, void* out, const void* k_slab, const void* v_slab,
+                              const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_first,
+                              const int32_t* pieces, int npieces,
+                              int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                              int max_len, void* workspace, size_t workspace_bytes, void* stream);
+int trimkv_append_attend_pieces(const void* q, void* out,
+                                void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                const int32_t* pieces, int npieces, int nseg, int kv_heads, int cap, int head_dim, int group,
+                                int kv_dtype, int lb_dtype,
+                                const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
+                                const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                float scale, int max_len_after,
+                                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * trimkv_decode_attn_static -- trimkv_decode_attn for callers that cannot allocate device memory (code under HIP

@@ -304,7 +304,9 @@ def test_ragged_decode_attention_matches_fp32_oracle(G):
     # the same kernel on PACKED rows + cu_seqlens_k, as a caller holding the reference's layout would pass them
     kw2 = {"head_lens": d.ref.head_lens[0].to(DEV), "cu_seqlens_k": d.ref.cu_seqlens_k[0].to(DEV), "batch_size": B, "num_kv_heads": H}
     out2, _, _ = attn(_Mod(), q.to(DEV), d.ref.key_cache[0].to(DEV), d.ref.value_cache[0].to(DEV), None, flash_attn_kwargs=kw2)
-    assert torch.equal(out2, out)
+    # the cache's own launch goes over its piece list, packed rows over the grid of (segment, split): the rows are cut at
+    # other places, so the two agree to rounding, not bit for bit
+    assert (out2.float() - out.float()).abs().max() < 4e-3 and attn_close(out2, want)[0]
 
 
 def test_single_key_and_equal_keys_closed_forms():

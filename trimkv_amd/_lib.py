@@ -48,10 +48,15 @@ SIGNATURES = {
     "trimkv_evict_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _i64, _p, _i, _i, _i, _i, _p, _sz, _p]),
     "trimkv_compact_threshold_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p, _i64, _i, _i, _i, _p, _sz, _p]),
     "trimkv_build_cu_seqlens": (_i, [_p, _i, _p, _p]),
+    "trimkv_build_cu_seqlens_layers": (_i, [_p, _p, _i, _i, _p]),
     "trimkv_decode_attn_workspace": (_sz, [_i, _i, _i, _i, _i]),
     "trimkv_decode_attn": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p]),
     "trimkv_append_attend": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64,
                                   _p, _i64, _i64, _p, _i64, _i64, _f, _i, _i, _p, _sz, _p]),
+    "trimkv_decode_attn_pieces_workspace": (_sz, [_i, _i]),
+    "trimkv_decode_attn_pieces": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p, _sz, _p]),
+    "trimkv_append_attend_pieces": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64,
+                                         _p, _i64, _i64, _p, _i64, _i64, _f, _i, _p, _sz, _p]),
     "trimkv_decode_attn_static": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "trimkv_prefill_attn": (_i, [_p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
 }

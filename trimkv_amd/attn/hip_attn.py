@@ -49,6 +49,20 @@ def _group_slice(group: int) -> int:
     return max(g for g in range(1, _MAX_GROUP + 1) if group % g == 0)
 
 
+_WS_ZERO: Dict[Tuple[str, int], torch.Tensor] = {}
+
+
+def _workspace_zeroed(device, nbytes: int, stream: int) -> torch.Tensor:
+    """Scratch of the piece-list launches: its counter header has to be zero on first use and is left zero by every launch,
+    so these buffers are allocated zero-filled and never shared with the other launches' scratch."""
+    key = (device, stream)
+    ws = _WS_ZERO.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        _WS_ZERO[key] = ws
+    return ws
+
+
 def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     """Split-K scratch, one buffer per (device, stream): launches that share a buffer must be ordered."""
     if nbytes <= 0:
@@ -91,7 +105,7 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
 
 
 def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: int = 0,
-                  seg_order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  seg_order: Optional[torch.Tensor] = None, pieces=None) -> torch.Tensor:
     """The deferred one-token append of ``slab`` (a cache layer whose ``update`` ran with ``fuse_decode_append``) and the
     attention over the layer including that token, in one launch: ``trimkv_append_attend``.  ``query`` [nseg*group, D]
     contiguous -> [nseg*group, D].  Clears the pending append."""
@@ -99,6 +113,16 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
     nseg, d = slab.B * slab.H, slab.D
     out = torch.empty_like(query)
     st = _lib.current_stream(query.device)
+    if pieces is not None:   # ragged lengths: one launch over the (segment, piece) list, merged inside it
+        plist, npieces = pieces
+        ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(npieces, group), st)
+        rc = lib.trimkv_append_attend_pieces(query.data_ptr(), out.data_ptr(), *slab.ptrs, plist.data_ptr(), npieces,
+                                             nseg, slab.H, slab.cap, d, group, *slab.codes, *slab.pending[0],
+                                             scale, slab.max_len, ws.data_ptr(), ws.numel(), st)
+        if rc:
+            _lib.check(rc, "trimkv_append_attend_pieces")
+        slab.pending = None
+        return out
     ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, slab.max_len, chunk)
     ws = _workspace(query.device, ws_bytes, st) if ws_bytes else None
     # slab.pending[0] = the new row's addresses and strides, in the order of the entry point's parameters
@@ -264,7 +288,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        out = append_attend(slab, q2, G, D ** -0.5, chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"))
+        out = append_attend(slab, q2, G, D ** -0.5, chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"), pieces=kw.get("pieces"))
         return out.view(B, 1, Hq, D), None, None
     seg_start = kw.get("seg_start")
     if seg_start is None:  # packed rows, as the reference stores them
@@ -281,6 +305,17 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         q2 = query.reshape(B * Hq, D)  # [B,Hq,1,D]: row seg*G+g is query head h*G+g of batch b
         if not q2.is_contiguous():
             q2 = q2.contiguous()
+        pieces = kw.get("pieces")
+        if pieces is not None and G <= _MAX_GROUP:
+            lib = _lib.load()
+            out = torch.empty_like(q2)
+            st = _lib.current_stream(q2.device)
+            ws = _workspace_zeroed(q2.device, lib.trimkv_decode_attn_pieces_workspace(pieces[1], G), st)
+            rc = lib.trimkv_decode_attn_pieces(q2.data_ptr(), out.data_ptr(), key.data_ptr(), value.data_ptr(), head_lens.data_ptr(),
+                                               seg_start.data_ptr(), None, pieces[0].data_ptr(), pieces[1], nseg, cap, D, G,
+                                               _lib.dtype_code(q2.dtype), D ** -0.5, max(1, max_len), ws.data_ptr(), ws.numel(), st)
+            _lib.check(rc, "trimkv_decode_attn_pieces")
+            return out.view(B, 1, Hq, D), None, None
         out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5,
                                chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"))
         return out.view(B, 1, Hq, D), None, None

@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libtrimkv_hip.so")
-SOURCES = ["api.hip", "append.hip", "evict.hip", "attn_decode.hip", "attn_decode_append.hip", "attn_prefill.hip", "gate.hip"]
+SOURCES = ["api.hip", "append.hip", "evict.hip", "attn_decode.hip", "attn_decode_append.hip", "attn_decode_pieces.hip", "attn_decode_append_pieces.hip", "attn_prefill.hip", "gate.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,
@@ -42,7 +42,7 @@ def build(verbose: bool = True) -> str:
         src, obj = pair
         return _run([hipcc] + HIPCC_FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj])
 
-    with ThreadPoolExecutor(max_workers=min(4, len(srcs))) as ex:
+    with ThreadPoolExecutor(max_workers=min(os.cpu_count() or 4, 8, len(srcs))) as ex:
         for src, out in zip(srcs, ex.map(compile_one, zip(srcs, objs))):
             if verbose and out.strip():
                 print("[%s]\n%s" % (src, out))

@@ -90,7 +90,7 @@ class _Slab:
     """Device storage of one layer."""
 
     __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order",
-                 "pending", "codes", "total")
+                 "pending", "codes", "total", "pieces", "pieces_total", "pieces_age")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -106,6 +106,8 @@ class _Slab:
         self.total = 0  # sum of lens (kept by the ragged caches, which size their split-K chunk from it)
         self.order = None  # ragged caches: segments by decreasing length/budget (dispatch order of the attention launch)
         self.pending = None  # a one-token append that the next attention call will carry out (see _SlabBacked._defer)
+        self.pieces = None   # ragged caches: (device piece list, number of pieces) of the decode-attention launch
+        self.pieces_total, self.pieces_age = 0, 0
         self._refresh_views()
 
     def _refresh_views(self) -> None:
@@ -325,7 +327,7 @@ class _SlabBacked(_CacheBase):
         for i, s in enumerate(slabs):
             arr[i] = (s.ptrs[0], s.ptrs[1], s.ptrs[2], s.ptrs[3], s.ptrs[4], 0, s.cap, 0)
         tables = {"slabs": torch.from_numpy(arr.view(np.uint8)).to(dev)}
-        for name, idx in (("k", 0), ("lb", 2), ("pos", 3), ("len", 4)):
+        for name, idx in (("k", 0), ("lb", 2), ("pos", 3), ("len", 4)) + ((("cu", 5),) if slabs[0].cu is not None else ()):
             tables[name] = torch.tensor([s.ptrs[idx] for s in slabs], dtype=torch.int64).to(dev)
         self._table_cache[key] = ([s.ptrs for s in slabs], [s.cap for s in slabs], tables)
         return tables
@@ -597,6 +599,7 @@ class TrimKVCache(_SlabBacked):
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
                 new.lens, new.max_len, new.order = slab.lens[lo:hi].copy(), slab.max_len, None
                 new.pending, new.total = None, int(new.lens.sum())
+                new.pieces, new.pieces_total, new.pieces_age = None, 0, 0
                 new._refresh_views()
                 part._slabs.append(new)
             out.append(part)
@@ -632,6 +635,7 @@ class TrimKVCache(_SlabBacked):
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
             c.lens, c.max_len, c.order = slab.lens.copy(), slab.max_len, None
             c.pending, c.total = None, slab.total
+            c.pieces, c.pieces_total, c.pieces_age = None, 0, 0
             c._refresh_views()
             new._slabs.append(c)
         return new
@@ -677,6 +681,7 @@ class _RaggedCache(_SlabBacked):
         # update() normally hands the attention call the slab rows plus ``seg_start`` (no copy).  With this flag, or with
         # ``cache_kwargs={"packed": True}`` on a call, it returns the reference's packed ``[sum(n), D]`` tensors instead.
         self.return_packed = False
+        self.attention_pieces = 400   # split-K tuning knob: about this many pieces per decode-attention launch
 
     # plain attributes in the reference; a property here because newer HF Cache classes define a
     # read-only `batch_size` of their own
@@ -736,19 +741,48 @@ class _RaggedCache(_SlabBacked):
         if packed:
             self._flush(slab)
             return self._packed(slab)
-        # split-K chunk for ragged lengths: about 384 pieces over the rows actually cached (the library's own default
-        # assumes every segment is max_len long); measured on 256 lognormal segments (128..8256 rows, 410 k rows): 1088-row pieces 52 us, 832 54.7, 1664 53 -- pieces
-        # long enough to stream, short enough that no compute unit ends up with much more than its share
-        chunk = max(512, ((slab.total // 384 + 63) // 64) * 64)
+        # grid-split fallback (callers that ignore "pieces"): rows per piece for about attention_pieces pieces
+        chunk = max(512, ((slab.total // self.attention_pieces + 63) // 64) * 64)
         kw = {"head_lens": slab.seg_len, "cu_seqlens_k": slab.cu,
               "seg_start": self._seg_start(slab), "seg_cap": slab.cap, "max_len": slab.max_len, "chunk": chunk,
-              "seg_order": slab.order}
+              "seg_order": slab.order, "pieces": self._piece_list(slab)}
         if slab.pending is not None:
             # head_lens / cu_seqlens_k still hold the values before this token: the attention call that receives this
             # dictionary appends the row and advances them in the same launch
             kw["pending_append"] = (self, slab)
         flat = (slab.k.view(-1, slab.D), slab.v.view(-1, slab.D), slab.lb.view(-1, 1), slab.pos.view(-1, 1))
         return flat, kw
+
+    def _piece_list(self, slab: _Slab):
+        """The decode-attention launch of a ragged layer as a list of (segment, piece) workgroups, see
+        ``trimkv_decode_attn_pieces``: every segment is cut into ``round(length / target)`` pieces with ``target`` = rows
+        cached / ``attention_pieces``, and the pieces are dispatched longest first, the second 256 in rising order so that
+        the two workgroups a compute unit starts with add up to about the same number of rows everywhere.  The kernel
+        derives row ranges from the lengths on the device, so the list only has to be roughly right: it is rebuilt when the
+        rows cached have drifted by 4 %, after an eviction that changed them wholesale, or after 64 steps."""
+        slab.pieces_age += 1
+        if (slab.pieces is not None and slab.pieces_age < 64 and abs(slab.total - slab.pieces_total) * 25 <= slab.pieces_total):
+            return slab.pieces
+        lens = slab.lens
+        nseg = lens.size
+        if nseg > 8192:
+            slab.pieces = None
+            return None
+        target = max(256.0, float(max(1, slab.total)) / self.attention_pieces)
+        nsp = np.maximum(1, np.rint(lens / target)).astype(np.int64)
+        slot0 = np.cumsum(nsp) - nsp
+        seg_ids = np.repeat(np.arange(nseg, dtype=np.int64), nsp)
+        which = np.arange(int(nsp.sum()), dtype=np.int64) - np.repeat(slot0, nsp)
+        rows = np.repeat(-(-lens // nsp), nsp)
+        order = np.argsort(-rows, kind="stable")
+        if order.size > 256:
+            # workgroups i and i + 256 start on the same compute unit: measured 1.66 ms per step with this pairing against
+            # 1.79 ms for a plain longest-first list (256 lognormal segments, 36 layers)
+            order[256:512] = order[256:512][::-1].copy()
+        arr = np.stack([seg_ids, which, np.repeat(nsp, nsp), np.repeat(slot0, nsp)], axis=1)[order].astype(np.int32)
+        slab.pieces = (torch.from_numpy(np.ascontiguousarray(arr)).to(slab.k.device), int(arr.shape[0]))
+        slab.pieces_total, slab.pieces_age = slab.total, 0
+        return slab.pieces
 
     def _seg_start(self, slab: _Slab) -> torch.Tensor:
         key = ("seg_start", slab.nseg, slab.cap, str(slab.k.device))
@@ -896,16 +930,23 @@ class _RaggedCache(_SlabBacked):
         """After an eviction: rebuild cu_seqlens on the device and bring the new lengths to the
         host -- the one synchronisation an eviction costs (the reference pays O(B*L*Hkv))."""
         lib = _lib.load()
-        for l in layers:
-            slab = self._slabs[l]
-            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
-            _lib.check(rc, "trimkv_build_cu_seqlens")
+        if len(layers) > 1 and self._layers_alike(layers):
+            t = self._device_tables(layers)
+            s0 = self._slabs[layers[0]]
+            rc = lib.trimkv_build_cu_seqlens_layers(t["len"].data_ptr(), t["cu"].data_ptr(), len(layers), s0.nseg, _lib.current_stream(s0.k.device))
+            _lib.check(rc, "trimkv_build_cu_seqlens_layers")
+        else:
+            for l in layers:
+                slab = self._slabs[l]
+                rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
+                _lib.check(rc, "trimkv_build_cu_seqlens")
         if layers:
             lens = torch.stack([self._slabs[l].seg_len for l in layers]).cpu().numpy().astype(np.int64)
             for i, l in enumerate(layers):
                 self._slabs[l].lens = lens[i].copy()
                 self._slabs[l].max_len = int(lens[i].max())
                 self._slabs[l].total = int(lens[i].sum())
+                self._slabs[l].pieces = None
                 if getattr(self, "_budgets_host", None) is None:
                     self._set_dispatch_order(self._slabs[l], lens[i])
 
@@ -936,54 +977,66 @@ class _RaggedCache(_SlabBacked):
         (cache_utils.py:508-521).  The trigger is evaluated on the host mirror of the lengths and
         again per segment on the device; no host synchronisation happens here."""
         self._flush_all()
-        layers = [l for l in range(len(self._slabs)) if self._slabs[l] is not None] if layers is None else layers
+        every = [l for l in range(len(self._slabs)) if self._slabs[l] is not None]
+        layers = every if layers is None else list(layers)
+        if not layers:
+            return
         lib = _lib.load()
         code = self._strategy_code(strategy)
-        due = []
-        for l in layers:
-            slab = self._slabs[l]
-            kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[l]
-            hit = (slab.lens > kh) & (slab.lens >= kh + buffer_size)
-            if hit.any():
-                due.append((l, kh, hit))
-        if not due:
+        # the trigger for all listed layers at once, on the host mirrors
+        lens_all = np.stack([self._slabs[l].lens for l in layers])
+        kh_all = self._budgets_host[None, :] if self._budgets_host.ndim == 1 else self._budgets_host[layers]
+        hit_all = (lens_all > kh_all) & (lens_all >= kh_all + buffer_size)
+        due_rows = np.flatnonzero(hit_all.any(axis=1))
+        if due_rows.size == 0:
             return
-        every = [l for l in range(len(self._slabs)) if self._slabs[l] is not None]
-        if len(due) > 1 and list(layers) == every and self._layers_alike(every):
+        due = [layers[i] for i in due_rows]
+        dev = self._slabs[layers[0]].k.device
+        q_idx = self.get_seq_length() + 1
+        if len(due) > 1 and layers == every and self._layers_alike(every):
             # One launch over every layer, whichever of them are due: the kernel re-checks the trigger per segment, so the
             # launch -- address table and budgets resident on the device -- is the same at every step and nothing is uploaded.
-            key = ("all", str(self._slabs[every[0]].k.device))
+            key = ("all", str(dev))
             keep = self._budgets_dev.get(key)
             if keep is None:
-                kh_all = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[every]
-                keep = torch.from_numpy(np.ascontiguousarray(kh_all, dtype=np.int32)).to(self._slabs[every[0]].k.device)
+                kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[every]
+                keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(dev)
                 self._budgets_dev[key] = keep
-            self._evict_layers(every, 0, keep, buffer_size, code, _lib.ROUND_NATIVE, 0, self.get_seq_length() + 1)
-        elif len(due) > 1 and self._layers_alike([l for l, _, _ in due]):   # a subset of the layers: its budgets are uploaded
-            self._evict_layers([l for l, _, _ in due], 0, np.stack([kh for _, kh, _ in due]), buffer_size, code, _lib.ROUND_NATIVE, 0,
-                               self.get_seq_length() + 1)
+            self._evict_layers(every, 0, keep, buffer_size, code, _lib.ROUND_NATIVE, 0, q_idx)
+            t = self._device_tables(every)
+            rc = lib.trimkv_build_cu_seqlens_layers(t["len"].data_ptr(), t["cu"].data_ptr(), len(every), self._slabs[every[0]].nseg,
+                                                    _lib.current_stream(dev))
+            _lib.check(rc, "trimkv_build_cu_seqlens_layers")
         else:
-            for l, kh, _ in due:
+            if len(due) > 1 and self._layers_alike(due):   # a subset of the layers: its budgets are uploaded
+                kh = np.broadcast_to(kh_all, lens_all.shape)[due_rows]
+                self._evict_layers(due, 0, np.ascontiguousarray(kh), buffer_size, code, _lib.ROUND_NATIVE, 0, q_idx)
+            else:
+                for l in due:
+                    slab = self._slabs[l]
+                    key = (l if self._budgets_host.ndim == 2 else -1, str(slab.k.device))
+                    keep = self._budgets_dev.get(key)
+                    if keep is None:
+                        kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[l]
+                        keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(slab.k.device)
+                        self._budgets_dev[key] = keep
+                    ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
+                    rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
+                                          slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
+                                          0, keep.data_ptr(), buffer_size, q_idx, code, _lib.ROUND_NATIVE,
+                                          0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(),
+                                          _lib.current_stream(slab.k.device))
+                    _lib.check(rc, "trimkv_evict")
+            for l in due:
                 slab = self._slabs[l]
-                key = (l if self._budgets_host.ndim == 2 else -1, str(slab.k.device))
-                keep = self._budgets_dev.get(key)
-                if keep is None:
-                    keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(slab.k.device)
-                    self._budgets_dev[key] = keep
-                ws = self._workspace(lib.trimkv_evict_workspace(slab.nseg, slab.max_len), slab.k.device)
-                rc = lib.trimkv_evict(slab.k.data_ptr(), slab.v.data_ptr(), slab.lb.data_ptr(), slab.pos.data_ptr(), slab.seg_len.data_ptr(),
-                                      slab.nseg, slab.cap, slab.D, _lib.dtype_code(slab.k.dtype), _lib.dtype_code(slab.lb.dtype),
-                                      0, keep.data_ptr(), buffer_size, self.get_seq_length() + 1, code, _lib.ROUND_NATIVE,
-                                      0, slab.max_len, None, 0, _lib.ptr(ws), 0 if ws is None else ws.numel(),
-                                      _lib.current_stream(slab.k.device))
-                _lib.check(rc, "trimkv_evict")
-        for l, kh, hit in due:
-            slab = self._slabs[l]
-            rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
-            _lib.check(rc, "trimkv_build_cu_seqlens")
-            slab.lens = np.where(hit, kh, slab.lens)
-            slab.max_len = int(slab.lens.max())
-            slab.total = int(slab.lens.sum())
+                rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
+                _lib.check(rc, "trimkv_build_cu_seqlens")
+        # host mirrors of the lengths, for all due layers at once
+        new_all = np.where(hit_all, np.broadcast_to(kh_all, lens_all.shape), lens_all)
+        maxes, sums = new_all.max(axis=1), new_all.sum(axis=1)
+        for i in due_rows:
+            slab = self._slabs[layers[i]]
+            slab.lens, slab.max_len, slab.total = new_all[i], int(maxes[i]), int(sums[i])
 
     def segment_positions(self):
         """Per layer, per segment: retained absolute positions (host tensors)."""

@@ -120,7 +120,18 @@ struct AttnArgs {
     float scale_log2;
     float* ws_o; float* ws_ml;
     AppendPart ap;   // read by APPEND kernels only
+    // piece-list launches (decode_attn_pieces_kernel): one workgroup per entry {segment, piece, pieces of the segment,
+    // first partial slot of the segment}; counters[seg] counts the finished pieces of a segment (zero between launches)
+    const int4* pieces; uint32_t* counters; int npieces;
 };
+
+// Partials that another workgroup of the same launch will read.  Workgroups of one launch run on different XCDs, whose L2
+// caches are not coherent with each other, so these accesses are device-scope atomics (relaxed): the stores write through
+// to memory and the loads do not hit a stale line.  Ordering between them and the per-segment counter is by completion:
+// the writer waits for its stores (s_waitcnt through a workgroup-scope release fence) before it bumps the counter, and the
+// reader issues its loads after the bump has returned.  No L2 write-back or invalidate is involved.
+__device__ __forceinline__ void store_shared_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_shared_partial(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
 // Length of segment `seg` as the launch sees it.  APPEND: the stored length is the one before this step's token; the token
 // lands in row n_old (returned through *new_row) unless the slab is full, in which case nothing is appended (-1).
@@ -145,7 +156,8 @@ __device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new
 // re-read the row's last piece and hold q = 0, so they add nothing to the scores; what they accumulate is not stored.
 // APPEND: row `new_row` of the segment (-1: none) is this step's token.  It is read from a.ap.k_new / v_new wherever the
 // stream reaches it, and the wavefront that owns it writes it into the slabs (K, V, log beta, position).
-template <int G, int ROW16, bool F16, bool APPEND>
+// COHERENT: the partials are read by another workgroup of this same launch (see store_shared_partial).
+template <int G, int ROW16, bool F16, bool APPEND, bool COHERENT = false>
 __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base, int new_row) {
     constexpr int D_REAL = ROW16 * 8;
     using C = AttnCfg<G>;
@@ -428,8 +440,13 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = to_kv_bits<F16>(y);
         } else {
             const int64_t slot = slot_base * G + g;
-            a.ws_o[slot * AT_D + d] = acc;
-            if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
+            if (COHERENT) {
+                store_shared_partial(&a.ws_o[slot * AT_D + d], acc);
+                if (d == 0) { store_shared_partial(&a.ws_ml[slot * 2], mx); store_shared_partial(&a.ws_ml[slot * 2 + 1], lsum); }
+            } else {
+                a.ws_o[slot * AT_D + d] = acc;
+                if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
+            }
         }
     }
 }
@@ -460,6 +477,75 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     const int rps = (live + nsp - 1) / nsp;
     const int t0 = first + split * rps, t1 = min(n, t0 + rps);
     attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split, new_row);
+}
+
+// Piece-list launch: one workgroup per entry of a.pieces, in the order of the list (the caller sorts it so that every
+// compute unit receives about the same number of rows), and no second launch: a segment cut into several pieces is
+// merged by whichever of its workgroups finishes last.  Every workgroup of the grid works on a piece, so once a segment's
+// counter is full nobody will read its length again and the merging workgroup may advance it (APPEND).
+template <int G, int ROW16, bool F16, bool APPEND>
+__global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_pieces_kernel(AttnArgs a) {
+    __shared__ int last_of_segment;
+    const int4 e = a.pieces[blockIdx.x];
+    const int seg = min(max(e.x, 0), a.nseg - 1), nsp = max(e.z, 1), piece = min(max(e.y, 0), nsp - 1);
+    if (nsp > 1 && (e.w < 0 || e.w + nsp > a.npieces)) return;   // a list whose partial slots do not fit the workspace: touch nothing
+    int new_row, first;
+    const int n = segment_rows<APPEND>(a, seg, &new_row, &first);
+    const int live = n - first;
+    const int rps = (live + nsp - 1) / nsp;
+    const int t0 = min(n, first + piece * rps), t1 = min(n, t0 + rps);   // may be empty: the piece then contributes nothing
+    if (nsp == 1) {
+        attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, true, 0, new_row);
+        return;
+    }
+    const int64_t slot0 = e.w;
+    attend_rows<G, ROW16, F16, APPEND, true>(a, seg, t0, t1, false, slot0 + piece, new_row);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every thread: its partial stores have completed
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const uint32_t done = __hip_atomic_fetch_add(&a.counters[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        last_of_segment = done + 1u == (uint32_t)nsp;
+    }
+    __syncthreads();
+    if (!last_of_segment) return;
+    for (int i = threadIdx.x; i < G * AT_D; i += AT_THREADS) {
+        const int g = i / AT_D, d = i - g * AT_D;
+        const int64_t base = slot0 * G + g;
+        float mx = AT_NEG, acc = 0.0f, lsum = 0.0f;
+        for (int sp0 = 0; sp0 < nsp; sp0 += 8) {   // eight pieces' loads in flight at a time
+            float m8[8], l8[8], o8[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int64_t slot = base + (int64_t)min(sp0 + u, nsp - 1) * G;
+                m8[u] = load_shared_partial(&a.ws_ml[slot * 2]);
+                l8[u] = load_shared_partial(&a.ws_ml[slot * 2 + 1]);
+                o8[u] = load_shared_partial(&a.ws_o[slot * AT_D + d]);
+            }
+            float bm = AT_NEG;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) bm = fmaxf(bm, sp0 + u < nsp ? m8[u] : AT_NEG);
+            const float m_new = fmaxf(mx, bm);
+            const float rescale = __builtin_amdgcn_exp2f(mx - m_new);
+            acc *= rescale;
+            lsum *= rescale;
+            mx = m_new;
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float f = sp0 + u < nsp ? __builtin_amdgcn_exp2f(m8[u] - mx) : 0.0f;
+                acc += f * o8[u];
+                lsum += f * l8[u];
+            }
+        }
+        const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+        if (d < ROW16 * 8) ((uint16_t*)a.out)[((int64_t)seg * G + g) * (ROW16 * 8) + d] = to_kv_bits<F16>(y);
+    }
+    if (threadIdx.x == 0) {
+        __hip_atomic_store(&a.counters[seg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // zero again for the next launch
+        if (APPEND && new_row >= 0) {
+            a.ap.seg_len[seg] = new_row + 1;
+            if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;
+        }
+    }
 }
 
 // Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
@@ -546,6 +632,61 @@ static void launch_attn(const AttnArgs& a, int head_dim, int dtype, hipStream_t 
     else launch_attn_dtype<G, false, APPEND>(a, head_dim, st);
 }
 
+template <int G, bool APPEND>
+static void launch_attn_pieces(const AttnArgs& a, int npieces, int head_dim, int dtype, hipStream_t st) {
+    const dim3 grid(npieces), block(AT_THREADS);
+    if (dtype == TRIMKV_F16) {
+        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, true, APPEND>), grid, block, 0, st, a);
+        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, true, APPEND>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, true, APPEND>), grid, block, 0, st, a);
+    } else {
+        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, false, APPEND>), grid, block, 0, st, a);
+        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, false, APPEND>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, false, APPEND>), grid, block, 0, st, a);
+    }
+}
+
+template <bool APPEND>
+static void launch_attn_pieces_group(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st) {
+    switch (group) {
+        case 1: launch_attn_pieces<1, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 2: launch_attn_pieces<2, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 3: launch_attn_pieces<3, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 4: launch_attn_pieces<4, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 5: launch_attn_pieces<5, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 6: launch_attn_pieces<6, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 7: launch_attn_pieces<7, APPEND>(a, npieces, head_dim, dtype, st); break;
+        default: launch_attn_pieces<8, APPEND>(a, npieces, head_dim, dtype, st); break;
+    }
+}
+
+// Workspace of a piece-list launch: a fixed header of per-segment counters (zero before the first use, left zero by
+// every launch), then one partial slot per piece.
+constexpr size_t AT_PIECE_COUNTER_BYTES = 32768;   // 8192 segments
+constexpr int AT_PIECE_MAX_SEGMENTS = (int)(AT_PIECE_COUNTER_BYTES / sizeof(uint32_t));
+static size_t pieces_workspace_bytes(int npieces, int group) {
+    return AT_PIECE_COUNTER_BYTES + (size_t)npieces * group * (AT_D + 2) * sizeof(float);
+}
+
+// Completes `a` (already through prepare_attn with chunk covering max_len, i.e. direct) for a piece-list launch.
+static int prepare_pieces(const char* fn, AttnArgs& a, const int32_t* pieces, int npieces, int nseg, int group,
+                          void* workspace, size_t workspace_bytes) {
+    if (!pieces) return fail(TRIMKV_ERR_NULL, "%s: null piece list", fn);
+    if (npieces <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: npieces=%d", fn, npieces);
+    if ((uintptr_t)pieces & 15) return fail(TRIMKV_ERR_SHAPE, "%s: the piece list must be 16-byte aligned", fn);
+    if (nseg > AT_PIECE_MAX_SEGMENTS) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: at most %d segments per piece-list launch (got %d)", fn, AT_PIECE_MAX_SEGMENTS, nseg);
+    const size_t need = pieces_workspace_bytes(npieces, group);
+    if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+    if ((uintptr_t)workspace & 15) return fail(TRIMKV_ERR_SHAPE, "%s: workspace must be 16-byte aligned", fn);
+    a.pieces = (const int4*)pieces;
+    a.npieces = npieces;
+    a.counters = (uint32_t*)workspace;
+    a.ws_o = (float*)((char*)workspace + AT_PIECE_COUNTER_BYTES);
+    a.ws_ml = a.ws_o + (size_t)npieces * group * AT_D;
+    a.direct = 0;
+    return TRIMKV_OK;
+}
+
 // group = 1..8 -> the matching instantiation
 template <bool APPEND>
 static void launch_attn_group(const AttnArgs& a, int group, int head_dim, int dtype, hipStream_t st) {
@@ -583,6 +724,7 @@ static int prepare_attn(const char* fn, AttnArgs& a, const void* q, void* out, c
     a.scale_log2 = scale * 1.4426950408889634f;
     a.ws_o = nullptr; a.ws_ml = nullptr;
     a.ap = AppendPart{};
+    a.pieces = nullptr; a.counters = nullptr; a.npieces = 0;
     if (!a.direct) {
         const size_t need = (size_t)nseg * a.nsplit * group * (AT_D + 2) * sizeof(float);   // partial rows are padded to 128 features
         if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);

@@ -7,6 +7,7 @@
 // The kernels are the decode-attention kernels instantiated with APPEND = true: the stream takes the new row from the
 // caller's tensor wherever it reaches it, and the wavefront that owns that row writes it into the slabs.
 #include "attn_decode.hip.h"
+#include "attn_decode_append.hip.h"
 
 using namespace trimkv;
 
@@ -20,20 +21,15 @@ extern "C" int trimkv_append_attend(const void* q, void* out,
                                     float scale, int max_len_after, int chunk,
                                     void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_append_attend";
-    if (!lb_slab || !pos_slab || !seg_len || !k_new || !v_new || !lb_new || !pos_new) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
-    if (dtype_bytes(lb_dtype) == 0) return fail(TRIMKV_ERR_DTYPE, "%s: lb_dtype must be f32/bf16/f16 (got %d)", fn, lb_dtype);
-    if (kv_heads <= 0 || nseg <= 0 || nseg % kv_heads) return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nseg=%d kv_heads=%d", fn, nseg, kv_heads);
-    if (((kv_stride_b * 2) | (kv_stride_h * 2)) & 15 || ((uintptr_t)k_new & 15) || ((uintptr_t)v_new & 15))
-        return fail(TRIMKV_ERR_SHAPE, "%s: new K/V rows must be 16-byte aligned (strides %lld,%lld elements)", fn, (long long)kv_stride_b, (long long)kv_stride_h);
-    AttnArgs a;
-    const int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, seg_order, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
-                                max_len_after, chunk, workspace, workspace_bytes);
+    int rc = check_append_args(fn, lb_slab, pos_slab, seg_len, k_new, v_new, lb_new, pos_new, nseg, kv_heads, lb_dtype, kv_stride_b, kv_stride_h);
     if (rc) return rc;
-    a.ap.k_new = (const char*)k_new; a.ap.v_new = (const char*)v_new; a.ap.kv_sb = kv_stride_b * 2; a.ap.kv_sh = kv_stride_h * 2;
-    a.ap.lb_new = lb_new; a.ap.lb_sb = lb_stride_b; a.ap.lb_sh = lb_stride_h;
-    a.ap.pos_new = pos_new; a.ap.pos_sb = pos_stride_b; a.ap.pos_sh = pos_stride_h;
-    a.ap.lb_slab = lb_slab; a.ap.pos_slab = pos_slab; a.ap.seg_len = seg_len; a.ap.cu = cu_seqlens;
-    a.ap.kv_heads = kv_heads; a.ap.lb_dtype = lb_dtype;
+    AttnArgs a;
+    rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, seg_order, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
+                      max_len_after, chunk, workspace, workspace_bytes);
+    if (rc) return rc;
+    fill_append_part(fn, a, lb_slab, pos_slab, seg_len, cu_seqlens, nseg, kv_heads, lb_dtype, k_new, v_new, kv_stride_b, kv_stride_h,
+                     lb_new, lb_stride_b, lb_stride_h, pos_new, pos_stride_b, pos_stride_h);
     launch_attn_group<true>(a, group, head_dim, kv_dtype, (hipStream_t)stream);
     return launch_status(fn);
 }
+

@@ -672,8 +672,10 @@ __global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
     if (i < n) p[i] = v;
 }
 
-__global__ void cu_seqlens_kernel(const int32_t* seg_len, int nseg, int32_t* cu) {
+// blockIdx.x selects a layer when the pointers come from device tables (seg_lens / cus non-null).
+__global__ void cu_seqlens_kernel(const int32_t* seg_len, int nseg, int32_t* cu, const int32_t* const* seg_lens, int32_t* const* cus) {
     __shared__ uint32_t scratch[1024 / 64 + 1];
+    if (seg_lens) { seg_len = seg_lens[blockIdx.x]; cu = cus[blockIdx.x]; }
     int32_t running = 0;
     if (threadIdx.x == 0) cu[0] = 0;
     for (int base = 0; base < nseg; base += 1024) {
@@ -930,6 +932,15 @@ extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const in
 extern "C" int trimkv_build_cu_seqlens(const int32_t* seg_len, int nseg, int32_t* cu_seqlens, void* stream) {
     if (!seg_len || !cu_seqlens) return fail(TRIMKV_ERR_NULL, "trimkv_build_cu_seqlens: null pointer argument");
     if (nseg <= 0) return fail(TRIMKV_ERR_SHAPE, "trimkv_build_cu_seqlens: nseg=%d", nseg);
-    hipLaunchKernelGGL(cu_seqlens_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seg_len, nseg, cu_seqlens);
+    hipLaunchKernelGGL(cu_seqlens_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seg_len, nseg, cu_seqlens,
+                       (const int32_t* const*)nullptr, (int32_t* const*)nullptr);
     return launch_status("trimkv_build_cu_seqlens");
+}
+
+extern "C" int trimkv_build_cu_seqlens_layers(const int32_t* const* seg_lens, int32_t* const* cu_seqlens, int nlayers, int nseg, void* stream) {
+    if (!seg_lens || !cu_seqlens) return fail(TRIMKV_ERR_NULL, "trimkv_build_cu_seqlens_layers: null pointer argument");
+    if (nseg <= 0 || nlayers <= 0 || nlayers > 65535) return fail(TRIMKV_ERR_SHAPE, "trimkv_build_cu_seqlens_layers: nlayers=%d nseg=%d", nlayers, nseg);
+    hipLaunchKernelGGL(cu_seqlens_kernel, dim3(nlayers), dim3(1024), 0, (hipStream_t)stream, (const int32_t*)nullptr, nseg, (int32_t*)nullptr,
+                       seg_lens, cu_seqlens);
+    return launch_status("trimkv_build_cu_seqlens_layers");
 }
