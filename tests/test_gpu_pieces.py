@@ -139,6 +139,40 @@ def test_append_attend_pieces_equals_append_then_attend():
         assert not ws_b[:32768].any()
 
 
+def test_alternating_layouts_reproduce_their_first_result():
+    """Three different piece lists take turns on ONE workspace, with the host synchronising between launches (every launch
+    then starts on an idle GPU and the pieces of a segment finish almost together).  Whatever a launch finds in the partial
+    slots was written by another layout, so a merge that read a slot before its writer's stores had landed would give
+    another result than that layout's first launch: every launch must reproduce it bit for bit."""
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    rng = np.random.default_rng(0)
+    nseg, cap, G, D = 256, 8320, 4, 128
+    lens = (np.clip(np.round(np.exp(rng.normal(np.log(1024), 1.0, size=nseg))), 64, 8192) + 64).astype(np.int32)
+    gen = torch.Generator().manual_seed(0)
+    k = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    v = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    LEN = torch.from_numpy(lens).to(DEV)
+    st = L.current_stream(torch.device(DEV))
+    layouts = [_piece_list(lens, t, rng, "shuffled" if i % 2 else "desc") for i, t in enumerate((300.0, 640.0, 1000.0))]
+    ws = torch.zeros(max(lib.trimkv_decode_attn_pieces_workspace(n, G) for _, n, _ in layouts), dtype=torch.uint8, device=DEV)
+    qs = [torch.randn(nseg * G, D, generator=gen).to(torch.bfloat16).to(DEV) for _ in range(2)]
+    first = {}
+    print("alternating piece layouts, 360 launches", flush=True)
+    for it in range(360):
+        li, qi = it % 3, (it // 3) % 2
+        plist, npieces, _ = layouts[li]
+        got = torch.empty_like(qs[qi])
+        L.check(lib.trimkv_decode_attn_pieces(qs[qi].data_ptr(), got.data_ptr(), k.data_ptr(), v.data_ptr(), LEN.data_ptr(), None, None,
+                                              plist.data_ptr(), npieces, nseg, cap, D, G, L.BF16, D ** -0.5, cap, ws.data_ptr(), ws.numel(), st), "pieces")
+        torch.cuda.synchronize()
+        if (li, qi) not in first:
+            first[(li, qi)] = got
+        else:
+            assert torch.equal(got, first[(li, qi)]), f"launch {it} (layout {li}) differs from the first launch of its layout"
+    assert not ws[:32768].any()
+
+
 def test_piece_list_arguments_are_checked():
     from trimkv_amd import _lib as L
     import ctypes

@@ -29,6 +29,11 @@ from .. import _lib
 
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
 _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
+# group sizes whose fused (append + attend) piece-list kernel fits the register file.  With more query heads per KV head it
+# spills (Qwen3-14B's group of 5, 64 segments of 8448 rows: 2.45 ms per step against 2.09 ms on the grid launch + merge
+# kernel): there the dense cache stays on the grid launch and the ragged caches run the append as its own launch in
+# front of the unfused piece-list kernel
+_FUSED_PIECES_GROUPS = (1, 2, 3, 4)
 _WARNED = set()
 dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)
 
@@ -63,6 +68,31 @@ def _workspace_zeroed(device, nbytes: int, stream: int) -> torch.Tensor:
     return ws
 
 
+_UNIFORM_PIECES: Dict[Tuple[str, int, int], torch.Tensor] = {}
+
+
+def _uniform_pieces(device, nseg: int, max_len: int):
+    """Piece list for segments of (nearly) equal length -- the dense cache.  With fewer than 256 segments each is cut so
+    that about 256 workgroups exist (a compute unit pulls about 50 GB/s whatever it runs, so all 256 are needed), but not
+    below 512 rows apiece; the pieces are merged inside the launch (``trimkv_decode_attn_pieces``), which saves the second
+    launch of the grid-split path.  None when the segments are attended whole (256 segments or more, or short ones)."""
+    if nseg >= 256 or nseg > 8192:
+        return None
+    want = (256 + nseg - 1) // nseg
+    chunk = max(512, (((max_len + want - 1) // want + 63) // 64) * 64)
+    nsp = (max_len + chunk - 1) // chunk
+    if nsp <= 1:
+        return None
+    key = (str(device), nseg, nsp)
+    t = _UNIFORM_PIECES.get(key)
+    if t is None:
+        seg = torch.arange(nseg, dtype=torch.int32).repeat(nsp)                        # piece-major: consecutive workgroups are
+        which = torch.arange(nsp, dtype=torch.int32).repeat_interleave(nseg)           # different segments (they spread over the XCDs)
+        t = torch.stack([seg, which, torch.full_like(seg, nsp), seg * nsp], dim=1).contiguous().to(device)
+        _UNIFORM_PIECES[key] = t
+    return t, nseg * nsp
+
+
 def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
     """Split-K scratch, one buffer per (device, stream): launches that share a buffer must be ordered."""
     if nbytes <= 0:
@@ -78,7 +108,7 @@ def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[to
 def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, nseg: int, group: int,
                      seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
                      scale: float, chunk: int = 0, seg_order: Optional[torch.Tensor] = None,
-                     seg_first: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     seg_first: Optional[torch.Tensor] = None, pieces=None) -> torch.Tensor:
     """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``.
     ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only).
     ``seg_first``: optional int32 [nseg], the first attended row of every segment (rows before it are masked)."""
@@ -88,11 +118,19 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
         g1 = _group_slice(group)
         q3 = query.view(nseg, group, -1)
         outs = [decode_attention(q3[:, a:a + g1].reshape(nseg * g1, -1), k_rows, v_rows, nseg, g1, seg_len, seg_start, cap, max_len,
-                                 scale, chunk, seg_order, seg_first).view(nseg, g1, -1) for a in range(0, group, g1)]
+                                 scale, chunk, seg_order, seg_first, pieces).view(nseg, g1, -1) for a in range(0, group, g1)]
         return torch.cat(outs, dim=1).view(nseg * group, -1)
     lib = _lib.load()
     d = query.shape[-1]
     out = torch.empty_like(query)
+    if pieces is not None:   # (device piece list, count): one launch, pieces merged inside it
+        st = _lib.current_stream(query.device)
+        ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(pieces[1], group), st)
+        rc = lib.trimkv_decode_attn_pieces(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(), _lib.ptr(seg_len),
+                                           _lib.ptr(seg_start), _lib.ptr(seg_first), pieces[0].data_ptr(), pieces[1], nseg, cap, d, group,
+                                           _lib.dtype_code(query.dtype), float(scale), max_len, ws.data_ptr(), ws.numel(), st)
+        _lib.check(rc, "trimkv_decode_attn_pieces")
+        return out
     ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, max_len, chunk)
     ws = _workspace(query.device, ws_bytes)
     rc = lib.trimkv_decode_attn(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(),
@@ -135,10 +173,11 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
     return out
 
 
-def _take_pending(kw: Optional[dict], query: torch.Tensor, key: torch.Tensor, group: int, fusable: bool):
+def _take_pending(kw: Optional[dict], query: torch.Tensor, key: torch.Tensor, group: int, fusable: bool, pieces=None):
     """The layer whose deferred append this attention call has to carry out, or None.  When the call cannot do it in
     its own launch (``fusable`` False, a query of another dtype, K that is not the cache's slab) the append is
-    carried out here with the ordinary kernel, so that the rows are in place either way."""
+    carried out here with the ordinary kernel, so that the rows are in place either way.  ``pieces``: the piece list the
+    launch would use (the fused piece-list kernel exists without spills only for some group sizes)."""
     pend = kw.get("pending_append") if kw else None
     if pend is None:
         return None
@@ -146,7 +185,7 @@ def _take_pending(kw: Optional[dict], query: torch.Tensor, key: torch.Tensor, gr
     if slab.pending is None:
         return None
     if (fusable and group <= _MAX_GROUP and query.is_cuda and query.dtype == slab.k.dtype and key.data_ptr() == slab.k.data_ptr()
-            and query.shape[-1] == slab.D):
+            and query.shape[-1] == slab.D and (pieces is None or group in _FUSED_PIECES_GROUPS)):
         return slab
     cache._flush(slab)
     return None
@@ -220,12 +259,15 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     Hkv, n = key.shape[1], key.shape[2]
     G = Hq // Hkv
     scale = D ** -0.5 if scaling is None else scaling
-    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None)
+    dense_pieces = None
+    if Q == 1 and not dense_chunk and G in _FUSED_PIECES_GROUPS:
+        dense_pieces = _uniform_pieces(query.device, B * Hkv, n)
+    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None, dense_pieces)
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        return append_attend(slab, q2, G, scale, chunk=dense_chunk).view(B, 1, Hq, D), None, None
+        return append_attend(slab, q2, G, scale, chunk=dense_chunk, pieces=dense_pieces).view(B, 1, Hq, D), None, None
     seg_first = None
     if attention_mask is not None and Q == 1 and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         seg_first = _left_padding_offsets(attention_mask, B, n, Hkv)   # a left-padding mask is a per-segment first row
@@ -241,7 +283,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
-        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first)
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first, pieces=dense_pieces)
         return out.view(B, 1, Hq, D), None, None
     if attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
@@ -283,7 +325,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
     if num_kv_heads is None:
         num_kv_heads = nseg // batch_size
     G = Hq // num_kv_heads
-    slab = _take_pending(kw, query, key, G, Q == 1 and kw.get("seg_start") is not None)
+    slab = _take_pending(kw, query, key, G, Q == 1 and kw.get("seg_start") is not None, kw.get("pieces"))
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
@@ -305,19 +347,9 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         q2 = query.reshape(B * Hq, D)  # [B,Hq,1,D]: row seg*G+g is query head h*G+g of batch b
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        pieces = kw.get("pieces")
-        if pieces is not None and G <= _MAX_GROUP:
-            lib = _lib.load()
-            out = torch.empty_like(q2)
-            st = _lib.current_stream(q2.device)
-            ws = _workspace_zeroed(q2.device, lib.trimkv_decode_attn_pieces_workspace(pieces[1], G), st)
-            rc = lib.trimkv_decode_attn_pieces(q2.data_ptr(), out.data_ptr(), key.data_ptr(), value.data_ptr(), head_lens.data_ptr(),
-                                               seg_start.data_ptr(), None, pieces[0].data_ptr(), pieces[1], nseg, cap, D, G,
-                                               _lib.dtype_code(q2.dtype), D ** -0.5, max(1, max_len), ws.data_ptr(), ws.numel(), st)
-            _lib.check(rc, "trimkv_decode_attn_pieces")
-            return out.view(B, 1, Hq, D), None, None
+        pieces = kw.get("pieces") if G <= _MAX_GROUP else None
         out = decode_attention(q2, key, value, nseg, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5,
-                               chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"))
+                               chunk=kw.get("chunk", 0), seg_order=kw.get("seg_order"), pieces=pieces)
         return out.view(B, 1, Hq, D), None, None
     out = prefill_attention(query, key, value, batch_size, num_kv_heads, G, head_lens, seg_start, cap, max(1, max_len), D ** -0.5)
     return out, None, None

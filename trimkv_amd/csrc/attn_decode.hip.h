@@ -192,20 +192,29 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     // APPEND: the new row is fetched by every wavefront right behind q (the same 512 bytes per segment; unconditional
     // loads keep the compiler's count of outstanding loads exact) and stored by the wavefront that owns it once q's wait
     // below has covered these loads too -- no round trip of its own.
+    // With more than four query heads the streaming loop has no registers to spare for the eleven that the row would
+    // occupy until then (it spilled): there the owning wavefront fetches and stores the row after its loop instead, at
+    // the price of one round trip at the end of that one wavefront.
+    constexpr bool APPEND_EARLY = APPEND && G <= 4;
     const uint4* knew = nullptr;
     const uint4* vnew = nullptr;
     uint4 kn = make_uint4(0u, 0u, 0u, 0u), vn = kn;
     float lbn = 0.0f;
     int64_t pn = 0;
+    int64_t lb_off = 0, pos_off = 0;
     if (APPEND) {
         const int b = seg / a.ap.kv_heads, h = seg - b * a.ap.kv_heads;
         const int64_t off = (int64_t)b * a.ap.kv_sb + (int64_t)h * a.ap.kv_sh + ((int64_t)cc << 4);
         knew = (const uint4*)(a.ap.k_new + off);
         vnew = (const uint4*)(a.ap.v_new + off);
-        kn = *knew;
-        vn = *vnew;
-        lbn = load_as_f32(a.ap.lb_new, (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh, a.ap.lb_dtype);
-        pn = a.ap.pos_new[(int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh];
+        lb_off = (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh;
+        pos_off = (int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh;
+        if (APPEND_EARLY) {
+            kn = *knew;
+            vn = *vnew;
+            lbn = load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype);
+            pn = a.ap.pos_new[pos_off];
+        }
     }
 
     // which (row-in-tile, head) this lane owns after the transposing reduction
@@ -366,7 +375,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         for (int sl = 0; sl < PD; ++sl) load_tile(kp, knew, w0 + sl * TILE_ROWS, ring[sl % RING]);
 #pragma unroll
         for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
-        if (APPEND && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
+        if (APPEND_EARLY && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
             const int64_t dst = row0 + new_row;
             if (r == 0 && c < ROW16) {
                 ((uint4*)a.k)[dst * ROW16 + c] = kn;
@@ -390,6 +399,20 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             else if (need <= 4) run_block(integral_constant<int, 4>{}, false_type{}, blk, rest);
             else if (need <= 8) run_block(integral_constant<int, (NT >= 8 ? 8 : NT)>{}, false_type{}, blk, rest);
             else run_block(integral_constant<int, NT>{}, false_type{}, blk, rest);
+        }
+    }
+
+    if (APPEND && !APPEND_EARLY && new_row >= w0 && new_row < w1) {   // the owning wavefront, after its loop (wide groups)
+        kn = *knew;
+        vn = *vnew;
+        const int64_t dst = row0 + new_row;
+        if (r == 0 && c < ROW16) {
+            ((uint4*)a.k)[dst * ROW16 + c] = kn;
+            ((uint4*)a.v)[dst * ROW16 + c] = vn;
+        }
+        if (lane == 0) {
+            store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype));
+            a.ap.pos_slab[dst] = a.ap.pos_new[pos_off];
         }
     }
 
@@ -494,13 +517,14 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     const int live = n - first;
     const int rps = (live + nsp - 1) / nsp;
     const int t0 = min(n, first + piece * rps), t1 = min(n, t0 + rps);   // may be empty: the piece then contributes nothing
-    if (nsp == 1) {
-        attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, true, 0, new_row);
-        return;
-    }
     const int64_t slot0 = e.w;
-    attend_rows<G, ROW16, F16, APPEND, true>(a, seg, t0, t1, false, slot0 + piece, new_row);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every thread: its partial stores have completed
+    // one instantiation for both cases (a second inlined copy of the streaming loop costs registers): a segment in one
+    // piece writes its output itself, the others leave partials
+    attend_rows<G, ROW16, F16, APPEND, true>(a, seg, t0, t1, nsp == 1, slot0 + piece, new_row);
+    if (nsp == 1) return;
+    // every thread waits until its own partial stores have been acknowledged (they are write-through stores: the
+    // acknowledgement comes from memory), only then may the counter move
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     if (threadIdx.x == 0) {
         const uint32_t done = __hip_atomic_fetch_add(&a.counters[seg], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
