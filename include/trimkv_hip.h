@@ -348,20 +348,30 @@ int trimkv_append_attend(const void* q, void* out,
  * Piece-list launches -- trimkv_decode_attn and trimkv_append_attend for very uneven segment lengths (per-head budgets,
  * src/trimkv/cache_utils.py:485-536, 789-806), in ONE launch even when segments are cut into pieces.
  *
- * `pieces` is a device array of npieces entries of four int32 {segment, piece, pieces_of_segment, first_slot}: the
- * workgroup of entry i attends rows [first + piece*r, first + (piece+1)*r) of its segment, r = ceil(rows /
- * pieces_of_segment) computed from the segment's length on the device (so the list stays valid while lengths drift; a
- * piece may turn out empty), and the pieces of one segment use partial slots first_slot .. first_slot +
+ * `pieces` is a device array of npieces entries of four int32
+ *     {segment, piece | begin << 16, pieces_of_segment | end << 16, first_slot}
+ * (piece and pieces_of_segment below 65536).  With begin = end = 0 the workgroup of entry i attends rows
+ * [first + piece*r, first + (piece+1)*r) of its segment, r = ceil(rows / pieces_of_segment): equal pieces.  Otherwise
+ * it attends rows [first + rows*begin/32768, first + rows*end/32768) (TRIMKV_PIECE_FRACTION = 32768, quotients rounded
+ * down): pieces of any size; consecutive pieces of a segment share a bound, the first begins at 0 and the last ends at
+ * 32768.  Either way the rows come from the segment's length on the device, so a list stays valid while lengths drift (a
+ * piece may turn out empty).  The pieces of one segment use partial slots first_slot .. first_slot +
  * pieces_of_segment - 1 (distinct segments: disjoint slot ranges below npieces).  Every segment must appear with all of
- * its pieces exactly once.  Workgroups are dispatched in list order: sort it so that consecutive entries carry
- * comparable row counts and long pieces come first.  A segment in one piece writes its output directly; otherwise the
+ * its pieces exactly once, and together they must cover its rows exactly once: the kernel bounds every access by the
+ * segment's length but cannot check the cover.  A segment in one piece writes its output directly; otherwise the
  * workgroup that finishes last merges the partials inside the same launch (no second kernel).
+ *
+ * Workgroups are dispatched in list order.  A launch of at most twice as many pieces as the GPU has compute units is
+ * resident from its first cycle, entries i and i + compute_units run on the same compute unit, and a compute unit's
+ * share of the memory bandwidth does not depend on how much it has to do: the launch ends with the compute unit that
+ * holds the most rows.  trimkv_plan_attn_pieces builds a list in which all hold the same.
  *
  * workspace: trimkv_decode_attn_pieces_workspace(npieces, group) bytes, 16-byte aligned.  Its first 32 KiB hold one
  * counter per segment and MUST be zero when the workspace is first used; every launch leaves them zero again.  At most
  * 8192 segments.  Launches that share a workspace must be ordered (same stream).  Other arguments as in
  * trimkv_decode_attn / trimkv_append_attend (no chunk, no seg_order: the list replaces both).
  */
+#define TRIMKV_PIECE_FRACTION 32768
 size_t trimkv_decode_attn_pieces_workspace(int npieces, int group);
 int trimkv_decode_attn_pieces(const void* q, void* out, const void* k_slab, const void* v_slab,
                               const int32_t* seg_len, const int32_t* seg_start, const int32_t* seg_first,
@@ -377,6 +387,25 @@ int trimkv_append_attend_pieces(const void* q, void* out,
                                 const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
                                 float scale, int max_len_after,
                                 void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * trimkv_plan_attn_pieces -- builds the piece list of the two entry points above on the HOST (no GPU work, nothing
+ * is launched; seg_len and pieces are host pointers).  It replaces nothing in the reference, whose varlen kernel
+ * schedules its own blocks (flash_attn_varlen_func, src/trimkv/attn/flash_attn.py:61-71); it exists because the best cut
+ * of very uneven segments depends on all of them together.
+ *
+ * Every compute unit gets total_rows / compute_units rows in at most two pieces: segments no longer than that stay
+ * whole, the longer ones are cut where a compute unit is full (pieces of different sizes, given as fractions).  Gaps
+ * and slivers of fewer than min_rows rows are not worth a piece (64 is a good value).  With fewer than 2*min_rows rows
+ * per compute unit, or more short segments than compute units, the list is simply every segment whole, longest first.
+ * seg_len: the lengths the launch will see, or close to them (the kernel scales the cuts to the lengths it finds);
+ * for trimkv_append_attend_pieces either the lengths before or after the append.  Copy the result to the device
+ * (16-byte aligned) and reuse it until the lengths have moved by a few per cent.
+ * Returns the number of entries written (>= nseg, <= nseg + 2*compute_units), or a negative trimkv_status:
+ * TRIMKV_ERR_WORKSPACE when max_pieces entries are too few.
+ */
+int trimkv_plan_attn_pieces(const int32_t* seg_len, int nseg, int compute_units, int min_rows,
+                            int32_t* pieces, int max_pieces);
 
 /*
  * trimkv_decode_attn_static -- trimkv_decode_attn for callers that cannot allocate device memory (code under HIP

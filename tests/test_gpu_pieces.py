@@ -86,6 +86,46 @@ def test_piece_list_launch_matches_fp32_and_the_grid_launch(G, D, order):
     assert (got.float() - want.float()).abs().max() < 6e-3
 
 
+@pytest.mark.parametrize("G,nseg,ncu", [(4, 256, 256), (1, 200, 256), (5, 64, 256), (2, 40, 16)])
+def test_planned_piece_list_matches_fp32_and_the_grid_launch(G, nseg, ncu):
+    """Lists from trimkv_plan_attn_pieces (pieces of unequal size, bounds as fractions) at the lengths they were planned for and
+    at drifted lengths; against the grid launch and the fp32 formula."""
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    D = 128
+    rng = np.random.default_rng(G * 1000 + nseg)
+    cap = 4300
+    lens = np.clip(np.round(np.exp(rng.normal(np.log(600), 1.0, size=nseg))), 0, cap - 200).astype(np.int32)
+    lens[0], lens[1], lens[2] = 0, 1, cap - 200
+    gen = torch.Generator().manual_seed(nseg)
+    k = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    v = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
+    q = torch.randn(nseg * G, D, generator=gen).to(torch.bfloat16).to(DEV)
+    st = L.current_stream(torch.device(DEV))
+    scale = D ** -0.5
+    room = nseg + 2 * ncu
+    host = np.zeros((room, 4), dtype=np.int32)
+    npieces = lib.trimkv_plan_attn_pieces(lens.ctypes.data, nseg, ncu, 64, host.ctypes.data, room)
+    assert npieces >= nseg
+    plist = torch.from_numpy(host[:npieces].copy()).to(DEV)
+    ws = torch.zeros(lib.trimkv_decode_attn_pieces_workspace(npieces, G), dtype=torch.uint8, device=DEV)
+    ws0 = torch.empty(max(16, lib.trimkv_decode_attn_workspace(nseg, G, D, cap, 512)), dtype=torch.uint8, device=DEV)
+    for seen in (lens, np.minimum(cap, lens + rng.integers(0, 150, size=nseg)).astype(np.int32)):
+        LEN = torch.from_numpy(seen).to(DEV)
+        want, got = torch.empty_like(q), torch.full_like(q, 3.0)
+        L.check(lib.trimkv_decode_attn(q.data_ptr(), want.data_ptr(), k.data_ptr(), v.data_ptr(), LEN.data_ptr(), None, None, None,
+                                       nseg, cap, D, G, L.BF16, scale, cap, 512, ws0.data_ptr(), ws0.numel(), st), "grid")
+        print(f"planned pieces G={G} nseg={nseg} ncu={ncu} npieces={npieces}", flush=True)
+        L.check(lib.trimkv_decode_attn_pieces(q.data_ptr(), got.data_ptr(), k.data_ptr(), v.data_ptr(), LEN.data_ptr(), None, None,
+                                              plist.data_ptr(), npieces, nseg, cap, D, G, L.BF16, scale, cap, ws.data_ptr(), ws.numel(), st), "pieces")
+        torch.cuda.synchronize()
+        assert not ws[:32768].any()
+        assert (got.float() - want.float()).abs().max() < 6e-3
+        segs = [0, 1, 2, 5, nseg // 2, nseg - 1]
+        ok, err = attn_close(got.view(nseg, G, D)[segs], _fp32(q, k, v, seen, G, segs))
+        assert ok, err
+
+
 def test_append_attend_pieces_equals_append_then_attend():
     """The fused piece-list launch against trimkv_append followed by the unfused piece-list launch: outputs, rows, lengths and
     cu_seqlens bit-identical, over several steps on the same workspace; includes a full slab (not appended)."""

@@ -90,7 +90,7 @@ class _Slab:
     """Device storage of one layer."""
 
     __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order",
-                 "pending", "codes", "total", "pieces", "pieces_total", "pieces_age")
+                 "pending", "codes", "total", "pieces", "pieces_total", "pieces_age", "pieces_buf")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -108,6 +108,7 @@ class _Slab:
         self.pending = None  # a one-token append that the next attention call will carry out (see _SlabBacked._defer)
         self.pieces = None   # ragged caches: (device piece list, number of pieces) of the decode-attention launch
         self.pieces_total, self.pieces_age = 0, 0
+        self.pieces_buf = None   # the list's storage: device tensor, two pinned host copies with an event each, next copy to use
         self._refresh_views()
 
     def _refresh_views(self) -> None:
@@ -599,7 +600,7 @@ class TrimKVCache(_SlabBacked):
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
                 new.lens, new.max_len, new.order = slab.lens[lo:hi].copy(), slab.max_len, None
                 new.pending, new.total = None, int(new.lens.sum())
-                new.pieces, new.pieces_total, new.pieces_age = None, 0, 0
+                new.pieces, new.pieces_total, new.pieces_age, new.pieces_buf = None, 0, 0, None
                 new._refresh_views()
                 part._slabs.append(new)
             out.append(part)
@@ -635,7 +636,7 @@ class TrimKVCache(_SlabBacked):
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
             c.lens, c.max_len, c.order = slab.lens.copy(), slab.max_len, None
             c.pending, c.total = None, slab.total
-            c.pieces, c.pieces_total, c.pieces_age = None, 0, 0
+            c.pieces, c.pieces_total, c.pieces_age, c.pieces_buf = None, 0, 0, None
             c._refresh_views()
             new._slabs.append(c)
         return new
@@ -681,7 +682,10 @@ class _RaggedCache(_SlabBacked):
         # update() normally hands the attention call the slab rows plus ``seg_start`` (no copy).  With this flag, or with
         # ``cache_kwargs={"packed": True}`` on a call, it returns the reference's packed ``[sum(n), D]`` tensors instead.
         self.return_packed = False
-        self.attention_pieces = 400   # split-K tuning knob: about this many pieces per decode-attention launch
+        self.attention_pieces = 400   # grid-split fallback only: about this many pieces per decode-attention launch
+        self.attention_compute_units = 256   # what the piece lists of the decode-attention launches are balanced for (MI355X)
+        self.attention_replan_steps = 32     # a layer's piece list is rebuilt at least this often
+        self._replans = 0
 
     # plain attributes in the reference; a property here because newer HF Cache classes define a
     # read-only `batch_size` of their own
@@ -755,33 +759,41 @@ class _RaggedCache(_SlabBacked):
 
     def _piece_list(self, slab: _Slab):
         """The decode-attention launch of a ragged layer as a list of (segment, piece) workgroups, see
-        ``trimkv_decode_attn_pieces``: every segment is cut into ``round(length / target)`` pieces with ``target`` = rows
-        cached / ``attention_pieces``, and the pieces are dispatched longest first, the second 256 in rising order so that
-        the two workgroups a compute unit starts with add up to about the same number of rows everywhere.  The kernel
-        derives row ranges from the lengths on the device, so the list only has to be roughly right: it is rebuilt when the
-        rows cached have drifted by 4 %, after an eviction that changed them wholesale, or after 64 steps."""
+        ``trimkv_decode_attn_pieces``.  ``trimkv_plan_attn_pieces`` cuts the segments so that every compute unit holds the same
+        number of rows in its two workgroups (a launch ends with the compute unit that holds the most).  The kernel scales the
+        cuts to the lengths it finds on the device, so the list only has to be roughly right: it is rebuilt when the rows
+        cached have drifted by 4 %, after an eviction that changed them wholesale, or after ``attention_replan_steps`` steps.
+        The list goes to the device through pinned memory with a copy in stream order: no synchronisation."""
         slab.pieces_age += 1
-        if (slab.pieces is not None and slab.pieces_age < 64 and abs(slab.total - slab.pieces_total) * 25 <= slab.pieces_total):
+        if (slab.pieces is not None and slab.pieces_age < self.attention_replan_steps
+                and abs(slab.total - slab.pieces_total) * 25 <= slab.pieces_total):
             return slab.pieces
-        lens = slab.lens
-        nseg = lens.size
+        nseg = slab.lens.size
         if nseg > 8192:
             slab.pieces = None
             return None
-        target = max(256.0, float(max(1, slab.total)) / self.attention_pieces)
-        nsp = np.maximum(1, np.rint(lens / target)).astype(np.int64)
-        slot0 = np.cumsum(nsp) - nsp
-        seg_ids = np.repeat(np.arange(nseg, dtype=np.int64), nsp)
-        which = np.arange(int(nsp.sum()), dtype=np.int64) - np.repeat(slot0, nsp)
-        rows = np.repeat(-(-lens // nsp), nsp)
-        order = np.argsort(-rows, kind="stable")
-        if order.size > 256:
-            # workgroups i and i + 256 start on the same compute unit: measured 1.66 ms per step with this pairing against
-            # 1.79 ms for a plain longest-first list (256 lognormal segments, 36 layers)
-            order[256:512] = order[256:512][::-1].copy()
-        arr = np.stack([seg_ids, which, np.repeat(nsp, nsp), np.repeat(slot0, nsp)], axis=1)[order].astype(np.int32)
-        slab.pieces = (torch.from_numpy(np.ascontiguousarray(arr)).to(slab.k.device), int(arr.shape[0]))
-        slab.pieces_total, slab.pieces_age = slab.total, 0
+        room = nseg + 2 * self.attention_compute_units
+        buf = slab.pieces_buf
+        if buf is None or buf[0].shape[0] < room:
+            dev = torch.empty(room, 4, dtype=torch.int32, device=slab.k.device)
+            host = [torch.empty(room, 4, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+            buf = slab.pieces_buf = [dev, host, [None, None], 0]
+        dev, host, events, which = buf
+        if events[which] is not None:
+            events[which].synchronize()   # the copy that last read this host buffer (two rebuilds ago) has long finished
+        lens32 = np.ascontiguousarray(slab.lens, dtype=np.int32)
+        n = _lib.load().trimkv_plan_attn_pieces(lens32.ctypes.data, nseg, self.attention_compute_units, 64, host[which].data_ptr(), room)
+        if n < 0:
+            _lib.check(n, "trimkv_plan_attn_pieces")
+        dev[:n].copy_(host[which][:n], non_blocking=True)
+        ev = events[which] or torch.cuda.Event()
+        ev.record()
+        events[which] = ev
+        buf[3] = which ^ 1
+        slab.pieces = (dev, int(n))
+        # layers that were planned in the same step come due a few steps apart: their rebuilds do not pile up in one step
+        self._replans = (self._replans + 1) % 8
+        slab.pieces_total, slab.pieces_age = slab.total, -self._replans
         return slab.pieces
 
     def _seg_start(self, slab: _Slab) -> torch.Tensor:

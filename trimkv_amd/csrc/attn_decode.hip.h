@@ -125,11 +125,18 @@ struct AttnArgs {
     const int4* pieces; uint32_t* counters; int npieces;
 };
 
+// Row bounds of a piece inside its segment are fractions with this denominator (trimkv_hip.h: TRIMKV_PIECE_FRACTION).
+constexpr int AT_PIECE_FRACTION_BITS = 15;
+constexpr int AT_PIECE_FRACTION = 1 << AT_PIECE_FRACTION_BITS;
+static_assert(AT_PIECE_FRACTION == TRIMKV_PIECE_FRACTION, "header and kernel disagree on the piece fraction");
+
 // Partials that another workgroup of the same launch will read.  Workgroups of one launch run on different XCDs, whose L2
 // caches are not coherent with each other, so these accesses are device-scope atomics (relaxed): the stores write through
 // to memory and the loads do not hit a stale line.  Ordering between them and the per-segment counter is by completion:
-// the writer waits for its stores (s_waitcnt through a workgroup-scope release fence) before it bumps the counter, and the
-// reader issues its loads after the bump has returned.  No L2 write-back or invalidate is involved.
+// every thread of the writer waits until its stores have been acknowledged (an explicit s_waitcnt vmcnt(0); a release fence
+// at workgroup scope does not wait for write-through stores and let a reader see an old slot now and then) before the
+// workgroup bumps the counter, and the reader issues its loads after the bump has returned.  No L2 write-back or
+// invalidate is involved.
 __device__ __forceinline__ void store_shared_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ float load_shared_partial(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
@@ -335,33 +342,34 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         // "wait for this tile, leave the prefetched ones in flight") only when every path issues
         // the same loads.  Rows are clamped to the wavefront's last row, so a load past the end is
         // legal and re-reads cached bytes; its scores are masked.
-        // CHAINED: the first PD slots are already in flight and the block prefetches the first PD
-        // slots of the block that follows it (the steady-state loop over full blocks).
-        auto run_block = [&](auto ntb_c, auto chained_c, int blk, int nrows) __attribute__((always_inline)) {
+        // Every block finds its first PD slots already in flight: the prefetch ahead of the loop or the block before it
+        // issued them.  NEXT: the block prefetches the first PD slots of the block that follows it (the steady-state loop
+        // over full blocks); the tail block does not.
+        auto run_block = [&](auto ntb_c, auto next_c, int blk, int nrows) __attribute__((always_inline)) {
             constexpr int NTB = decltype(ntb_c)::value;
-            constexpr bool CHAINED = decltype(chained_c)::value;
+            constexpr bool NEXT = decltype(next_c)::value;
             constexpr int SL = 2 * NTB;
-            static_assert(!CHAINED || (SL % RING == 0 && PD <= NTB), "chained blocks need ring-aligned slots");
+            static_assert(!NEXT || (SL % RING == 0 && PD <= NTB), "chained blocks need ring-aligned slots");
             auto load_slot = [&](int slot, int base_row, uint4 (&dst)[NJ]) __attribute__((always_inline)) {
                 if (slot < NTB) load_tile(kp, knew, base_row + slot * TILE_ROWS, dst);
                 else load_tile(vp, vnew, base_row + (slot - NTB) * TILE_ROWS, dst);
             };
-            if (!CHAINED) {
+            // A block of fewer than PD tiles: the tiles in flight beyond its own K tiles belong to rows past the end and
+            // are dropped; its first V tiles take their ring slots.
 #pragma unroll
-                for (int sl = 0; sl < (PD < SL ? PD : SL); ++sl) load_slot(sl, blk, ring[sl % RING]);
-            }
+            for (int sl = NTB; sl < (PD < SL ? PD : SL); ++sl) load_slot(sl, blk, ring[sl % RING]);
 #pragma unroll
             for (int sl = 0; sl < SL; ++sl) {
                 const int ahead = sl + PD;
                 if (ahead < SL) load_slot(ahead, blk, ring[ahead % RING]);
-                else if (CHAINED) load_slot(ahead - SL, blk + NTB * TILE_ROWS, ring[ahead % RING]);
+                else if (NEXT) load_slot(ahead - SL, blk + NTB * TILE_ROWS, ring[ahead % RING]);
                 // keep the prefetch where it is: left alone, the scheduler sinks these loads past
                 // the arithmetic to shorten live ranges, which empties the pipeline
                 __builtin_amdgcn_sched_barrier(0);
                 if (sl == NTB) softmax_of_block(ntb_c, nrows);
                 if (sl < NTB) {
                     s[sl] = scores_of_tile(sl, blk, ring[sl % RING]);
-                } else if (CHAINED || (sl - NTB) * TILE_ROWS < nrows) {
+                } else if (NEXT || (sl - NTB) * TILE_ROWS < nrows) {
                     accumulate_tile(sl - NTB, ring[sl % RING]);
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -390,7 +398,10 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
 #pragma unroll 1
         for (; blk + AT_BLOCK_ROWS <= w1; blk += AT_BLOCK_ROWS)
             run_block(integral_constant<int, NT>{}, true_type{}, blk, AT_BLOCK_ROWS);
-        // the tail (< 128 rows): the smallest power-of-two block that covers it, one pipelined pass
+        // the tail (< 128 rows): the smallest power-of-two block that covers it, entered with its first tiles in flight
+        // like any other block (a tail that started its own loads would expose one more memory round trip per wavefront,
+        // a large part of a short piece's time).  Small blocks matter: at a wavefront's end nothing hides the arithmetic of
+        // tiles that are only there to be masked.
         const int rest = w1 - blk;
         if (rest > 0) {
             const int need = (rest + TILE_ROWS - 1) / TILE_ROWS;  // 1 .. NT tiles
@@ -510,13 +521,23 @@ template <int G, int ROW16, bool F16, bool APPEND>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_pieces_kernel(AttnArgs a) {
     __shared__ int last_of_segment;
     const int4 e = a.pieces[blockIdx.x];
-    const int seg = min(max(e.x, 0), a.nseg - 1), nsp = max(e.z, 1), piece = min(max(e.y, 0), nsp - 1);
+    // entry = {segment, piece | begin << 16, pieces of the segment | end << 16, first partial slot}
+    const uint32_t ey = (uint32_t)e.y, ez = (uint32_t)e.z;
+    const int seg = min(max(e.x, 0), a.nseg - 1), nsp = max((int)(ez & 0xffffu), 1), piece = min((int)(ey & 0xffffu), nsp - 1);
     if (nsp > 1 && (e.w < 0 || e.w + nsp > a.npieces)) return;   // a list whose partial slots do not fit the workspace: touch nothing
     int new_row, first;
     const int n = segment_rows<APPEND>(a, seg, &new_row, &first);
     const int live = n - first;
-    const int rps = (live + nsp - 1) / nsp;
-    const int t0 = min(n, first + piece * rps), t1 = min(n, t0 + rps);   // may be empty: the piece then contributes nothing
+    int t0, t1;   // may be empty: the piece then contributes nothing
+    const uint32_t f1 = min(ez >> 16, (uint32_t)AT_PIECE_FRACTION), f0 = min(ey >> 16, f1);
+    if (f1 == 0) {           // equal pieces
+        const int rps = (live + nsp - 1) / nsp;
+        t0 = min(n, first + piece * rps);
+        t1 = min(n, t0 + rps);
+    } else {                 // rows [begin, end) / 32768 of the segment: neighbours that share a bound share the row it maps to
+        t0 = first + (int)(((int64_t)live * f0) >> AT_PIECE_FRACTION_BITS);
+        t1 = first + (int)(((int64_t)live * f1) >> AT_PIECE_FRACTION_BITS);
+    }
     const int64_t slot0 = e.w;
     // one instantiation for both cases (a second inlined copy of the streaming loop costs registers): a segment in one
     // piece writes its output itself, the others leave partials
@@ -572,11 +593,11 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     }
 }
 
-// Merge of the split-K partials of one segment: thread (g, d) reads the (max, sum) pairs of all
-// splits first (independent loads), then the accumulators.  A separate launch on purpose: the
-// kernel boundary is what makes partials written on one XCD visible on another; doing the same
-// inside one kernel needs device-scope fences (an L2 write-back and invalidate per workgroup on
-// this part), which costs far more than the launch.
+// Merge of the split-K partials of one segment after a grid launch: thread (g, d) reads the (max, sum)
+// pairs and the accumulators of eight splits per round trip.  As a launch of its own, the kernel
+// boundary is what makes partials written on one XCD visible on another, with plain stores and loads;
+// the piece-list kernel above merges inside its launch instead and pays for that with write-through
+// accesses and a counter per segment.
 template <int G, int ROW16, bool F16, bool APPEND>
 __global__ __launch_bounds__(G * AT_D) void decode_attn_merge_kernel(AttnArgs a) {
     const int seg = blockIdx.x, g = threadIdx.x / AT_D, d = threadIdx.x - g * AT_D;
