@@ -281,7 +281,7 @@ def ragged_main(args):
     cache = BatchedDynamicBudgetTrimKVCache()
     cache.fuse_decode_append = not args.no_fuse
     if args.chunk:
-        cache.attention_pieces = args.chunk     # with --config 4: pieces per launch instead of rows per piece
+        cache.attention_pieces = args.chunk     # with --config 4: pieces per launch of the grid-split fallback (the fused step plans its own)
     S0 = int(start.max())
     cache.set_budgets(start)
     for l in range(L):   # ragged initial state: every head keeps its best min(budget, prompt) tokens of a synthetic prompt

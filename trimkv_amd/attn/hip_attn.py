@@ -35,6 +35,7 @@ _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
 # front of the unfused piece-list kernel
 _FUSED_PIECES_GROUPS = (1, 2, 3, 4)
 _WARNED = set()
+dense_workgroups, dense_min_rows = 256, 512   # piece-list launches of the dense cache: workgroups wanted, fewest rows apiece
 dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)
 
 
@@ -78,8 +79,8 @@ def _uniform_pieces(device, nseg: int, max_len: int):
     launch of the grid-split path.  None when the segments are attended whole (256 segments or more, or short ones)."""
     if nseg >= 256 or nseg > 8192:
         return None
-    want = (256 + nseg - 1) // nseg
-    chunk = max(512, (((max_len + want - 1) // want + 63) // 64) * 64)
+    want = (dense_workgroups + nseg - 1) // nseg
+    chunk = max(dense_min_rows, (((max_len + want - 1) // want + 63) // 64) * 64)
     nsp = (max_len + chunk - 1) // chunk
     if nsp <= 1:
         return None
