@@ -260,6 +260,22 @@ int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg,
                         void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * trimkv_evict_listed -- trimkv_evict_layers for the (layer, segment) pairs of a list only: `work` is a device array of
+ * nwork int32, each layer * nseg + segment (layer = index into `layers`); one workgroup per entry, entries that name no
+ * pair of this launch are skipped, a pair must not appear twice.  For per-head budgets that come due a few segments at a
+ * time (src/trimkv/cache_utils.py:508-521 runs its top-k over every head at every compress): a launch over all
+ * nlayers * nseg pairs, of which most return at once, costs about 0.1 ms per 10 000 workgroups in dispatch alone.
+ * Every listed segment is still checked against its budget and `slack` on the device.  Other arguments and results as
+ * trimkv_evict_layers.  nwork = 0 launches nothing.
+ */
+int trimkv_evict_listed(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                        int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                        int64_t q_idx, const int64_t* q_idx_dev,
+                        int strategy, int rounding, int sliding_window, int max_len,
+                        const int32_t* work, int nwork,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * trimkv_compact_threshold_layers -- trimkv_compact_threshold for nlayers layers in one launch
  * (the per-layer rebuild loops at cache_utils.py:466-482, 912-943).  thr_key / tie_take are
  * [ngroups] shared by all layers (thr_layer_stride = 0: one budget across layers) or

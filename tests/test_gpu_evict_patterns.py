@@ -73,3 +73,58 @@ def test_ragged_per_segment_budgets_including_zero_shift_and_single_row():
         assert torch.equal(rows_k[off:off + want.numel()], k[b, h, want]), f"segment {seg}"
         off += want.numel()
     assert cache.head_lens[0].cpu().tolist() == budgets.tolist()
+
+
+def test_listed_eviction_equals_the_launch_over_every_pair():
+    """trimkv_evict_listed with the due (layer, segment) pairs -- plus pairs that are not due, and entries that name no pair --
+    against trimkv_evict_layers over all pairs: identical slabs and lengths; untouched pairs stay untouched."""
+    import numpy as np
+    from trimkv_amd import _lib as L
+    from trimkv_amd.cache_utils import _SlabBacked
+    lib = L.load()
+    nlayers, nseg, D, cap, buf = 5, 24, 128, 700, 32
+    rng = np.random.default_rng(11)
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    budgets = rng.integers(40, 500, size=(nlayers, nseg)).astype(np.int32)
+    lens = (budgets + rng.integers(0, 2 * buf, size=budgets.shape)).astype(np.int32)      # about half are due (len >= budget + buf)
+    lens[0, 0], budgets[0, 0] = 0, 10
+    due = (lens > budgets) & (lens >= budgets + buf)
+    assert 0 < due.sum() < due.size
+
+    def state():
+        g = torch.Generator(device=DEV).manual_seed(5)
+        layers = []
+        for l in range(nlayers):
+            layers.append(dict(K=torch.randn(nseg, cap, D, generator=g, device=DEV).to(torch.bfloat16),
+                               V=torch.randn(nseg, cap, D, generator=g, device=DEV).to(torch.bfloat16),
+                               LB=-torch.rand(nseg, cap, generator=g, device=DEV),
+                               POS=torch.arange(cap, device=DEV).repeat(nseg, 1).contiguous(),
+                               LEN=torch.from_numpy(lens[l].copy()).to(DEV)))
+        arr = np.zeros(nlayers, dtype=_SlabBacked._LAYER_DT)
+        for i, s in enumerate(layers):
+            arr[i] = (s["K"].data_ptr(), s["V"].data_ptr(), s["LB"].data_ptr(), s["POS"].data_ptr(), s["LEN"].data_ptr(), 0, cap, 0)
+        return layers, torch.from_numpy(arr.view(np.uint8)).to(DEV)
+
+    keep = torch.from_numpy(budgets).to(DEV)
+    st = L.current_stream(torch.device(DEV))
+    a, ta = state()
+    b, tb = state()
+    L.check(lib.trimkv_evict_layers(ta.data_ptr(), nlayers, nseg, D, L.BF16, L.F32, 0, keep.data_ptr(), nseg, buf, cap + 1, None,
+                                    L.SCORE_ALPHA, L.ROUND_UPCAST, 0, cap, None, 0, st), "evict_layers")
+    not_due = np.flatnonzero(~due.ravel())[:7]
+    work = np.concatenate([np.flatnonzero(due.ravel())[::-1], not_due, [-1, nlayers * nseg, 1 << 30]]).astype(np.int32)
+    wdev = torch.from_numpy(work).to(DEV)
+    print(f"listed eviction: {int(due.sum())} due of {due.size}, list of {work.size}", flush=True)
+    L.check(lib.trimkv_evict_listed(tb.data_ptr(), nlayers, nseg, D, L.BF16, L.F32, 0, keep.data_ptr(), nseg, buf, cap + 1, None,
+                                    L.SCORE_ALPHA, L.ROUND_UPCAST, 0, cap, wdev.data_ptr(), work.size, None, 0, st), "evict_listed")
+    torch.cuda.synchronize()
+    want_len = np.where(due, budgets, lens)
+    for l in range(nlayers):
+        assert (a[l]["LEN"].cpu().numpy() == want_len[l]).all()
+        for key in ("LEN", "K", "V", "LB", "POS"):
+            assert torch.equal(a[l][key], b[l][key]), f"layer {l}: {key} differs"
+    # an empty list launches nothing and succeeds; a null list with entries is refused
+    assert lib.trimkv_evict_listed(tb.data_ptr(), nlayers, nseg, D, L.BF16, L.F32, 0, keep.data_ptr(), nseg, buf, cap + 1, None,
+                                   L.SCORE_ALPHA, L.ROUND_UPCAST, 0, cap, None, 0, None, 0, st) == 0
+    assert lib.trimkv_evict_listed(tb.data_ptr(), nlayers, nseg, D, L.BF16, L.F32, 0, keep.data_ptr(), nseg, buf, cap + 1, None,
+                                   L.SCORE_ALPHA, L.ROUND_UPCAST, 0, cap, None, 3, None, 0, st) < 0

@@ -46,6 +46,7 @@ SIGNATURES = {
     "trimkv_compact_threshold": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _p, _i64, _i, _i, _i,
                                       _p, _sz, _p]),
     "trimkv_evict_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _i64, _p, _i, _i, _i, _i, _p, _sz, _p]),
+    "trimkv_evict_listed": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _i, _i, _i64, _p, _i, _i, _i, _i, _p, _i, _p, _sz, _p]),
     "trimkv_compact_threshold_layers": (_i, [_p, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p, _i64, _i, _i, _i, _p, _sz, _p]),
     "trimkv_build_cu_seqlens": (_i, [_p, _i, _p, _p]),
     "trimkv_build_cu_seqlens_layers": (_i, [_p, _p, _i, _i, _p]),

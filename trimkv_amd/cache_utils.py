@@ -343,10 +343,12 @@ class _SlabBacked(_CacheBase):
         return torch.from_numpy(arr.view(np.uint8)).to(self._slabs[layers[0]].k.device)
 
     def _evict_layers(self, layers: List[int], keep: int, keep_per_seg, slack: int, strategy_code: int,
-                      rounding: int, sliding_window: int, q_idx) -> None:
+                      rounding: int, sliding_window: int, q_idx, work: Optional[np.ndarray] = None) -> None:
         """``trimkv_evict_layers`` over ``layers`` (all of one shape): one launch of nseg x len(layers) workgroups.
         ``q_idx``: the query index, one int or one per layer.  ``keep_per_seg``: None, a host array (uploaded) or a device
-        int32 tensor, ``[nseg]`` or ``[len(layers), nseg]``."""
+        int32 tensor, ``[nseg]`` or ``[len(layers), nseg]``.  ``work``: host int32 array of ``index in layers * nseg +
+        segment``: only these pairs get a workgroup (``trimkv_evict_listed``); it reaches the device through pinned memory
+        in stream order."""
         s0 = self._slabs[layers[0]]
         dev = s0.k.device
         max_len = max(self._slabs[l].max_len for l in layers)
@@ -364,11 +366,38 @@ class _SlabBacked(_CacheBase):
             stride = 0 if kdev.dim() == 1 else s0.nseg
         lib = _lib.load()
         ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, max_len), dev)
-        rc = lib.trimkv_evict_layers(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
-                                     int(keep), _lib.ptr(kdev), stride, int(slack), q_all, None, strategy_code, rounding, int(sliding_window),
-                                     max_len, _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
-        _lib.check(rc, "trimkv_evict_layers")
+        if work is not None:
+            wdev = self._upload_work(work, len(layers) * s0.nseg, dev)
+            rc = lib.trimkv_evict_listed(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                         int(keep), _lib.ptr(kdev), stride, int(slack), q_all, None, strategy_code, rounding, int(sliding_window),
+                                         max_len, wdev.data_ptr(), int(work.size), _lib.ptr(ws), 0 if ws is None else ws.numel(),
+                                         _lib.current_stream(dev))
+            _lib.check(rc, "trimkv_evict_listed")
+        else:
+            rc = lib.trimkv_evict_layers(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                         int(keep), _lib.ptr(kdev), stride, int(slack), q_all, None, strategy_code, rounding, int(sliding_window),
+                                         max_len, _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
+            _lib.check(rc, "trimkv_evict_layers")
         self._keepalive_layers = (table, kdev)   # read asynchronously by the launch
+
+    def _upload_work(self, work: np.ndarray, room: int, dev) -> torch.Tensor:
+        """A host int32 list on the device without a synchronisation: four pinned staging buffers take turns (an event per
+        buffer says when its last copy has been read), one device buffer receives them in stream order."""
+        st = getattr(self, "_work_staging", None)
+        if st is None or st[0].numel() < room or st[0].device != dev:
+            st = self._work_staging = [torch.empty(room, dtype=torch.int32, device=dev),
+                                       [torch.empty(room, dtype=torch.int32, pin_memory=True) for _ in range(4)], [None] * 4, 0]
+        wdev, host, events, which = st
+        if events[which] is not None:
+            events[which].synchronize()
+        n = int(work.size)
+        host[which][:n].numpy()[:] = work
+        wdev[:n].copy_(host[which][:n], non_blocking=True)
+        ev = events[which] or torch.cuda.Event()
+        ev.record()
+        events[which] = ev
+        st[3] = (which + 1) % 4
+        return wdev
 
     def _ensure_layer(self, layer: int) -> None:
         while len(self._slabs) <= layer:
@@ -1014,7 +1043,11 @@ class _RaggedCache(_SlabBacked):
                 kh = self._budgets_host if self._budgets_host.ndim == 1 else self._budgets_host[every]
                 keep = torch.from_numpy(np.ascontiguousarray(kh, dtype=np.int32)).to(dev)
                 self._budgets_dev[key] = keep
-            self._evict_layers(every, 0, keep, buffer_size, code, _lib.ROUND_NATIVE, 0, q_idx)
+            # With few segments due, only those get a workgroup (their list is uploaded in stream order): a launch over every
+            # (layer, segment) costs about 0.1 ms in dispatch alone when nearly all of them have nothing to do.
+            ndue = int(hit_all.sum())
+            work = np.flatnonzero(hit_all).astype(np.int32) if ndue * 4 < hit_all.size else None
+            self._evict_layers(every, 0, keep, buffer_size, code, _lib.ROUND_NATIVE, 0, q_idx, work=work)
             t = self._device_tables(every)
             rc = lib.trimkv_build_cu_seqlens_layers(t["len"].data_ptr(), t["cu"].data_ptr(), len(every), self._slabs[every[0]].nseg,
                                                     _lib.current_stream(dev))

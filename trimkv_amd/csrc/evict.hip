@@ -287,13 +287,22 @@ struct EvictArgs {
     const trimkv_layer_slabs* layers; int keep_layer_stride, thr_layer_stride;
     // query index of a layered launch: *q_idx_dev if given, else q_idx_all if positive, else the table's per-layer value
     const int64_t* q_idx_dev; int64_t q_idx_all;
+    // listed launch: workgroup i works on entry work[i] = layer * nseg + segment instead of (blockIdx.y, blockIdx.x)
+    const int32_t* work; int nlayers;
 };
 
-// blockIdx.y selects a layer: its slab addresses, capacity and query index replace the scalar fields, and the
-// per-layer parts of the other arrays are stepped to.
-__device__ __forceinline__ void select_layer(EvictArgs& a) {
-    if (!a.layers) return;
-    const int layer = blockIdx.y;
+// blockIdx.y (or the work list) selects a layer: its slab addresses, capacity and query index replace the scalar fields,
+// and the per-layer parts of the other arrays are stepped to.  Returns the workgroup's segment, -1 for a list entry that
+// names no (layer, segment) of this launch.
+__device__ __forceinline__ int select_layer(EvictArgs& a) {
+    if (!a.layers) return blockIdx.x;
+    int layer = blockIdx.y, seg = blockIdx.x;
+    if (a.work) {
+        const int item = a.work[blockIdx.x];
+        if (item < 0 || item >= a.nlayers * a.nseg) return -1;
+        layer = item / a.nseg;
+        seg = item - layer * a.nseg;
+    }
     const trimkv_layer_slabs L = a.layers[layer];
     a.k_slab = (char*)L.k_slab; a.v_slab = (char*)L.v_slab; a.lb_slab = (char*)L.lb_slab; a.pos_slab = L.pos_slab; a.seg_len = L.seg_len;
     a.q_idx = a.q_idx_dev ? *a.q_idx_dev : (a.q_idx_all > 0 ? a.q_idx_all : L.q_idx);
@@ -302,6 +311,7 @@ __device__ __forceinline__ void select_layer(EvictArgs& a) {
     if (a.tie_base) a.tie_base += (int64_t)layer * a.nseg;
     if (a.thr_key) { a.thr_key += (int64_t)layer * a.thr_layer_stride; a.tie_take += (int64_t)layer * a.thr_layer_stride; }
     if (a.ws_keys) a.ws_keys += (int64_t)layer * a.nseg * a.ws_stride;
+    return seg;
 }
 
 // SELECT = true: find the cut inside the segment (trimkv_evict).
@@ -313,8 +323,8 @@ __global__ __launch_bounds__(EV_THREADS) void evict_kernel(EvictArgs a) {
     __shared__ uint32_t scratch[EV_THREADS / 64 + 4];
     __shared__ int first_evicted;
 
-    select_layer(a);
-    const int seg = blockIdx.x;
+    const int seg = select_layer(a);
+    if (seg < 0) return;
     const int n = a.seg_len[seg];
     // nothing cached, a corrupt length, or more rows than the caller's bound (which sized the key array): touch nothing
     if (n <= 0 || n > a.cap || n > a.max_len) return;
@@ -697,9 +707,11 @@ static int lpr_shift_of(int row_bytes) {
 }
 
 template <bool SELECT>
-static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st, int nlayers = 1) {
+static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspace, size_t workspace_bytes, hipStream_t st, int nlayers = 1, int nwork = 0) {
     const size_t key_bytes = (size_t)max_len * 4;
     a.max_len = max_len;
+    a.nlayers = nlayers;
+    const dim3 grid = a.work ? dim3(nwork, 1) : dim3(a.nseg, nlayers);
     if (key_bytes <= (size_t)EV_LDS_KEY_BYTES) {
         // allow more than the default 64 KB of dynamic LDS (gfx950 has 160 KB per workgroup): once per device and
         // instantiation; the flag is only ever set, so a race repeats the call at worst
@@ -711,14 +723,14 @@ static int launch_evict(const char* fn, EvictArgs& a, int max_len, void* workspa
             if (e != hipSuccess) return fail((int)e, "%s: hipFuncSetAttribute: %s", fn, hipGetErrorString(e));
             if (dev >= 0) attr_set[dev] = true;
         }
-        hipLaunchKernelGGL((evict_kernel<true, SELECT>), dim3(a.nseg, nlayers), dim3(EV_THREADS), key_bytes, st, a);
+        hipLaunchKernelGGL((evict_kernel<true, SELECT>), grid, dim3(EV_THREADS), key_bytes, st, a);
     } else {
         const size_t need = (size_t)nlayers * a.nseg * max_len * 4;
         if (!workspace || workspace_bytes < need)
             return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed for max_len=%d, got %zu", fn, need, max_len, workspace_bytes);
         a.ws_keys = (uint32_t*)workspace;
         a.ws_stride = max_len;
-        hipLaunchKernelGGL((evict_kernel<false, SELECT>), dim3(a.nseg, nlayers), dim3(EV_THREADS), 0, st, a);
+        hipLaunchKernelGGL((evict_kernel<false, SELECT>), grid, dim3(EV_THREADS), 0, st, a);
     }
     return launch_status(fn);
 }
@@ -801,12 +813,12 @@ static int check_layer_args(const char* fn, const trimkv_layer_slabs* layers, in
     return TRIMKV_OK;
 }
 
-extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
-                                   int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
-                                   int64_t q_idx, const int64_t* q_idx_dev,
-                                   int strategy, int rounding, int sliding_window, int max_len,
-                                   void* workspace, size_t workspace_bytes, void* stream) {
-    const char* fn = "trimkv_evict_layers";
+static int evict_layers_common(const char* fn, const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                               int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                               int64_t q_idx, const int64_t* q_idx_dev,
+                               int strategy, int rounding, int sliding_window, int max_len,
+                               const int32_t* work, int nwork,
+                               void* workspace, size_t workspace_bytes, void* stream) {
     int lpr_shift;
     int rc = check_layer_args(fn, layers, nlayers, nseg, head_dim, kv_dtype, lb_dtype, max_len, &lpr_shift);
     if (rc) return rc;
@@ -821,7 +833,31 @@ extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers
     a.keep = keep; a.keep_per_seg = keep_per_seg; a.slack = slack < 0 ? 0 : slack;
     a.strategy = strategy; a.rounding = rounding; a.sliding_window = sliding_window < 0 ? 0 : sliding_window;
     a.segs_per_group = 1;
-    return launch_evict<true>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream, nlayers);
+    a.work = work;
+    return launch_evict<true>(fn, a, max_len, workspace, workspace_bytes, (hipStream_t)stream, nlayers, nwork);
+}
+
+extern "C" int trimkv_evict_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                                   int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                                   int64_t q_idx, const int64_t* q_idx_dev,
+                                   int strategy, int rounding, int sliding_window, int max_len,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+    return evict_layers_common("trimkv_evict_layers", layers, nlayers, nseg, head_dim, kv_dtype, lb_dtype, keep, keep_per_seg, keep_layer_stride,
+                               slack, q_idx, q_idx_dev, strategy, rounding, sliding_window, max_len, nullptr, 0, workspace, workspace_bytes, stream);
+}
+
+extern "C" int trimkv_evict_listed(const trimkv_layer_slabs* layers, int nlayers, int nseg, int head_dim, int kv_dtype, int lb_dtype,
+                                   int keep, const int32_t* keep_per_seg, int keep_layer_stride, int slack,
+                                   int64_t q_idx, const int64_t* q_idx_dev,
+                                   int strategy, int rounding, int sliding_window, int max_len,
+                                   const int32_t* work, int nwork,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_evict_listed";
+    if (nwork == 0) return TRIMKV_OK;
+    if (!work) return fail(TRIMKV_ERR_NULL, "%s: null work list", fn);
+    if (nwork < 0) return fail(TRIMKV_ERR_SHAPE, "%s: nwork=%d", fn, nwork);
+    return evict_layers_common(fn, layers, nlayers, nseg, head_dim, kv_dtype, lb_dtype, keep, keep_per_seg, keep_layer_stride,
+                               slack, q_idx, q_idx_dev, strategy, rounding, sliding_window, max_len, work, nwork, workspace, workspace_bytes, stream);
 }
 
 extern "C" int trimkv_compact_threshold_layers(const trimkv_layer_slabs* layers, int nlayers, int nseg, int segs_per_group, int head_dim,
