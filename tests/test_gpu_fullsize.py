@@ -213,11 +213,15 @@ def test_config3_all_36_layers_evicted_by_one_launch():
         assert torch.equal(K[ok], k.gather(2, idx)[ok]) and torch.equal(V[ok], v.gather(2, idx)[ok])
 
 
-def test_config4_ragged_lognormal_budgets():
+@pytest.mark.parametrize("fused", [False, True])
+def test_config4_ragged_lognormal_budgets(fused):
     """B=32, 8 KV heads, G=4; per-head budgets lognormal(median 1024, sigma 1) clipped to [64, 8192],
-    prompt lengths U[512, 16384] per batch element; decode steps with per-head eviction at budget + 128."""
+    prompt lengths U[512, 16384] per batch element; decode steps with per-head eviction at budget + 128.
+    ``fused``: two layers, the append carried out by the attention launch (planned piece lists), evictions of both layers in
+    one launch (over every pair, or over the list of due pairs when few are due).  Attention is checked on every segment."""
     from trimkv_amd import BatchedDynamicBudgetTrimKVCache, get_attention_interface
     B, H, G, buf = 32, 8, 4, 128
+    L = 2 if fused else 1
     rng = np.random.default_rng(4)
     budgets = np.clip(np.round(np.exp(rng.normal(np.log(1024), 1.0, size=B * H))), 64, 8192).astype(np.int64)
     prompt = rng.integers(512, 16385, size=B)
@@ -225,45 +229,55 @@ def test_config4_ragged_lognormal_budgets():
     S = int(start.max())
     gen = torch.Generator(device=DEV).manual_seed(4)
     cache = BatchedDynamicBudgetTrimKVCache()
-    k = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
-    v = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    cache.fuse_decode_append = fused
     lb = torch.nn.functional.logsigmoid(torch.randn(B, H, S, generator=gen, device=DEV) * 1.5 + 3.0)
-    cache.update(k, v, lb, torch.arange(S, device=DEV), 0)
+    for l in range(L):
+        k = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        v = torch.randn(B, H, S, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        cache.update(k, v, lb, torch.arange(S, device=DEV), l)
+    del k, v
     cache.set_budgets(start)
     cache.evict_to_budgets(buffer_size=0)                     # ragged initial state
-    assert cache.head_lens[0].cpu().tolist() == start.tolist()
-    pos0 = cache.segment_positions()[0]
     sc = lb.float() * (S + 1 - torch.arange(S, device=DEV))
-    for seg in rng.choice(B * H, 24, replace=False):           # kept set = top-start[seg] of the prompt, in order
-        want = torch.sort(torch.topk(sc.view(B * H, S)[seg], int(start[seg])).indices).values.cpu()
-        assert torch.equal(pos0[seg], want)
+    for l in range(L):
+        assert cache.head_lens[l].cpu().tolist() == start.tolist()
+        pos0 = cache.segment_positions()[l]
+        for seg in rng.choice(B * H, 24, replace=False):       # kept set = top-start[seg] of the prompt, in order
+            want = torch.sort(torch.topk(sc.view(B * H, S)[seg], int(start[seg])).indices).values.cpu()
+            assert torch.equal(pos0[seg], want)
     cache.set_budgets(budgets)
     attn = get_attention_interface("db_attn_flash_batched")
     lens = start.copy()
     for t in range(140):
-        kn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
-        vn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
-        lbn = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) * 1.5 + 3.0)
-        K, V, _, _, kw = cache.update(kn, vn, lbn, torch.arange(S + t, S + t + 1, device=DEV), 0)
+        check = t % 35 == 0
+        for l in range(L):
+            kn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+            vn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+            lbn = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) * 1.5 + 3.0)
+            K, V, _, _, kw = cache.update(kn, vn, lbn, torch.arange(S + t, S + t + 1, device=DEV), l)
+            if check or fused:                                # a deferred append is carried out by the attention call
+                q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+                out, _, _ = attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw)
+            if check:
+                slab = cache._slabs[l]
+                worst = 0.0
+                for seg in range(B * H):
+                    n = int(lens[seg]) + 1
+                    kk, vv = slab.k[seg, :n].float(), slab.v[seg, :n].float()
+                    p = torch.softmax(q.view(B * H, G, 128)[seg].float() @ kk.T * 128 ** -0.5, -1)
+                    ok, err = attn_close(out.view(B * H, G, 128)[seg], p @ vv)
+                    assert ok, (l, seg, err)
         lens += 1
-        if t % 35 == 0:
-            q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
-            out, _, _ = attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw)
-            slab = cache._slabs[0]
-            for seg in (0, 37, 101, 255):
-                n = int(lens[seg])
-                kk, vv = slab.k[seg, :n].float(), slab.v[seg, :n].float()
-                p = torch.softmax(q.view(B * H, G, 128)[seg].float() @ kk.T * 128 ** -0.5, -1)
-                ok, err = attn_close(out.view(B * H, G, 128)[seg], p @ vv)
-                assert ok, (seg, err)
         cache.evict_to_budgets(buffer_size=buf)
         hit = (lens > budgets) & (lens >= budgets + buf)
         lens = np.where(hit, budgets, lens)
-        assert cache._slabs[0].lens.tolist() == lens.tolist()
-    assert cache.head_lens[0].cpu().tolist() == lens.tolist()
-    assert cache.cu_seqlens_k[0].cpu().tolist() == [0] + np.cumsum(lens).tolist()
-    for seg, p in enumerate(cache.segment_positions()[0]):
-        assert p.numel() == lens[seg] and (p[1:] > p[:-1]).all()
+        for l in range(L):
+            assert cache._slabs[l].lens.tolist() == lens.tolist()
+    for l in range(L):
+        assert cache.head_lens[l].cpu().tolist() == lens.tolist()
+        assert cache.cu_seqlens_k[l].cpu().tolist() == [0] + np.cumsum(lens).tolist()
+        for seg, p in enumerate(cache.segment_positions()[l]):
+            assert p.numel() == lens[seg] and (p[1:] > p[:-1]).all()
     assert hit.sum() == 0 and (lens <= budgets + buf).all()
 
 
