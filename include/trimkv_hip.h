@@ -349,6 +349,11 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
  * append (<= cap); a segment whose slab is full is left as it is and attends its old rows.  chunk, workspace (size:
  * trimkv_decode_attn_workspace(nseg, group, head_dim, max_len_after, chunk)) and seg_order as in trimkv_decode_attn; when
  * segments are split the lengths are advanced by the merge launch.
+ * gate_part / gate_nslice / gate_bias: when gate_part is given, the new row's log beta is not read from lb_new (which may
+ * then be null) but finished here from the retention gate's partial sums, exactly as trimkv_append_gated does for one new
+ * token per sequence: log beta[b][h] = logsigmoid(sum over slices of gate_part[slice][b][h] + gate_bias[h]), rounded
+ * where a module in lb_dtype rounds (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:171-179).  gate_part is
+ * [gate_nslice][batch][kv_heads] fp32 as trimkv_gate_hidden writes it, gate_nslice <= 64.  Pass null, 0, null otherwise.
  */
 int trimkv_append_attend(const void* q, void* out,
                          void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
@@ -357,6 +362,7 @@ int trimkv_append_attend(const void* q, void* out,
                          const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
                          const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
                          const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                         const float* gate_part, int gate_nslice, const float* gate_bias,
                          float scale, int max_len_after, int chunk,
                          void* workspace, size_t workspace_bytes, void* stream);
 
@@ -401,6 +407,7 @@ int trimkv_append_attend_pieces(const void* q, void* out,
                                 const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
                                 const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
                                 const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                const float* gate_part, int gate_nslice, const float* gate_bias,
                                 float scale, int max_len_after,
                                 void* workspace, size_t workspace_bytes, void* stream);
 

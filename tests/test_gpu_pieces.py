@@ -169,7 +169,7 @@ def test_append_attend_pieces_equals_append_then_attend():
         L.check(lib.trimkv_append_attend_pieces(q.data_ptr(), got.data_ptr(), b["k"].data_ptr(), b["v"].data_ptr(), b["lb"].data_ptr(), b["pos"].data_ptr(),
                                                 b["seg_len"].data_ptr(), b["cu"].data_ptr(), plist.data_ptr(), npieces, nseg, H, cap, D, G, L.BF16, L.F32,
                                                 kn.data_ptr(), vn.data_ptr(), kn.stride(0), kn.stride(1), lbn.data_ptr(), lbn.stride(0), lbn.stride(1),
-                                                posn.data_ptr(), 0, 0, D ** -0.5, cap, ws_b.data_ptr(), ws_b.numel(), st), "append_attend_pieces")
+                                                posn.data_ptr(), 0, 0, None, 0, None, D ** -0.5, cap, ws_b.data_ptr(), ws_b.numel(), st), "append_attend_pieces")
         torch.cuda.synchronize()
         assert torch.equal(got, want)
         lens = np.where(lens < cap, lens + 1, lens)
