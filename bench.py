@@ -296,6 +296,13 @@ def ragged_main(args):
               torch.randn(B, Hkv, 1, D, generator=gen, device=dev).to(torch.bfloat16), draw_lb(B, Hkv, 1),
               torch.randn(B, Hq, 1, D, generator=gen, device=dev).to(torch.bfloat16)) for _ in range(POOL)] for _ in range(L)]
     torch.cuda.synchronize()
+    if args.calibrate_copy:  # 2**30 bytes read + 2**30 bytes written by one elementwise kernel
+        src = torch.empty(2 ** 28, dtype=torch.float32, device=dev).normal_()
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        torch.add(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     T = S0
     events, step_bytes = [], []
 
