@@ -54,11 +54,11 @@ def algorithmic_bytes(c):
     return dict(attn=attn_kv + attn_qo, append=append, evict=evict, step=c["L"] * (attn_kv + attn_qo + append + evict))
 
 
-def measured_traffic_ratio():
+def measured_traffic_ratio(config=3):
     """HBM bytes per attention launch over algorithmic bytes, as measured with rocprofv3 --pmc
     FETCH_SIZE / WRITE_SIZE (scaled by a copy kernel of known size); the summary of those two runs
     is committed under profiles/ and carries the ratio on a `traffic_over_algorithmic:` line."""
-    path = os.path.join(ROOT, "profiles", "decode_attn_config3_pmc_traffic.md")
+    path = os.path.join(ROOT, "profiles", f"decode_attn_config{config}_pmc_traffic.md")
     try:
         for line in open(path):
             if line.startswith("traffic_over_algorithmic:"):
@@ -362,8 +362,10 @@ def ragged_main(args):
         avg_s = sum(e0.elapsed_time(e1) for e0, e1, _ in events) * 1e-3 / len(events)
         avg_b = sum(n * 2 * D * 2 + nseg * 2 * G * D * 2 for _, _, n in events) / len(events)
         targs = f"<{G}, 16, false, {'true' if cache.fuse_decode_append else 'false'}>"
+        ratio, src = measured_traffic_ratio(4) if cache.fuse_decode_append else (None, None)
         roof = {"bound": "hbm", "kernel": f"decode_attn_pieces_kernel{targs}", "achieved": round(avg_b / avg_s / 1e9, 1),
-                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(avg_b / avg_s / 1e9 / HBM_PEAK_GBS, 4), "traffic": None,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(avg_b / avg_s / 1e9 / HBM_PEAK_GBS, 4),
+                "traffic": None if ratio is None else int(avg_b * ratio), "traffic_source": src, "traffic_measured_in_run": False,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(events), "algorithmic_bytes_per_launch": int(avg_b)}
     out_json = {
         "metric": "decode tokens/s (ragged append + varlen attn + per-head evict), Qwen3-4B shape", "value": round(B * args.steps / seconds, 1),
