@@ -582,7 +582,7 @@ def main():
         durs = [e0.elapsed_time(e1) * 1e-3 for e0, e1, _ in events]
         lens = [n for _, _, n in events]
         avg_s = sum(durs) / len(durs)
-        fused = cache.fuse_decode_append   # the sampled launch then also writes the new rows (and finishes the gate, with --gate)
+        fused = cache.fuse_decode_append and not args.gate   # the sampled launch then also writes the new rows
         avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens) + (append_bytes if fused else 0)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
@@ -614,10 +614,8 @@ def main():
                                f"head_dim {D}, memory_size {M}, buffer_size {buf}, steady-state decode (append + attend per layer, "
                                f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
                    "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(),
-                   "launches_per_layer_step": (("2: trimkv_gate_hidden, then gate epilogue + append + attend in one launch (trimkv_append_attend)" if args.gate
-                                                else "1: append + attend in one launch (trimkv_append_attend)") if cache.fuse_decode_append
-                                               else ("3: trimkv_gate_hidden, trimkv_append_gated, trimkv_decode_attn" if args.gate
-                                                     else "2: trimkv_append, trimkv_decode_attn")) + ("" if B * Hkv >= 256 else " + split-K merge"),
+                   "launches_per_layer_step": ("1: append + attend in one launch (trimkv_append_attend)" if cache.fuse_decode_append and not args.gate
+                                               else "2: trimkv_append, trimkv_decode_attn") + ("" if B * Hkv >= 256 else " + split-K merge"),
                    **timing},
         "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
                      "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),

@@ -349,11 +349,6 @@ int trimkv_decode_attn(const void* q, void* out, const void* k_slab, const void*
  * append (<= cap); a segment whose slab is full is left as it is and attends its old rows.  chunk, workspace (size:
  * trimkv_decode_attn_workspace(nseg, group, head_dim, max_len_after, chunk)) and seg_order as in trimkv_decode_attn; when
  * segments are split the lengths are advanced by the merge launch.
- * gate_part / gate_nslice / gate_bias: when gate_part is given, the new row's log beta is not read from lb_new (which may
- * then be null) but finished here from the retention gate's partial sums, exactly as trimkv_append_gated does for one new
- * token per sequence: log beta[b][h] = logsigmoid(sum over slices of gate_part[slice][b][h] + gate_bias[h]), rounded
- * where a module in lb_dtype rounds (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:171-179).  gate_part is
- * [gate_nslice][batch][kv_heads] fp32 as trimkv_gate_hidden writes it, gate_nslice <= 64.  Pass null, 0, null otherwise.
  */
 int trimkv_append_attend(const void* q, void* out,
                          void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
@@ -362,7 +357,6 @@ int trimkv_append_attend(const void* q, void* out,
                          const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
                          const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
                          const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
-                         const float* gate_part, int gate_nslice, const float* gate_bias,
                          float scale, int max_len_after, int chunk,
                          void* workspace, size_t workspace_bytes, void* stream);
 
@@ -407,7 +401,6 @@ int trimkv_append_attend_pieces(const void* q, void* out,
                                 const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
                                 const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
                                 const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
-                                const float* gate_part, int gate_nslice, const float* gate_bias,
                                 float scale, int max_len_after,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
@@ -420,11 +413,14 @@ int trimkv_append_attend_pieces(const void* q, void* out,
  * Every compute unit gets total_rows / compute_units rows in at most two pieces: segments no longer than that stay
  * whole, the longer ones are cut where a compute unit is full (pieces of different sizes, given as fractions).  Gaps
  * and slivers of fewer than min_rows rows are not worth a piece (64 is a good value).  With fewer than 2*min_rows rows
- * per compute unit, or more short segments than compute units, the list is simply every segment whole, longest first.
+ * per compute unit the list is every segment whole, longest first; with more short segments than compute units (a unit
+ * would need three pieces) the segments longer than a unit's share are cut into equal pieces and the list runs longest
+ * first, its second compute_units entries shortest first when everything fits 2*compute_units entries (entry i +
+ * compute_units then pairs the i-th shortest piece with the i-th longest).
  * seg_len: the lengths the launch will see, or close to them (the kernel scales the cuts to the lengths it finds);
  * for trimkv_append_attend_pieces either the lengths before or after the append.  Copy the result to the device
  * (16-byte aligned) and reuse it until the lengths have moved by a few per cent.
- * Returns the number of entries written (>= nseg, <= nseg + 2*compute_units), or a negative trimkv_status:
+ * Returns the number of entries written (>= nseg, <= 2*nseg + 2*compute_units), or a negative trimkv_status:
  * TRIMKV_ERR_WORKSPACE when max_pieces entries are too few.
  */
 int trimkv_plan_attn_pieces(const int32_t* seg_len, int nseg, int compute_units, int min_rows,

@@ -212,7 +212,7 @@ def test_c_abi_append_attend_other_shapes_full_slabs_and_cu(D, dtype, lb_dtype):
         L.check(lib.trimkv_append_attend(q.data_ptr(), got.data_ptr(), b["k"].data_ptr(), b["v"].data_ptr(), b["lb"].data_ptr(), b["pos"].data_ptr(),
                                          b["seg_len"].data_ptr(), b["cu"].data_ptr(), None, nseg, H, cap, D, G, code, lcode,
                                          kn.data_ptr(), vn.data_ptr(), kn.stride(0), kn.stride(1), lbn.data_ptr(), lbn.stride(0), lbn.stride(1),
-                                         posn.data_ptr(), 0, 0, None, 0, None, scale, cap, chunk, ws.data_ptr(), ws.numel(), st), "append_attend")
+                                         posn.data_ptr(), 0, 0, scale, cap, chunk, ws.data_ptr(), ws.numel(), st), "append_attend")
         torch.cuda.synchronize()
         assert torch.equal(got, want)
         after = np.where(lens < cap, lens + 1, lens)

@@ -59,51 +59,6 @@ def test_append_gated_writes_the_same_log_beta_as_materialize():
     assert cache_a.get_cache_length(0) == 7
 
 
-@pytest.mark.parametrize("ragged,G", [(False, 4), (False, 5), (True, 4), (True, 6)])
-def test_fused_step_finishes_the_gate_in_the_attention_launch(ragged, G):
-    """With fuse_decode_append the lazy gate output is finished by the attention launch (sum of the slices, bias, logsigmoid,
-    rounding, store): state and attention output must equal the cache that runs trimkv_append_gated and attends separately."""
-    from trimkv_amd import TrimKVCache, BatchedDynamicBudgetTrimKVCache, get_attention_interface
-    B, H, hidden, D = 4, 8, 2048, 128
-    g = _gate(hidden, H, std=0.05).to(DEV)
-    gen = torch.Generator().manual_seed(3)
-    cls = BatchedDynamicBudgetTrimKVCache if ragged else TrimKVCache
-    attn = get_attention_interface("db_attn_flash_batched" if ragged else "trimkv_hip")
-
-    class Mod:
-        training = False
-        num_key_value_groups = G
-
-    caches = [cls(), cls()]
-    caches[1].fuse_decode_append = True
-    T = 0
-    for step, S in enumerate((700, 1, 1, 1, 1, 1)):
-        x = torch.randn(B, S, hidden, generator=gen).to(torch.bfloat16).to(DEV)
-        k, v = draw_kv(gen, B, H, S)
-        q = torch.randn(B, H * G, S, D, generator=gen).to(torch.bfloat16).to(DEV)
-        pos = torch.arange(T, T + S, device=DEV)
-        outs = []
-        for c in caches:
-            lazy = g(x).transpose(1, 2)
-            K, V, _, _, kw = c.update(k.to(DEV), v.to(DEV), lazy, pos, 0)
-            if S == 1:
-                assert (c._slabs[0].pending is not None) == c.fuse_decode_append
-                out = attn(Mod, q, K, V, None, **({"flash_attn_kwargs": kw} if kw else {}))[0]
-                outs.append(out)
-        T += S
-        if outs:
-            assert torch.equal(outs[0], outs[1]), f"step {step}"
-        a, b = caches[0]._slabs[0], caches[1]._slabs[0]
-        assert b.pending is None and a.lens.tolist() == b.lens.tolist()
-        assert torch.equal(a.seg_len, b.seg_len)
-        for name in ("key_cache", "value_cache", "retention_weights", "kv_positions"):      # the live rows
-            assert torch.equal(getattr(caches[0], name)[0], getattr(caches[1], name)[0]), (step, name)
-        if ragged and step == 2:
-            for c in caches:
-                c.set_budgets([600 - 7 * i for i in range(B * H)])
-                c.evict_to_budgets(buffer_size=0)
-
-
 @pytest.mark.parametrize("kind", ["rg2", "rg3"])
 @pytest.mark.parametrize("B,S,H", [(64, 1, 8), (2, 70, 4), (1, 300, 8)])
 def test_kv_gates_match_oracle(kind, B, S, H):

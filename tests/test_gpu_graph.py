@@ -128,7 +128,7 @@ def test_decode_step_including_eviction_replays_from_a_hip_graph():
             L.check(lib.trimkv_append_attend(qin[l].data_ptr(), state["out"][l].data_ptr(), s["K"].data_ptr(), s["V"].data_ptr(), s["LB"].data_ptr(),
                                              s["POS"].data_ptr(), s["LEN"].data_ptr(), None, None, nseg, H, cap, D, G, L.BF16, L.F32,
                                              k.data_ptr(), v.data_ptr(), k.stride(0), k.stride(1), lb.data_ptr(), lb.stride(0), lb.stride(1),
-                                             posin.data_ptr(), 0, 0, None, 0, None, D ** -0.5, cap, 0, ws.data_ptr(), ws.numel(), stream), "append_attend")
+                                             posin.data_ptr(), 0, 0, D ** -0.5, cap, 0, ws.data_ptr(), ws.numel(), stream), "append_attend")
         L.check(lib.trimkv_evict_layers(state["table"].data_ptr(), nlayers, nseg, D, L.BF16, L.F32, M, None, 0, buf, 0, state["q"].data_ptr(),
                                         L.SCORE_ALPHA, L.ROUND_UPCAST, 0, cap, None, 0, stream), "evict_layers")
 

@@ -16,7 +16,7 @@ FR = 32768
 def _plan(lens, ncu=256, min_rows=64, room=None):
     lib = _lib.load()
     lens = np.ascontiguousarray(lens, dtype=np.int32)
-    room = lens.size + 2 * ncu if room is None else room
+    room = 2 * lens.size + 2 * ncu if room is None else room
     out = np.full((max(room, 1), 4), -1, dtype=np.int32)
     n = lib.trimkv_plan_attn_pieces(lens.ctypes.data, lens.size, ncu, min_rows, out.ctypes.data, room)
     return n, out
@@ -88,14 +88,39 @@ def test_every_compute_unit_gets_the_same_rows(seed):
     _check_cover(lens, entries, scale_to=drift)
 
 
-def test_short_totals_and_many_short_segments_fall_back_to_whole_segments():
+def test_short_totals_keep_segments_whole_longest_first():
     rng = np.random.default_rng(1)
-    for lens in (rng.integers(0, 40, size=100), np.concatenate([rng.integers(1, 50, size=400), [60000]])):
-        n, out = _plan(lens)
-        assert n == len(lens)
-        _check_cover(np.asarray(lens), out[:n])
-        rows = [int(lens[e[0]]) for e in out[:n]]
-        assert rows == sorted(rows, reverse=True)
+    lens = rng.integers(0, 40, size=100)
+    n, out = _plan(lens)
+    assert n == len(lens)
+    _check_cover(np.asarray(lens), out[:n])
+    rows = [int(lens[e[0]]) for e in out[:n]]
+    assert rows == sorted(rows, reverse=True)
+
+
+@pytest.mark.parametrize("nseg,seed", [(400, 0), (512, 1), (2000, 2)])
+def test_more_short_segments_than_compute_units(nseg, seed):
+    """More than one segment per compute unit: long segments are cut into equal pieces of at most a unit's share, the list
+    runs longest first, and while everything is resident (<= 512 entries) its second half runs shortest first, so the
+    pair of a compute unit is (i-th longest, i-th shortest)."""
+    rng = np.random.default_rng(seed)
+    lens = _lognormal(rng, nseg)
+    lens[3] = 60000
+    n, out = _plan(lens)
+    entries = out[:n]
+    _check_cover(lens, entries)
+    S = -(-int(lens.sum()) // 256)
+    rows = np.array([_rows(e, int(lens[e[0]]))[3] - _rows(e, int(lens[e[0]]))[2] for e in entries])
+    assert rows.max() <= S + 1
+    slack = 32                                   # the last of a segment's equal pieces is a few rows shorter than the rest
+    assert (np.diff(rows[:256]) <= slack).all()
+    if n <= 512:
+        assert (np.diff(rows[256:]) >= -slack).all()
+        pair = rows[:256].astype(np.int64)
+        pair[: n - 256] += rows[256:]
+        assert pair.max() <= 1.35 * pair.mean()
+    else:
+        assert (np.diff(rows) <= slack).all()
 
 
 def test_empty_segments_and_one_giant_segment():

@@ -199,21 +199,12 @@ class _SlabBacked(_CacheBase):
         (``_flush``).  Returns False when this update cannot be deferred (the ordinary append runs then)."""
         if slab.pending is not None:
             self._flush(slab)
+        if isinstance(lb, LazyLogBeta) or not (k.is_cuda and lb.is_cuda):
+            return False
         B, H, D = slab.B, slab.H, slab.D
-        if not k.is_cuda or tuple(k.shape) != (B, H, 1, D) or v.shape != k.shape or v.dtype != k.dtype or k.dtype != slab.k.dtype:
+        if tuple(k.shape) != (B, H, 1, D) or v.shape != k.shape or v.dtype != k.dtype or k.dtype != slab.k.dtype:
             return False
         if tuple(lb.shape) != (B, H, 1) or lb.dtype != slab.lb.dtype:
-            return False
-        if isinstance(lb, LazyLogBeta):
-            # the attention launch also finishes the gate: per-slice partial sums [slices, B, Hkv] + bias -> log beta
-            if not lb.transposed or lb.part.shape[0] > 64 or not lb.part.is_contiguous():
-                return False
-            lb_args = (0, 0, 0)
-            gate = (lb.part.data_ptr(), int(lb.part.shape[0]), lb.bias_f32.data_ptr())
-        elif lb.is_cuda:
-            lb_args = (lb.data_ptr(), lb.stride(0), lb.stride(1))
-            gate = (None, 0, None)
-        else:
             return False
         ks = k.stride()
         if ks[3] != 1 or (ks[0] | ks[1]) % 8 or v.stride() != ks or (k.data_ptr() | v.data_ptr()) % 16:
@@ -230,7 +221,7 @@ class _SlabBacked(_CacheBase):
             slab.regrow(self._new_capacity(slab, slab.max_len + 1, 1))
         # [0]: what trimkv_append_attend needs of the new row (addresses, element strides over batch and head);
         # [1:]: the tensors themselves, kept alive and used by _flush
-        slab.pending = ((k.data_ptr(), v.data_ptr(), ks[0], ks[1], *lb_args, pos.data_ptr(), ps[0], ps[1], *gate),
+        slab.pending = ((k.data_ptr(), v.data_ptr(), ks[0], ks[1], lb.data_ptr(), lb.stride(0), lb.stride(1), pos.data_ptr(), ps[0], ps[1]),
                         k, v, lb, pos)
         slab.lens += 1
         slab.max_len += 1
@@ -721,7 +712,7 @@ class _RaggedCache(_SlabBacked):
         # ``cache_kwargs={"packed": True}`` on a call, it returns the reference's packed ``[sum(n), D]`` tensors instead.
         self.return_packed = False
         self.attention_pieces = 400   # grid-split fallback only: about this many pieces per decode-attention launch
-        self.attention_compute_units = 256   # what the piece lists of the decode-attention launches are balanced for (MI355X)
+        self.attention_compute_units = 0     # what the piece lists of the decode-attention launches are balanced for; 0: ask the device
         self.attention_replan_steps = 32     # a layer's piece list is rebuilt at least this often
         self._replans = 0
 
@@ -810,7 +801,9 @@ class _RaggedCache(_SlabBacked):
         if nseg > 8192:
             slab.pieces = None
             return None
-        room = nseg + 2 * self.attention_compute_units
+        if not self.attention_compute_units:
+            self.attention_compute_units = int(torch.cuda.get_device_properties(slab.k.device).multi_processor_count)
+        room = 2 * nseg + 2 * self.attention_compute_units
         buf = slab.pieces_buf
         if buf is None or buf[0].shape[0] < room:
             dev = torch.empty(room, 4, dtype=torch.int32, device=slab.k.device)

@@ -110,28 +110,7 @@ struct AppendPart {
     const int64_t* pos_new; int64_t pos_sb, pos_sh;
     void* lb_slab; int64_t* pos_slab; int32_t* seg_len; int32_t* cu;
     int kv_heads, lb_dtype;
-    // optional: log beta of the new row from the retention gate's partial sums [gate_nslice][batch][kv_heads] (fp32) + bias
-    const float* gate_part; const float* gate_bias; int gate_nslice, gate_ntok;
 };
-
-// logsigmoid the way the gated append computes it: min(x, 0) - log1p(exp(-|x|))
-__device__ __forceinline__ float attn_log_sigmoid(float x) { return fminf(x, 0.0f) - log1pf(__expf(-fabsf(x))); }
-
-// log beta of this step's token of (batch b, kv head h), in two parts so that the load can be issued early and its
-// result used late.  Load: the caller's value, or this lane's slice of the retention gate's partial sums.  Finish (all 64
-// lanes of a wavefront together): nothing, or the gate's epilogue -- a fixed butterfly over the lanes, bias, logsigmoid,
-// rounded where a module in the slab's dtype rounds; the order trimkv_append_gated uses, so both give the same bits.
-__device__ __forceinline__ float new_log_beta_load(const AppendPart& ap, int b, int h, int64_t lb_off, int lane) {
-    if (!ap.gate_part) return load_as_f32(ap.lb_new, lb_off, ap.lb_dtype);
-    return lane < ap.gate_nslice ? ap.gate_part[((int64_t)lane * ap.gate_ntok + b) * ap.kv_heads + h] : 0.0f;
-}
-__device__ __forceinline__ float new_log_beta_finish(const AppendPart& ap, int h, float acc) {
-    if (!ap.gate_part) return acc;
-#pragma unroll
-    for (int d = 32; d > 0; d >>= 1) acc += __shfl_xor(acc, d, 64);
-    acc = round_to_dtype(acc, ap.lb_dtype);
-    return attn_log_sigmoid(round_to_dtype(acc + ap.gate_bias[h], ap.lb_dtype));
-}
 
 struct AttnArgs {
     const uint4* q; void* out; const uint4* k; const uint4* v;
@@ -240,7 +219,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         if (APPEND_EARLY) {
             kn = *knew;
             vn = *vnew;
-            lbn = new_log_beta_load(a.ap, b, h, lb_off, lane);
+            lbn = load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype);
             pn = a.ap.pos_new[pos_off];
         }
     }
@@ -410,7 +389,6 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
                 ((uint4*)a.k)[dst * ROW16 + c] = kn;
                 ((uint4*)a.v)[dst * ROW16 + c] = vn;
             }
-            lbn = new_log_beta_finish(a.ap, seg % a.ap.kv_heads, lbn);
             if (lane == 0) {
                 store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
                 a.ap.pos_slab[dst] = pn;
@@ -443,10 +421,8 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             ((uint4*)a.k)[dst * ROW16 + c] = kn;
             ((uint4*)a.v)[dst * ROW16 + c] = vn;
         }
-        const int bb = seg / a.ap.kv_heads;
-        const float lb_late = new_log_beta_finish(a.ap, seg - bb * a.ap.kv_heads, new_log_beta_load(a.ap, bb, seg - bb * a.ap.kv_heads, lb_off, lane));
         if (lane == 0) {
-            store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lb_late);
+            store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype));
             a.ap.pos_slab[dst] = a.ap.pos_new[pos_off];
         }
     }

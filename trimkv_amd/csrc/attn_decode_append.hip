@@ -18,19 +18,17 @@ extern "C" int trimkv_append_attend(const void* q, void* out,
                                     const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
                                     const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
                                     const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
-                                    const float* gate_part, int gate_nslice, const float* gate_bias,
                                     float scale, int max_len_after, int chunk,
                                     void* workspace, size_t workspace_bytes, void* stream) {
     const char* fn = "trimkv_append_attend";
-    int rc = check_append_args(fn, lb_slab, pos_slab, seg_len, k_new, v_new, lb_new, pos_new, nseg, kv_heads, lb_dtype, kv_stride_b, kv_stride_h,
-                               gate_part, gate_nslice, gate_bias);
+    int rc = check_append_args(fn, lb_slab, pos_slab, seg_len, k_new, v_new, lb_new, pos_new, nseg, kv_heads, lb_dtype, kv_stride_b, kv_stride_h);
     if (rc) return rc;
     AttnArgs a;
     rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, seg_order, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
                       max_len_after, chunk, workspace, workspace_bytes);
     if (rc) return rc;
     fill_append_part(fn, a, lb_slab, pos_slab, seg_len, cu_seqlens, nseg, kv_heads, lb_dtype, k_new, v_new, kv_stride_b, kv_stride_h,
-                     lb_new, lb_stride_b, lb_stride_h, pos_new, pos_stride_b, pos_stride_h, gate_part, gate_nslice, gate_bias);
+                     lb_new, lb_stride_b, lb_stride_h, pos_new, pos_stride_b, pos_stride_h);
     launch_attn_group<true>(a, group, head_dim, kv_dtype, (hipStream_t)stream);
     return launch_status(fn);
 }

@@ -11,6 +11,8 @@
 //     the segment's tail together with the head of the next long segment.
 // Rows that find no room (gaps too small to be worth a piece were left open) become extra pieces at the end of the list:
 // the hardware starts them wherever a workgroup finishes first.
+// More short segments than compute units (more than one segment per unit on average) is a different problem: see the
+// fallback at the top of the function.
 #include "common.hip.h"
 
 #include <algorithm>
@@ -56,13 +58,30 @@ extern "C" int trimkv_plan_attn_pieces(const int32_t* seg_len, int nseg, int com
     int nshort = 0;
     for (int s = 0; s < nseg; ++s) nshort += seg_len[s] > 0 && seg_len[s] <= S;
     if (S < 2 * (int64_t)min_rows || nshort > ncu) {
-        // too few rows to be worth cutting, or more short segments than compute units: whole segments, longest first
-        if (nseg > max_pieces) return fail(TRIMKV_ERR_WORKSPACE, "%s: %d pieces needed, room for %d", fn, nseg, max_pieces);
-        for (int i = 0; i < nseg; ++i) {
-            int32_t* e = pieces + 4 * (size_t)i;
-            e[0] = order[i]; e[1] = 0; e[2] = 1; e[3] = i;
+        // Too few rows to be worth planning, or more short segments than compute units (a unit would need three pieces):
+        // segments longer than S are cut into equal pieces of at most S rows, and the pieces go out longest first.  When
+        // they all fit the resident set (2 per compute unit) the second half of the list runs shortest first, so that
+        // entry i + compute_units pairs the i-th shortest piece with the i-th longest.
+        struct Piece { int seg, idx, cnt, rows; };
+        std::vector<Piece> ps;
+        std::vector<int> first_slot(nseg);
+        int total_pieces = 0;
+        for (int s = 0; s < nseg; ++s) {
+            const int n = seg_len[s];
+            int cnt = (S >= 2 * (int64_t)min_rows && n > S) ? (int)((n + S - 1) / S) : 1;
+            if (cnt > 0xffff) cnt = 0xffff;
+            first_slot[s] = total_pieces;
+            total_pieces += cnt;
+            for (int i = 0; i < cnt; ++i) ps.push_back(Piece{s, i, cnt, (n + cnt - 1) / cnt});
         }
-        return nseg;
+        if (total_pieces > max_pieces) return fail(TRIMKV_ERR_WORKSPACE, "%s: %d pieces needed, room for %d", fn, total_pieces, max_pieces);
+        std::stable_sort(ps.begin(), ps.end(), [](const Piece& x, const Piece& y) { return x.rows > y.rows; });
+        if (total_pieces > ncu && total_pieces <= 2 * ncu) std::reverse(ps.begin() + ncu, ps.end());
+        for (int i = 0; i < total_pieces; ++i) {
+            int32_t* e = pieces + 4 * (size_t)i;
+            e[0] = ps[i].seg; e[1] = ps[i].idx; e[2] = ps[i].cnt; e[3] = first_slot[ps[i].seg];   // bounds 0: equal pieces
+        }
+        return total_pieces;
     }
 
     struct Gap { int64_t room; int unit; };
