@@ -123,7 +123,7 @@ def test_a_deferred_append_is_carried_out_by_whatever_touches_the_layer_first():
     assert fused.get_seq_length() == plain.get_seq_length() == T
 
 
-@pytest.mark.parametrize("G", [2, 4])
+@pytest.mark.parametrize("G", [2, 4, 5, 6, 8])
 def test_ragged_fused_step_equals_separate_launches(G):
     """Per-head budgets (config-4 style): lengths differ by 50x, segments are split and dispatched longest first; the merge
     launch advances head_lens and cu_seqlens_k."""

@@ -29,11 +29,13 @@ from .. import _lib
 
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
 _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
-# group sizes whose fused (append + attend) piece-list kernel fits the register file.  With more query heads per KV head it
-# spills (Qwen3-14B's group of 5, 64 segments of 8448 rows: 2.45 ms per step against 2.09 ms on the grid launch + merge
-# kernel): there the dense cache stays on the grid launch and the ragged caches run the append as its own launch in
-# front of the unfused piece-list kernel
-_FUSED_PIECES_GROUPS = (1, 2, 3, 4)
+# Group sizes that use the fused (append + attend) piece-list kernel.  It fits the register file up to six query heads per
+# KV head (one spilled dword at five) and spills badly at eight.  Ragged caches, whose alternative is the append as a
+# launch of its own in front of the unfused piece-list kernel: 43.0 against 45.1 us per layer at a group of 5, 44.0 against
+# 46.0 at 6, 63.9 against 59.9 at 8 (256 lognormal segments).  Dense cache, whose alternative is the fused grid launch +
+# merge kernel: equal at a group of 5 (2.044 against 2.039 ms per step at Qwen3-14B's shape), so it stays there.
+_FUSED_PIECES_GROUPS = (1, 2, 3, 4, 5, 6)
+_DENSE_PIECES_GROUPS = (1, 2, 3, 4)
 _WARNED = set()
 dense_workgroups, dense_min_rows = 256, 512   # piece-list launches of the dense cache: workgroups wanted, fewest rows apiece
 dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)
@@ -261,7 +263,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     G = Hq // Hkv
     scale = D ** -0.5 if scaling is None else scaling
     dense_pieces = None
-    if Q == 1 and not dense_chunk and G in _FUSED_PIECES_GROUPS:
+    if Q == 1 and not dense_chunk and G in _DENSE_PIECES_GROUPS:
         dense_pieces = _uniform_pieces(query.device, B * Hkv, n)
     slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None, dense_pieces)
     if slab is not None:
