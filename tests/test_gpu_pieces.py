@@ -194,7 +194,11 @@ def test_alternating_layouts_reproduce_their_first_result():
     v = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
     LEN = torch.from_numpy(lens).to(DEV)
     st = L.current_stream(torch.device(DEV))
-    layouts = [_piece_list(lens, t, rng, "shuffled" if i % 2 else "desc") for i, t in enumerate((300.0, 640.0, 1000.0))]
+    layouts = [_piece_list(lens, t, rng, "shuffled" if i % 2 else "desc") for i, t in enumerate((300.0, 640.0))]
+    host = np.zeros((2 * nseg + 512, 4), dtype=np.int32)      # and a planned list: pieces of unequal size, every compute unit equally full
+    n = lib.trimkv_plan_attn_pieces(lens.ctypes.data, nseg, 256, 64, host.ctypes.data, host.shape[0])
+    assert n >= nseg
+    layouts.append((torch.from_numpy(host[:n].copy()).to(DEV), int(n), 0))
     ws = torch.zeros(max(lib.trimkv_decode_attn_pieces_workspace(n, G) for _, n, _ in layouts), dtype=torch.uint8, device=DEV)
     qs = [torch.randn(nseg * G, D, generator=gen).to(torch.bfloat16).to(DEV) for _ in range(2)]
     first = {}
