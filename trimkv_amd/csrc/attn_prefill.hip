@@ -304,8 +304,19 @@ template <bool F16>
 __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
 
-    const int seg = blockIdx.y;
-    const int tile = (int)gridDim.x - 1 - (int)blockIdx.x;  // later times see more keys: dispatch them first
+    // Workgroups are handed to the 8 XCDs round robin in dispatch order (x fastest), and each XCD has its own L2.  All
+    // query tiles of a segment read the same K/V, so they are mapped to one XCD (segment s on XCD s % 8, its tiles in
+    // consecutive turns of that XCD, later times first: they see more keys): the K/V tiles that several of them walk at
+    // about the same time are then fetched into one L2 instead of eight.
+    int seg = blockIdx.y, tile = (int)gridDim.x - 1 - (int)blockIdx.x;
+#ifndef TRIMKV_PF_NO_XCD_MAP
+    if ((gridDim.y & 7) == 0) {
+        const int lin = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;
+        const int turn = lin >> 3;
+        seg = (lin & 7) + 8 * (turn / (int)gridDim.x);
+        tile = (int)gridDim.x - 1 - turn % (int)gridDim.x;
+    }
+#endif
     const int b = seg / a.kv_heads, h = seg - b * a.kv_heads;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
