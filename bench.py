@@ -112,26 +112,41 @@ def cpu_baseline(c, budget_s=20.0):
             "os_cpu_count": cores}
 
 
-def attention_gate(cache, c, attn_fn, mod):
-    """Outside the timed region: the attention of a few segments of layer 0 against fp32 softmax.
+def attention_gate(cache, c, attn_fn, mod, pos_next):
+    """Outside the timed region: one more decode call of layer 0 made exactly as the timed ones are (update() defers the
+    append when the cache fuses it, the attention launch carries it out), checked on a few segments against fp32 softmax
+    over the rows the slab held before the call plus the NEW row taken from the call's inputs -- so a wrongly appended or
+    wrongly attended row shows -- and the row the launch wrote is compared with those inputs.
     (The full oracle comparison lives in tests/; this gate only guards the run that was just timed.)"""
     import torch
 
     slab = cache._slabs[0]
-    n = slab.max_len
-    k = slab.k[:8, :n].float().cpu()
-    v = slab.v[:8, :n].float().cpu()
-    G = c["Hq"] // c["Hkv"]
-    q = torch.randn(c["B"], c["Hq"], 1, D, device=slab.k.device).to(torch.bfloat16)
-    out, _, _ = attn_fn(mod, q, cache.key_cache[0], cache.value_cache[0], None, scaling=D ** -0.5,
-                        flash_attn_kwargs={"seg_len": slab.seg_len, "max_len": n})
+    dev = slab.k.device
+    B, Hkv, G = c["B"], c["Hkv"], c["Hq"] // c["Hkv"]
+    n_old = slab.max_len
+    k_old = slab.k[:8, :n_old].float().cpu()
+    v_old = slab.v[:8, :n_old].float().cpu()
+    kn = torch.randn(B, Hkv, 1, D, device=dev).to(torch.bfloat16)
+    vn = torch.randn(B, Hkv, 1, D, device=dev).to(torch.bfloat16)
+    lbn = torch.nn.functional.logsigmoid(torch.randn(B, Hkv, 1, device=dev) * c["sigma"] + c["mu"]).to(slab.lb.dtype)
+    pos = torch.full((1,), pos_next, dtype=torch.int64, device=dev)
+    q = torch.randn(B, c["Hq"], 1, D, device=dev).to(torch.bfloat16)
+    K, V, _, _, kw = cache.update(kn, vn, lbn, pos, 0)
+    carried = "pending_append" in kw
+    out, _, _ = attn_fn(mod, q, K, V, None, scaling=D ** -0.5, flash_attn_kwargs=kw)
+    k = torch.cat([k_old, kn.view(-1, 1, D)[:8].float().cpu()], dim=1)
+    v = torch.cat([v_old, vn.view(-1, 1, D)[:8].float().cpu()], dim=1)
     q8 = q.reshape(-1, G, D)[:8].float().cpu()
     s = torch.einsum("sgd,snd->sgn", q8, k) * D ** -0.5
     want = torch.einsum("sgn,snd->sgd", torch.softmax(s, -1), v)
     got = out.reshape(-1, G, D)[:8].float().cpu()
     err = (got - want).abs()
     attn_ok = bool((err <= 2e-2 + 1e-2 * want.abs()).all())
-    return {"attention_max_abs_err": float(err.max()), "attention_within_2e-2_abs_1e-2_rel": attn_ok}
+    row_ok = (slab.pending is None and slab.max_len == n_old + 1 and bool((slab.seg_len == n_old + 1).all())
+              and torch.equal(slab.k[:, n_old], kn.view(-1, D)) and torch.equal(slab.v[:, n_old], vn.view(-1, D))
+              and torch.equal(slab.lb[:, n_old], lbn.view(-1)) and bool((slab.pos[:, n_old] == pos_next).all()))
+    return {"attention_max_abs_err": float(err.max()), "attention_within_2e-2_abs_1e-2_rel": attn_ok,
+            "gate_call_append_carried_by_attention_launch": carried, "appended_row_and_lengths_equal_inputs": bool(row_ok)}
 
 
 def timed_checked_eviction(cache, c, layers_to_check):
@@ -608,7 +623,7 @@ def main():
                 "mfma_utilisation": 0.0,
                 "mfma_note": f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
                              "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
-    parity = attention_gate(cache, c, attn_fn, mod)
+    parity = attention_gate(cache, c, attn_fn, mod, T)
     parity.update(evict_parity)
     timing = {"host_enqueue_ms_per_step": round(enqueue_seconds * 1e3 / args.steps, 4), "ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}
     if amortised:

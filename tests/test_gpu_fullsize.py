@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from tests.gpu_util import DEV, attn_close
+from tests.gpu_util import DEV, attn_close, boundary_ties
 
 pytestmark = pytest.mark.gpu
 
@@ -365,3 +365,75 @@ def test_uncompressed_long_context_decode_and_chunk():
             want = torch.softmax(s.masked_fill(~vis, float("-inf")), -1) @ v[seg].float()
             ok, err = attn_close(outc[0, rows, seg * G + g], want)
             assert ok, (seg, g, err)
+
+
+@pytest.mark.parametrize("name,B,H,G,M,buf,mu,sigma", [
+    ("config3", 64, 8, 4, 4096, 128, 3.0, 1.5),     # 512 segments: one workgroup per segment, the append rides in the attention launch
+    ("config2", 16, 8, 2, 2048, 128, 3.0, 1.0),     # 128 segments: fused piece list, two pieces per segment merged in the launch
+    ("config5", 8, 8, 5, 8192, 512, 2.0, 2.0),      # 64 segments: fused grid launch (4 splits) + merge kernel, which advances the lengths
+])
+def test_fused_decode_step_at_full_shape_across_an_eviction(name, B, H, G, M, buf, mu, sigma):
+    """The launches the benchmark times, at their own shapes: ``fuse_decode_append`` on, one layer, four decode steps that
+    cross an eviction (M+buf-1 -> M+buf -> evict -> M+1 -> M+2 rows).  Every step: the fused output equals the output of an
+    unfused twin cache bit for bit and fp32 softmax on >= 16 sampled segments within the tolerance; the row the launch wrote
+    (K, V, log beta, position at n-1) equals the inputs; lengths, positions and the whole K/V state equal the CPU oracle's
+    (reference: cache_utils.py:104-110 append, :140-198 eviction; call order modeling_trimkv_qwen3.py:353 -> :365)."""
+    from oracle.dense_ref import DenseCacheRef
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    attn = get_attention_interface("trimkv_hip")
+    nseg = B * H
+    n = M + buf - 2
+    gen = torch.Generator(device=DEV).manual_seed(B * 1000 + G)
+    k = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    v = torch.randn(B, H, n, 128, generator=gen, device=DEV).to(torch.bfloat16)
+    lb = torch.nn.functional.logsigmoid(torch.randn(B, H, n, generator=gen, device=DEV) * sigma + mu)
+    pos = torch.arange(n, device=DEV)
+    plain, fused, ref = TrimKVCache(), TrimKVCache(), DenseCacheRef()
+    fused.fuse_decode_append = True
+    for c in (plain, fused):
+        c.update(k, v, lb, pos, 0)
+        c.compress("alpha", M, buf)                            # not due: only teaches the caches their budget
+    ref.update(k.cpu(), v.cpu(), lb.cpu(), pos.cpu(), 0)
+    del k, v, lb
+    segs = torch.arange(0, nseg, max(1, nseg // 16), device=DEV)[:32]
+    assert segs.numel() >= 16
+    lengths = []
+    tied = torch.zeros(B, H, dtype=torch.bool)
+    for t in range(4):
+        kn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        vn = torch.randn(B, H, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        lbn = torch.nn.functional.logsigmoid(torch.randn(B, H, 1, generator=gen, device=DEV) * sigma + mu)
+        q = torch.randn(B, H * G, 1, 128, generator=gen, device=DEV).to(torch.bfloat16)
+        posn = torch.full((1,), M + buf - 2 + t, dtype=torch.int64, device=DEV)
+        print(f"{name}: fused step {t}, {plain.get_cache_length(0) + 1} rows", flush=True)
+        ref.update(kn.cpu(), vn.cpu(), lbn.cpu(), posn.cpu(), 0)
+        Kp, Vp, _, _, kwp = plain.update(kn, vn, lbn, posn, 0)
+        Kf, Vf, _, _, kwf = fused.update(kn, vn, lbn, posn, 0)
+        n = ref.get_cache_length(0)
+        lengths.append(n)
+        assert "pending_append" in kwf and "pending_append" not in kwp and fused._slabs[0].pending is not None
+        assert Kf.shape == Kp.shape == (B, H, n, 128) and kwf["max_len"] == n
+        want, _, _ = attn(_Mod(), q, Kp, Vp, None, scaling=128 ** -0.5, flash_attn_kwargs=kwp)
+        got, _, _ = attn(_Mod(), q, Kf, Vf, None, scaling=128 ** -0.5, flash_attn_kwargs=kwf)
+        slab = fused._slabs[0]
+        assert slab.pending is None, "the attention call did not carry the append out"
+        assert torch.equal(got, want), "fused launch differs from append + attend"
+        fp32 = _fp32_attention_on_segments(q, plain._slabs[0].k, plain._slabs[0].v, segs, G, n)
+        ok, err = attn_close(got.view(nseg, G, 128)[segs], fp32)
+        assert ok, (t, err)
+        # the row this launch wrote, and the lengths it advanced
+        assert torch.equal(slab.k[:, n - 1], kn.view(nseg, 128)) and torch.equal(slab.v[:, n - 1], vn.view(nseg, 128))
+        assert torch.equal(slab.lb[:, n - 1], lbn.view(nseg)) and bool((slab.pos[:, n - 1] == posn).all())
+        assert bool((slab.seg_len == n).all()) and slab.lens.tolist() == [n] * nseg
+        if n >= M + buf:   # rows whose cut is a tie have no defined parity (topk's tie order is the library's): left out from here on
+            tied |= boundary_ties(ref.retention_weights[0], ref.kv_positions[0], ref.get_seq_length(0) + 1, M)
+        for c in (plain, fused, ref):
+            c.compress("alpha", M, buf)
+        assert fused.get_cache_length(0) == ref.get_cache_length(0) == plain.get_cache_length(0)
+        assert torch.equal(fused.kv_positions[0].cpu()[~tied], ref.kv_positions[0][~tied]), "retained positions differ from the oracle"
+        assert torch.equal(fused._slabs[0].seg_len, plain._slabs[0].seg_len)
+    assert lengths == [M + buf - 1, M + buf, M + 1, M + 2] and int(tied.sum()) <= 2
+    for a, b in zip(fused[0], plain[0]):
+        assert torch.equal(a, b)
+    assert torch.equal(fused.key_cache[0].cpu()[~tied], ref.key_cache[0][~tied]) and torch.equal(fused.value_cache[0].cpu()[~tied], ref.value_cache[0][~tied])
+    assert torch.equal(fused.retention_weights[0].cpu()[~tied], ref.retention_weights[0][~tied])
