@@ -169,6 +169,8 @@ int trimkv_evict(void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, i
  * first_kept (optional, [nlayers*nseg]) receives 1 where the segment's oldest token (row 0) is among the kept ones and 0
  * elsewhere: what the single-sequence floor branch needs to reproduce bucketize(right=False) against the inclusive
  * cumulative lengths (cache_utils.py:496), which credits a chosen first row to the previous head.
+ * With strategy TRIMKV_SCORE_KNORM_ALPHA the K rows are read as 16-byte pieces: head_dim must be a multiple of 8 (at most
+ * 512; TRIMKV_ERR_UNSUPPORTED otherwise) and every k slab 16-byte aligned, as all K/V slabs of this library are.
  */
 int trimkv_group_threshold(const void* const* lb_slabs, const int64_t* const* pos_slabs,
                            const void* const* k_slabs, const int32_t* const* seg_lens,

@@ -85,6 +85,11 @@ def test_bad_arguments_are_refused_without_a_launch():
                                       one, one, one, one, None, None) == -2  # 3 does not divide 8
     assert lib.trimkv_group_threshold(one, one, None, one, 1, 8, 4, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 1, 1,
                                       one, one, one, one, None, None) == -1  # knorm without K
+    for bad_dim in (100, 4, 1032):   # knorm reads K rows as 16-byte pieces: head_dim must be a multiple of 8, at most 512
+        assert lib.trimkv_group_threshold(one, one, one, one, 1, 8, 4, 64, bad_dim, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 1, 1,
+                                          one, one, one, one, None, None) == -6
+        assert lib.trimkv_group_threshold_wide(one, one, one, one, 2, 8, 4, 64, bad_dim, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 1, 1,
+                                               one, one, one, one, None, one, 1 << 20, None) == -6
     assert lib.trimkv_group_threshold_each_layer(one, one, None, one, 3, 8, 3, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 0, 1,
                                                  one, one, one, one, one, None) == -2
     wide = lambda spg, ws, wsb, strat=0: lib.trimkv_group_threshold_wide(one, one, None, one, 2, 8, spg, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0,

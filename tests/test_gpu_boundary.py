@@ -143,3 +143,133 @@ def test_ragged_update_can_return_the_reference_packed_layout():
     cache.return_packed = True
     K2, _, _, _, kw2 = cache.update(None, None, None, None, 0)
     assert torch.equal(K2, K) and "seg_start" not in kw2
+
+
+def _window_mask(Q, n, window, causal=True):
+    """Additive mask of the sliding-window rule: a query at absolute row p = n-Q+t sees rows p-window+1 .. p (and as far
+    ahead when not causal), the meaning HF flash_attention_2 gives ``sliding_window`` (window_size=(w-1, w-1))."""
+    p = (n - Q + torch.arange(Q))[:, None]
+    j = torch.arange(n)[None, :]
+    hidden = (p - j) > window - 1
+    hidden |= (j > p) if causal else ((j - p) > window - 1)
+    return torch.zeros(1, 1, Q, n).masked_fill(hidden[None, None], float("-inf"))
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_sliding_window_at_decode_runs_on_the_kernel(fused, monkeypatch):
+    """The reference forwards ``sliding_window`` to HF flash attention (modeling_trimkv_qwen3.py:365-380 ->
+    attn/__init__.py:15-26).  At Q_LEN == 1 it is a first attended row (n - window) and stays on the kernel (TRIMKV_STRICT
+    is set); a window that covers the whole cache changes nothing; a deferred append is carried out first."""
+    from trimkv_amd import TrimKVCache, get_attention_interface
+    monkeypatch.setenv("TRIMKV_STRICT", "1")
+    B, H, G, n = 2, 4, 2, 900
+    gen = torch.Generator().manual_seed(11)
+    k, v = draw_kv(gen, B, H, n)
+    lb = draw_log_beta(gen, B, H, n)
+    cache = TrimKVCache()
+    cache.fuse_decode_append = fused
+    cache.update(k[:, :, :-1].to(DEV), v[:, :, :-1].to(DEV), lb[:, :, :-1].to(DEV), torch.arange(n - 1).to(DEV), 0)
+    K, V, _, _, kw = cache.update(k[:, :, -1:].to(DEV), v[:, :, -1:].to(DEV), lb[:, :, -1:].to(DEV), torch.arange(n - 1, n).to(DEV), 0)
+    assert ("pending_append" in kw) == fused
+    q = torch.randn(B, H * G, 1, 128, generator=gen).to(torch.bfloat16)
+    attn = get_attention_interface("trimkv_hip")
+    for window in (1, 37, 512, 899):
+        out, _, _ = attn(_Mod(), q.to(DEV), K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, sliding_window=window, is_causal=True, dropout=0.0)
+        want, _ = eager_attention(q.float(), k.float(), v.float(), G, 128 ** -0.5, attention_mask=_window_mask(1, n, window))
+        ok, err = attn_close(out, want)
+        assert ok, (window, err)
+        assert cache._slabs[0].pending is None
+    full, _, _ = attn(_Mod(), q.to(DEV), K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw)
+    for window in (900, 4096):    # not longer than the window: plain attention, bit for bit
+        out, _, _ = attn(_Mod(), q.to(DEV), K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, sliding_window=window, is_causal=False)
+        assert torch.equal(out, full)
+    # a window together with a left-padding mask: the later of the two first rows
+    keep = torch.ones(B, n, dtype=torch.int64)
+    keep[1, :700] = 0
+    out, _, _ = attn(_Mod(), q.to(DEV), K, V, keep.to(DEV), scaling=128 ** -0.5, flash_attn_kwargs=kw, sliding_window=512)
+    additive = torch.zeros(B, 1, 1, n).masked_fill(keep[:, None, None, :] == 0, float("-inf")) + _window_mask(1, n, 512)
+    want, _ = eager_attention(q.float(), k.float(), v.float(), G, 128 ** -0.5, attention_mask=additive)
+    ok, err = attn_close(out, want)
+    assert ok, err
+
+
+def test_forwarded_kwargs_that_leave_the_kernels_are_honoured_and_announced(monkeypatch):
+    """``sliding_window`` / ``is_causal=False`` on a query block, ``dropout`` > 0 and ``softcap`` are computed with torch ops
+    to the meaning HF flash_attention_2 gives them, warn once per cause, and raise under TRIMKV_STRICT."""
+    from trimkv_amd import _lib, get_attention_interface
+    from trimkv_amd.attn import hip_attn
+    B, H, G, n, Q = 2, 2, 2, 300, 70
+    gen, k, v, K, V, kw = _dense(B, H, n, seed=12)
+    q = torch.randn(B, H * G, Q, 128, generator=gen).to(torch.bfloat16)
+    attn = get_attention_interface("trimkv_hip")
+    hip_attn._WARNED.clear()
+
+    def call(**extra):
+        with warnings.catch_warnings(record=True) as rec:
+            warnings.simplefilter("always")
+            out, _, _ = attn(_Mod(), q.to(DEV), K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, **extra)
+        return out, [w for w in rec if issubclass(w.category, RuntimeWarning)]
+
+    base, rec = call(is_causal=True, sliding_window=None, dropout=0.0)          # the kernel: nothing to announce
+    assert not rec
+    causal = _window_mask(Q, n, n)                                              # plain bottom-right causal rule
+    want, _ = eager_attention(q.float(), k.float(), v.float(), G, 128 ** -0.5, attention_mask=causal)
+    assert attn_close(base, want)[0]
+    for extra, mask in (({"sliding_window": 50}, _window_mask(Q, n, 50)),
+                        ({"sliding_window": 50, "is_causal": False}, _window_mask(Q, n, 50, causal=False)),
+                        ({"is_causal": False}, torch.zeros(1, 1, Q, n))):
+        out, rec = call(**extra)
+        assert len(rec) <= 1
+        want, _ = eager_attention(q.float(), k.float(), v.float(), G, 128 ** -0.5, attention_mask=mask)
+        ok, err = attn_close(out, want)
+        assert ok, (extra, err)
+    out, rec = call(sliding_window=50)                                          # the same cause again: no second warning
+    assert not rec
+    # softcap: scores squashed before the softmax
+    out, rec = call(softcap=5.0)
+    s = torch.einsum("bhqd,bhnd->bhqn", q.float(), k.float().repeat_interleave(G, dim=1)) * 128 ** -0.5
+    p = torch.softmax(5.0 * torch.tanh(s / 5.0) + causal, -1)
+    want = torch.einsum("bhqn,bhnd->bqhd", p, v.float().repeat_interleave(G, dim=1))
+    ok, err = attn_close(out, want)
+    assert ok and len(rec) == 1, err
+    # dropout: random, so only its statistics: with V == 1 every output is sum(kept p) / (1 - rate), mean 1
+    ones = torch.ones_like(V)
+    with warnings.catch_warnings(record=True) as rec:
+        warnings.simplefilter("always")
+        out, _, _ = attn(_Mod(), q.to(DEV), K, ones, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, dropout=0.5)
+    assert any("dropout" in str(w.message) for w in rec)
+    assert abs(float(out.float().mean()) - 1.0) < 0.05 and float(out.float().std()) > 0.01
+    nodrop, _, _ = attn(_Mod(), q.to(DEV), K, ones, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, dropout=0.0)
+    assert float((nodrop.float() - 1.0).abs().max()) < 1e-2
+    monkeypatch.setenv("TRIMKV_STRICT", "1")
+    for extra in ({"sliding_window": 50}, {"is_causal": False}, {"dropout": 0.1}, {"softcap": 5.0}):
+        with pytest.raises(_lib.TrimKVLibraryError):
+            attn(_Mod(), q.to(DEV), K, V, None, scaling=128 ** -0.5, flash_attn_kwargs=kw, **extra)
+
+
+def test_ragged_entry_points_ignore_what_the_reference_ignores_and_honour_dropout_p(monkeypatch):
+    """flash_attn.py:79-89 takes ``sliding_window`` / ``is_causal`` / ``dropout`` into **kwargs and drops them; only
+    ``dropout_p`` reaches flash_attn_varlen_func (:143).  Same here: the first three change nothing (bit for bit, on the
+    kernel), ``dropout_p`` > 0 is computed with torch ops and announced."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, _lib, get_attention_interface
+    B, H, G, n = 2, 4, 2, 260
+    gen = torch.Generator().manual_seed(13)
+    k, v = draw_kv(gen, B, H, n)
+    lb = draw_log_beta(gen, B, H, n)
+    cache = BatchedDynamicBudgetTrimKVCache()
+    K, V, _, _, kw = cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), torch.arange(n).to(DEV), 0)
+    attn = get_attention_interface("db_attn_flash_batched")
+    q = torch.randn(B, H * G, 1, 128, generator=gen).to(torch.bfloat16).to(DEV)
+    monkeypatch.setenv("TRIMKV_STRICT", "1")
+    base, _, _ = attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw)
+    same, _, _ = attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw, sliding_window=16, is_causal=False, dropout=0.3, scaling=7.0)
+    assert torch.equal(base, same)
+    with pytest.raises(_lib.TrimKVLibraryError):
+        attn(_Mod(), q, K, V, None, flash_attn_kwargs=kw, dropout_p=0.3)
+    monkeypatch.setenv("TRIMKV_STRICT", "0")
+    ones = torch.ones_like(V)
+    with warnings.catch_warnings(record=True) as rec:
+        warnings.simplefilter("always")
+        out, _, _ = attn(_Mod(), q, K, ones, None, flash_attn_kwargs=kw, dropout_p=0.5)
+    assert any("dropout_p" in str(w.message) for w in rec)
+    assert out.shape == base.shape and abs(float(out.float().mean()) - 1.0) < 0.1 and float(out.float().std()) > 0.01

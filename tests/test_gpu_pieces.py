@@ -180,10 +180,12 @@ def test_append_attend_pieces_equals_append_then_attend():
 
 
 def test_alternating_layouts_reproduce_their_first_result():
-    """Three different piece lists take turns on ONE workspace, with the host synchronising between launches (every launch
-    then starts on an idle GPU and the pieces of a segment finish almost together).  Whatever a launch finds in the partial
-    slots was written by another layout, so a merge that read a slot before its writer's stores had landed would give
-    another result than that layout's first launch: every launch must reproduce it bit for bit."""
+    """The in-launch merge, attacked deterministically.  Three different piece lists take turns on ONE workspace, the host
+    synchronising after every launch (each launch then starts on an idle GPU and the pieces of a segment finish almost
+    together), and before every launch the partial slots are overwritten with NaN.  A merging workgroup that read a slot
+    before its writer's stores had landed would therefore read NaN (or, without the poison, another layout's partial) and
+    the output would differ from that layout's first launch, which was itself checked against the separate merge kernel:
+    every one of the 2000 launches must reproduce it bit for bit; the loop stops at the first that does not."""
     from trimkv_amd import _lib as L
     lib = L.load()
     rng = np.random.default_rng(0)
@@ -200,20 +202,33 @@ def test_alternating_layouts_reproduce_their_first_result():
     assert n >= nseg
     layouts.append((torch.from_numpy(host[:n].copy()).to(DEV), int(n), 0))
     ws = torch.zeros(max(lib.trimkv_decode_attn_pieces_workspace(n, G) for _, n, _ in layouts), dtype=torch.uint8, device=DEV)
+    slots = ws[32768:32768 + (ws.numel() - 32768) // 4 * 4].view(torch.float32)     # behind the counter header: the partials
     qs = [torch.randn(nseg * G, D, generator=gen).to(torch.bfloat16).to(DEV) for _ in range(2)]
+    # what every layout has to produce: the grid launch + separate merge kernel agrees with it up to the output rounding
+    ws0 = torch.empty(max(16, lib.trimkv_decode_attn_workspace(nseg, G, D, cap, 512)), dtype=torch.uint8, device=DEV)
+    grid = []
+    for q in qs:
+        want = torch.empty_like(q)
+        L.check(lib.trimkv_decode_attn(q.data_ptr(), want.data_ptr(), k.data_ptr(), v.data_ptr(), LEN.data_ptr(), None, None, None,
+                                       nseg, cap, D, G, L.BF16, D ** -0.5, cap, 512, ws0.data_ptr(), ws0.numel(), st), "grid")
+        grid.append(want)
     first = {}
-    print("alternating piece layouts, 360 launches", flush=True)
-    for it in range(360):
+    launches = 2000
+    print(f"alternating piece layouts with poisoned partial slots, {launches} launches", flush=True)
+    for it in range(launches):
         li, qi = it % 3, (it // 3) % 2
         plist, npieces, _ = layouts[li]
         got = torch.empty_like(qs[qi])
+        slots.fill_(float("nan"))
         L.check(lib.trimkv_decode_attn_pieces(qs[qi].data_ptr(), got.data_ptr(), k.data_ptr(), v.data_ptr(), LEN.data_ptr(), None, None,
                                               plist.data_ptr(), npieces, nseg, cap, D, G, L.BF16, D ** -0.5, cap, ws.data_ptr(), ws.numel(), st), "pieces")
         torch.cuda.synchronize()
         if (li, qi) not in first:
+            assert not torch.isnan(got.float()).any() and (got.float() - grid[qi].float()).abs().max() < 4e-3
             first[(li, qi)] = got
-        else:
-            assert torch.equal(got, first[(li, qi)]), f"launch {it} (layout {li}) differs from the first launch of its layout"
+        elif not torch.equal(got, first[(li, qi)]):
+            bad = (got != first[(li, qi)]).any(dim=-1).nonzero().flatten()[:8].tolist()
+            pytest.fail(f"launch {it} (layout {li}) differs from the first launch of its layout in rows {bad}; NaN: {bool(torch.isnan(got.float()).any())}")
     assert not ws[:32768].any()
 
 

@@ -215,6 +215,39 @@ def test_single_sequence_floor_branch_credits_boundary_token_to_previous_head():
         d.cache.compress("bogus", 1, 0)
 
 
+def test_single_sequence_floor_branch_credit_skips_an_empty_head():
+    """cache_utils.py:496 with an empty head in front of the boundary token: bucketize credits the first head whose
+    inclusive cumsum equals the token's flat index, i.e. the nearest head BEFORE the run of empty heads, not the empty head
+    itself.  Head 1 of layer 0 is emptied by a first shared-budget eviction; a second one with a smaller budget and a floor
+    then credits head 2's first row to head 0, which keeps one token more than it would otherwise."""
+    from trimkv_amd import DynamicBudgetTrimKVCache
+    H, L, M1, M2, buf, floor = 3, 2, 24, 14, 2, 0.34
+    d = _Driver(DynamicBudgetTrimKVCache(), SingleRaggedCacheRef(), 1, H, L, seed=78)
+    pos = torch.arange(40)
+    for l in range(L):
+        k, v = draw_kv(d.gen, 1, H, 40)
+        lb = draw_log_beta(d.gen, 1, H, 40, sigma=1.5)
+        if l == 0:
+            lb[0, 1, :] = -50.0 - torch.arange(40) * 1e-3          # hopeless: head 1 of layer 0 loses every token
+            lb[0, 2, :] = lb[0, 2, :].clamp(max=-1e-3)
+            lb[0, 2, 0] = -1e-7                                     # head 2's first row survives and will be chosen again
+        d.ref.update(k, v, lb, pos, l)
+        d.cache.update(k.to(DEV), v.to(DEV), lb.to(DEV), pos.to(DEV), l)
+    d.T = 40
+    for c in (d.ref, d.cache):
+        c.compress("alpha", M1, buf)
+    _same(d.cache, d.ref)
+    assert d.ref.head_lens[0].tolist()[1] == 0 and int(d.ref.segment_positions()[0][2][0]) == 0
+    before = d.ref.head_lens[0].tolist()
+    snap = _snapshot(d.ref, "alpha")
+    kw = dict(strategy="alpha", memory_size=M2, buffer_size=buf, floor_budget_ratio=floor)
+    d.ref.compress(**kw)
+    d.cache.compress(**kw)
+    assert d.ref.head_lens[0].tolist() != before
+    _assert_no_tie_at_a_cut(snap, d.ref)
+    _same(d.cache, d.ref)
+
+
 def test_bf16_log_beta_scores_stay_bf16_in_the_ragged_classes():
     """int64 age * bf16 log beta -> bf16 (age rounded to bf16 first); ties are common, so the kept
     SCORES are compared: the multiset of kept scores must equal the oracle's."""

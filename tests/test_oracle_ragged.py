@@ -262,6 +262,56 @@ def test_single_sequence_floor_branch_with_boundary_credit():
         ref.compress("alpha_threshold", M, buf, floor_budget_ratio=floor)
 
 
+def test_single_sequence_floor_branch_credit_skips_empty_heads():
+    """bucketize(right=False) with an EMPTY head in front of the boundary token: the first row of head j sits at flat index
+    cu[j-1] == cu[j-2] when head j-1 is empty, so it is counted for the head before the run of empty heads (torch.bucketize
+    ([3], [3, 3, 5]) -> 0), not for j-1.  A head is emptied by a first eviction under a shared budget (its log beta is made
+    hopeless), a second eviction with a smaller budget and a floor then runs the crediting across it."""
+    assert torch.bucketize(torch.tensor([3]), torch.tensor([3, 3, 5])).tolist() == [0]
+    rng = np.random.default_rng(16)
+    H, L, M1, M2, buf, floor = 3, 2, 8, 5, 1, 0.34
+    ref, brute = SingleRaggedCacheRef(), _Brute(1, H, L)
+    _fill(ref, brute, rng, 1, H, L, [12])
+    # head 1 of layer 0: every token hopeless -> emptied by the shared-budget eviction
+    lo, hi = int(ref.cu_seqlens_k[0][1]), int(ref.cu_seqlens_k[0][2])
+    ref.retention_weights[0][lo:hi] = -50.0
+    brute.seg[0][1] = [(p, np.float32(-50.0), kr) for p, _, kr in brute.seg[0][1]]
+    ref.compress("alpha", M1, buf)
+    toks = [(l, h, i) for l in range(L) for h in range(H) for i in range(len(brute.seg[l][h]))]
+    mask = brute.topk_mask([brute.score(brute.seg[l][h][i], False) for l, h, i in toks], L * H * M1)
+    kept = {(l, h): [] for l in range(L) for h in range(H)}
+    for j, (l, h, i) in enumerate(toks):
+        if mask[j]:
+            kept[(l, h)].append(brute.seg[l][h][i])
+    for (l, h), lst in kept.items():
+        brute.seg[l][h] = lst
+    _assert_same(ref, brute, L)
+    assert brute.lens(0)[1] == 0, "the test needs an empty head"
+    # the first row of head 2 of layer 0 (flat index cu[1] == cu[0]) is certain to be chosen
+    ref.retention_weights[0][ref.cu_seqlens_k[0][2]] = -1e-6
+    p, _, kr = brute.seg[0][2][0]
+    brute.seg[0][2][0] = (p, np.float32(-1e-6), kr)
+    ref.compress("alpha", M2, buf, floor_budget_ratio=floor)
+    toks = [(l, h, i) for l in range(L) for h in range(H) for i in range(len(brute.seg[l][h]))]
+    sc = [brute.score(brute.seg[l][h][i], False) for l, h, i in toks]
+    chosen = np.flatnonzero(brute.topk_mask(sc, int(L * H * M2 * (1 - floor))))
+    lens = [len(brute.seg[l][h]) for l in range(L) for h in range(H)]
+    incl = np.cumsum(lens)
+    cnt = np.zeros(L * H, dtype=int)
+    for j in chosen:
+        cnt[int(np.searchsorted(incl, j, side="left"))] += 1
+    assert int(incl[0]) in chosen.tolist() and cnt[1] == 0      # the boundary token went past the empty head 1 to head 0
+    cnt = cnt + int(M2 * floor)
+    for l in range(L):
+        for h in range(H):
+            seg = brute.seg[l][h]
+            if cnt[l * H + h] >= len(seg):
+                continue
+            m = brute.topk_mask([brute.score(t, False) for t in seg], cnt[l * H + h])
+            brute.seg[l][h] = [t for t, keep in zip(seg, m) if keep]
+    _assert_same(ref, brute, L)
+
+
 def test_ragged_scores_stay_in_log_beta_dtype():
     """int64 * bf16 -> bf16 with the age rounded to bf16 first: restated bit by bit."""
     rng = np.random.default_rng(7)

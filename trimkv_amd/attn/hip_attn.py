@@ -222,12 +222,6 @@ def prefill_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.T
     return out
 
 
-def _causal_bottom_right(qlen: int, n: int, device) -> torch.Tensor:
-    t = torch.arange(qlen, device=device)[:, None]
-    j = torch.arange(n, device=device)[None, :]
-    return j <= (n - qlen + t)
-
-
 _PAD_CACHE: Dict[str, tuple] = {}
 
 
@@ -254,27 +248,97 @@ def _left_padding_offsets(attention_mask: torch.Tensor, batch: int, n: int, kv_h
     return seg_first
 
 
+_WINDOW_FIRST: Dict[Tuple[str, int, int], torch.Tensor] = {}
+
+
+def _window_first(device, nseg: int, first: int) -> torch.Tensor:
+    """int32 [nseg] filled with ``first``: the first attended row of every segment under a sliding window at Q_LEN == 1.
+    A handful of tensors is kept (the window start moves by one row per step and wraps every eviction cycle)."""
+    key = (str(device), nseg, first)
+    t = _WINDOW_FIRST.get(key)
+    if t is None:
+        if len(_WINDOW_FIRST) > 4096:
+            _WINDOW_FIRST.clear()
+        t = torch.full((nseg,), first, dtype=torch.int32, device=device)
+        _WINDOW_FIRST[key] = t
+    return t
+
+
+def _dense_torch_attention(query, key, value, attention_mask, scale: float, causal: bool, window: Optional[int],
+                           dropout: float, softcap: Optional[float]):
+    """The dense attention with torch ops, for the calls the kernels do not take: fp32 softmax over
+    ``q k^T * scale`` (optionally soft-capped), keys hidden by the bottom-right aligned causal rule, by a sliding window
+    (query at absolute row p sees rows p-window+1 .. p, and as far ahead when not causal: flash-attn's
+    ``window_size=(window-1, window-1)``), by ``attention_mask``; dropout on the probabilities."""
+    B, Hq, Q, D = query.shape
+    Hkv, n = key.shape[1], key.shape[2]
+    G = Hq // Hkv
+    mask_is_causal = attention_mask is not None and attention_mask.dim() == 4   # HF's 4-D additive masks carry the causal rule
+    if attention_mask is not None and attention_mask.dim() == 2:   # HF's 2-D keep-mask -> additive
+        attention_mask = torch.zeros(B, 1, 1, n, dtype=torch.float32, device=query.device).masked_fill(attention_mask[:, None, None, :n] == 0, float("-inf"))
+    k = key.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
+    v = value.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
+    w = torch.matmul(query, k.transpose(2, 3)).float() * scale
+    if softcap is not None:
+        w = softcap * torch.tanh(w / softcap)
+    if attention_mask is not None:
+        w = w + attention_mask[:, :, :, :n].float()
+    qpos = (n - Q + torch.arange(Q, device=query.device))[:, None]
+    j = torch.arange(n, device=query.device)[None, :]
+    hidden = None
+    if causal and Q > 1 and not mask_is_causal:
+        hidden = j > qpos
+    if window is not None:
+        far = (qpos - j) > window - 1
+        if not causal:
+            far = far | ((j - qpos) > window - 1)
+        hidden = far if hidden is None else (hidden | far)
+    if hidden is not None:
+        w = w.masked_fill(hidden, float("-inf"))
+    w = torch.softmax(w, dim=-1)
+    if dropout > 0.0:
+        w = torch.dropout(w, dropout, True)
+    return torch.matmul(w.to(query.dtype), v).transpose(1, 2).contiguous()
+
+
 def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                             attention_mask: Optional[torch.Tensor] = None, scaling: Optional[float] = None,
-                            dropout: float = 0.0, flash_attn_kwargs: Optional[dict] = None, **kwargs):
-    """Dense-cache attention.  query [B,Hq,Q,D], key/value [B,Hkv,n,D] -> ([B,Q,Hq,D], None, None)."""
+                            dropout: float = 0.0, flash_attn_kwargs: Optional[dict] = None, sliding_window: Optional[int] = None,
+                            is_causal: Optional[bool] = None, softcap: Optional[float] = None, **kwargs):
+    """Dense-cache attention.  query [B,Hq,Q,D], key/value [B,Hkv,n,D] -> ([B,Q,Hq,D], None, None).
+
+    The keyword arguments the reference's attention module forwards (modeling_trimkv_qwen3.py:365-380) mean what they
+    mean to HF's flash_attention_2, which the reference's dense path calls (attn/__init__.py:15-26):
+    ``sliding_window`` limits a query to the last ``sliding_window`` rows once the cache holds more than that;
+    ``is_causal`` (default: ``module.is_causal``, else True) switches the bottom-right causal rule of a query block;
+    ``dropout`` > 0 drops probabilities; ``softcap`` caps the scores.  At Q_LEN == 1 a window is a first attended row per
+    segment and runs on the kernel, causality changes nothing; a window or ``is_causal=False`` on a query block, dropout
+    and softcap run on torch ops and say so (``slow_path``)."""
     B, Hq, Q, D = query.shape
     Hkv, n = key.shape[1], key.shape[2]
     G = Hq // Hkv
     scale = D ** -0.5 if scaling is None else scaling
+    causal = bool(getattr(module, "is_causal", True)) if is_causal is None else bool(is_causal)
+    window = int(sliding_window) if sliding_window is not None and n > int(sliding_window) else None
+    plain = not dropout and softcap is None        # what the kernels compute: softmax(q k^T * scale) v
     dense_pieces = None
     if Q == 1 and not dense_chunk and G in _DENSE_PIECES_GROUPS:
         dense_pieces = _uniform_pieces(query.device, B * Hkv, n)
-    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None, dense_pieces)
+    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None and window is None and plain, dense_pieces)
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
         return append_attend(slab, q2, G, scale, chunk=dense_chunk, pieces=dense_pieces).view(B, 1, Hq, D), None, None
+    kernel_ok = plain and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128)
     seg_first = None
-    if attention_mask is not None and Q == 1 and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
-        seg_first = _left_padding_offsets(attention_mask, B, n, Hkv)   # a left-padding mask is a per-segment first row
-    if Q == 1 and (attention_mask is None or seg_first is not None):
+    if kernel_ok and Q == 1:
+        if attention_mask is not None:
+            seg_first = _left_padding_offsets(attention_mask, B, n, Hkv)   # a left-padding mask is a per-segment first row
+        if window is not None and (attention_mask is None or seg_first is not None):
+            wf = _window_first(query.device, B * Hkv, n - window)
+            seg_first = wf if seg_first is None else torch.maximum(seg_first, wf)
+    if kernel_ok and Q == 1 and (seg_first is not None or (attention_mask is None and window is None)):
         ks = key.stride()
         if not (ks[3] == 1 and ks[2] == D and ks[0] == Hkv * ks[1] and value.stride() == ks and ks[1] % D == 0):
             key, value = key.contiguous(), value.contiguous()
@@ -288,7 +352,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             seg_len = None
         out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first, pieces=dense_pieces)
         return out.view(B, 1, Hq, D), None, None
-    if attention_mask is None and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128):
+    if kernel_ok and Q > 1 and attention_mask is None and window is None and causal:
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)
               and value.stride() == key.stride() and key.stride(1) % D == 0)
         if not ok:
@@ -298,25 +362,46 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             seg_len = None
         out = prefill_attention(query, key, value, B, Hkv, G, seg_len, None, key.stride(1) // D, n, scale)
         return out, None, None
-    # what is left: masks that are not a left-padding prefix at Q_LEN == 1, any mask with a query block, fp32 tensors,
-    # other head dims -- torch ops, announced
-    slow_path("dense attention with " + ("an attention_mask that is not plain left padding at decode time" if attention_mask is not None and Q == 1
-                                         else "an attention_mask on a query block" if attention_mask is not None
-                                         else f"dtype {query.dtype} / head_dim {D}"))
-    if attention_mask is not None and attention_mask.dim() == 2:   # HF's 2-D keep-mask -> additive
-        attention_mask = torch.zeros(B, 1, 1, n, dtype=torch.float32, device=query.device).masked_fill(attention_mask[:, None, None, :n] == 0, float("-inf"))
-    k = key.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
-    v = value.unsqueeze(2).expand(B, Hkv, G, n, D).reshape(B, Hq, n, D)
-    w = torch.matmul(query, k.transpose(2, 3)).float() * scale
-    if attention_mask is not None:
-        w = w + attention_mask[:, :, :, :n].float()
-    elif Q > 1:
-        w = w.masked_fill(~_causal_bottom_right(Q, n, query.device), float("-inf"))
-    w = torch.softmax(w, dim=-1).to(query.dtype)
-    return torch.matmul(w, v).transpose(1, 2).contiguous(), None, None
+    # what is left -- torch ops, announced: masks that are not a left-padding prefix at Q_LEN == 1, any mask, window or
+    # is_causal=False with a query block, dropout, softcap, fp32 tensors, other head dims
+    if dropout:
+        why = f"dropout={dropout}"
+    elif softcap is not None:
+        why = "a score soft-cap"
+    elif attention_mask is not None:
+        why = "an attention_mask that is not plain left padding at decode time" if Q == 1 else "an attention_mask on a query block"
+    elif window is not None:
+        why = "a sliding window on a query block"
+    elif Q > 1 and not causal and kernel_ok:
+        why = "is_causal=False on a query block"
+    else:
+        why = f"dtype {query.dtype} / head_dim {D}"
+    slow_path("dense attention with " + why)
+    return _dense_torch_attention(query, key, value, attention_mask, scale, causal, window, float(dropout or 0.0), softcap), None, None
 
 
-def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_heads):
+def _ragged_torch_attention(query, key, value, head_lens, seg_start, G: int, dropout_p: float):
+    """Ragged attention with torch ops, segment by segment (only reached with ``dropout_p`` > 0, which the kernels do not
+    implement): fp32 softmax over ``q k^T / sqrt(D)``, bottom-right causal within a query block, dropout on the probabilities."""
+    B, Hq, Q, D = query.shape
+    lens, starts = head_lens.tolist(), seg_start.tolist()
+    hkv = Hq // G
+    out = torch.zeros(B, Q, Hq, D, dtype=query.dtype, device=query.device)
+    for seg, (n, s0) in enumerate(zip(lens, starts)):
+        if n <= 0:
+            continue
+        b, h = divmod(seg, hkv)
+        k, v = key[s0:s0 + n], value[s0:s0 + n]
+        w = torch.einsum("gqd,nd->gqn", query[b, h * G:(h + 1) * G].float(), k.float()) * D ** -0.5
+        if Q > 1:
+            vis = torch.arange(n, device=query.device)[None, :] <= (n - Q + torch.arange(Q, device=query.device))[:, None]
+            w = w.masked_fill(~vis, float("-inf"))
+        p = torch.dropout(torch.nan_to_num(torch.softmax(w, dim=-1)), dropout_p, True)
+        out[b, :, h * G:(h + 1) * G] = torch.einsum("gqn,nd->qgd", p.to(query.dtype), v)
+    return out
+
+
+def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_heads, dropout_p: float = 0.0):
     kw = flash_attn_kwargs or {}
     head_lens, cu = kw.get("head_lens"), kw.get("cu_seqlens_k")
     if head_lens is None or cu is None:
@@ -328,7 +413,7 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
     if num_kv_heads is None:
         num_kv_heads = nseg // batch_size
     G = Hq // num_kv_heads
-    slab = _take_pending(kw, query, key, G, Q == 1 and kw.get("seg_start") is not None, kw.get("pieces"))
+    slab = _take_pending(kw, query, key, G, Q == 1 and kw.get("seg_start") is not None and not dropout_p, kw.get("pieces"))
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
@@ -346,6 +431,9 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
         cap = max(1, max_len)   # unused with packed rows; the library only wants it positive (every segment may be empty)
     else:
         max_len, cap = kw["max_len"], kw["seg_cap"]
+    if dropout_p:   # flash_attn_varlen_func applies it whatever the module's mode (flash_attn.py:69, 143)
+        slow_path(f"ragged attention with dropout_p={dropout_p}")
+        return _ragged_torch_attention(query, key, value, head_lens, seg_start, G, float(dropout_p)), None, None
     if Q == 1:
         q2 = query.reshape(B * Hq, D)  # [B,Hq,1,D]: row seg*G+g is query head h*G+g of batch b
         if not q2.is_contiguous():
@@ -361,12 +449,15 @@ def _ragged_common(query, key, value, flash_attn_kwargs, batch_size, num_kv_head
 def batched_dynamic_kv_budget_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                                 attention_mask: Optional[torch.Tensor] = None, scaling: float = None,
                                                 dropout_p: float = 0.0, flash_attn_kwargs: dict = {}, **kwargs):
+    """As in the reference (flash_attn.py:79-151), ``attention_mask``, ``scaling`` and whatever else arrives in ``kwargs``
+    (``sliding_window``, ``is_causal``, ``dropout``) have no effect: the call is causal, unwindowed, scaled by
+    ``D**-0.5``; only ``dropout_p`` reaches the attention."""
     kw = flash_attn_kwargs or {}
-    return _ragged_common(query, key, value, kw, kw.get("batch_size"), kw.get("num_kv_heads"))
+    return _ragged_common(query, key, value, kw, kw.get("batch_size"), kw.get("num_kv_heads"), dropout_p)
 
 
 def dynamic_kv_budget_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                         attention_mask: Optional[torch.Tensor] = None, scaling: float = None,
                                         dropout_p: float = 0.0, flash_attn_kwargs: dict = {}, **kwargs):
     assert query.shape[0] == 1, "Batch size greater than 1 not supported in dynamic KV budget attention."
-    return _ragged_common(query, key, value, flash_attn_kwargs, 1, None)
+    return _ragged_common(query, key, value, flash_attn_kwargs, 1, None, dropout_p)

@@ -1230,13 +1230,17 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
         adaptive = int(total_budget * (1 - floor_budget_ratio))
         _, _, _, chosen, first = self._group_select(layers, H, adaptive, strategy, want_first_kept=True)
         # bucketize against the inclusive cumsum with right=False (cache_utils.py:496): a chosen token that is the FIRST row
-        # of head j >= 1 is counted for head j-1.  first[j] says whether head j's first row was chosen (0 for an empty head);
-        # all of it stays on the device.
+        # of head j >= 1 sits at flat index cu[j-1] and is counted for the first head i with cu[i] == cu[j-1]: the nearest
+        # head before j that holds any token (head 0 when there is none), not simply j-1 -- empty heads in between do not
+        # collect it.  first[j] says whether head j's first row was chosen (0 for an empty head); all of it stays on the device.
         chosen = chosen.reshape(-1).to(torch.int64)          # per (layer, head), flattened in the reference's order
         moved = first.reshape(-1).to(torch.int64)
         moved[0] = 0
+        held = torch.cat([self._slabs[l].seg_len for l in layers]) > 0
+        where = torch.arange(held.numel(), device=held.device)
+        last_held = torch.cummax(torch.where(held, where, torch.full_like(where, -1)), dim=0).values   # nearest head <= i that holds tokens
         credited = chosen - moved
-        credited[:-1] += moved[1:]
+        credited.index_add_(0, last_held[:-1].clamp_min(0), moved[1:])
         head_cnt = (credited + int(memory_size * floor_budget_ratio)).to(torch.int32)
         if len(layers) > 1 and self._layers_alike(layers):   # k >= len keeps all (:514-516)
             self._evict_layers(layers, 0, head_cnt.view(len(layers), H), 0, self._strategy_code(strategy), _lib.ROUND_NATIVE, 0,

@@ -895,6 +895,9 @@ static int group_threshold_common(const char* fn, int per_layer, const void* con
     if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0) return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
     if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0 || nseg % segs_per_group || cap <= 0 || head_dim <= 0)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d segs_per_group=%d cap=%d head_dim=%d", fn, nlayers, nseg, segs_per_group, cap, head_dim);
+    // the knorm term reads K rows as 16-byte pieces: rows (head_dim 16-bit elements) must be whole pieces, and so aligned
+    if (strategy == TRIMKV_SCORE_KNORM_ALPHA && lpr_shift_of(head_dim * 2) < 0)
+        return fail(TRIMKV_ERR_UNSUPPORTED, "%s: knorm_alpha needs head_dim to be a multiple of 8, at most 512 (got %d)", fn, head_dim);
     GroupArgs a;
     a.lb_slabs = lb_slabs; a.pos_slabs = pos_slabs; a.k_slabs = strategy == TRIMKV_SCORE_KNORM_ALPHA ? k_slabs : nullptr; a.seg_lens = seg_lens;
     a.nlayers = nlayers; a.nseg = nseg; a.segs_per_group = segs_per_group; a.cap = cap; a.row_bytes = head_dim * 2;
@@ -939,6 +942,9 @@ extern "C" int trimkv_group_threshold_wide(const void* const* lb_slabs, const in
     if (dtype_bytes(kv_dtype) != 2 || dtype_bytes(lb_dtype) == 0) return fail(TRIMKV_ERR_DTYPE, "%s: kv_dtype must be bf16/f16 and lb_dtype f32/bf16/f16", fn);
     if (nlayers <= 0 || nseg <= 0 || segs_per_group <= 0 || nseg % segs_per_group || cap <= 0 || head_dim <= 0)
         return fail(TRIMKV_ERR_SHAPE, "%s: bad sizes nlayers=%d nseg=%d segs_per_group=%d cap=%d head_dim=%d", fn, nlayers, nseg, segs_per_group, cap, head_dim);
+    // the knorm term reads K rows as 16-byte pieces: rows (head_dim 16-bit elements) must be whole pieces, and so aligned
+    if (strategy == TRIMKV_SCORE_KNORM_ALPHA && lpr_shift_of(head_dim * 2) < 0)
+        return fail(TRIMKV_ERR_UNSUPPORTED, "%s: knorm_alpha needs head_dim to be a multiple of 8, at most 512 (got %d)", fn, head_dim);
     const int ngroups = nseg / segs_per_group;
     if (nlayers > 65535 || ngroups > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: nlayers=%d or groups=%d exceeds the grid limit 65535", fn, nlayers, ngroups);
     const size_t need = trimkv_group_threshold_workspace(nlayers, nseg, segs_per_group);
