@@ -407,6 +407,35 @@ int trimkv_append_attend_pieces(const void* q, void* out,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * trimkv_append_attend_gated / trimkv_append_attend_pieces_gated -- trimkv_append_attend(_pieces) whose new row takes its
+ * log beta from the retention gate's partial sums instead of a finished tensor: the second linear's slice sum, the bias,
+ * the logsigmoid (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:177-179, called at :332-333 before update at :353) and
+ * the roundings of a 16-bit module happen inside the launch that appends and attends, as in trimkv_append_gated, and the
+ * stored bits are the same as that call's.  gate_part: [gate_nslice][nseg / kv_heads][kv_heads] fp32 as written by
+ * trimkv_gate_hidden(_swiglu) for ONE token per batch element, gate_nslice = trimkv_gate_slices(inter) <= 64
+ * (TRIMKV_ERR_UNSUPPORTED beyond: use trimkv_append_gated + trimkv_decode_attn); gate_bias: [kv_heads] fp32.  The other
+ * arguments are those of trimkv_append_attend / trimkv_append_attend_pieces without lb_new and its strides.
+ */
+int trimkv_append_attend_gated(const void* q, void* out,
+                               void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                               const int32_t* seg_order, int nseg, int kv_heads, int cap, int head_dim, int group,
+                               int kv_dtype, int lb_dtype,
+                               const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                               const float* gate_part, int gate_nslice, const float* gate_bias,
+                               const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                               float scale, int max_len_after, int chunk,
+                               void* workspace, size_t workspace_bytes, void* stream);
+int trimkv_append_attend_pieces_gated(const void* q, void* out,
+                                      void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                      const int32_t* pieces, int npieces, int nseg, int kv_heads, int cap, int head_dim, int group,
+                                      int kv_dtype, int lb_dtype,
+                                      const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                      const float* gate_part, int gate_nslice, const float* gate_bias,
+                                      const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                      float scale, int max_len_after,
+                                      void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * trimkv_plan_attn_pieces -- builds the piece list of the two entry points above on the HOST (no GPU work, nothing
  * is launched; seg_len and pieces are host pointers).  It replaces nothing in the reference, whose varlen kernel
  * schedules its own blocks (flash_attn_varlen_func, src/trimkv/attn/flash_attn.py:61-71); it exists because the best cut

@@ -122,3 +122,115 @@ def test_fp16_gates_run_fused(kind):
     a.update(k, k, lazy.transpose(1, 2), torch.arange(S, device=DEV), 0)
     b.update(k, k, lazy.transpose(1, 2).materialize(), torch.arange(S, device=DEV), 0)
     assert a.retention_weights[0].dtype == torch.float16 and torch.equal(a.retention_weights[0], b.retention_weights[0])
+
+
+class _Mod:
+    training = False
+
+
+@pytest.mark.parametrize("B,H,G,hidden,dtype,prefill,M,buf", [
+    (64, 8, 4, 4096, torch.bfloat16, 300, 256, 16),     # the Qwen3-8B gate shape: 512 segments, one workgroup each
+    (2, 2, 4, 1024, torch.bfloat16, 700, 512, 16),      # 4 segments: split-K + merge launch advances the lengths
+    (16, 8, 2, 2048, torch.float16, 900, 768, 8),       # 128 segments: piece list, two pieces per segment merged in the launch
+    (1, 8, 5, 512, torch.bfloat16, 300, 256, 32),       # G = 5: the new row is written after the streaming loop
+    (3, 4, 8, 1024, torch.bfloat16, 40, 32, 4)])
+def test_fused_step_with_a_lazy_log_beta_equals_the_separate_launches(B, H, G, hidden, dtype, prefill, M, buf):
+    """``fuse_decode_append`` with the fused gate: update() defers the row together with the gate's partial sums and the
+    attention launch finishes the gate, appends and attends (trimkv_append_attend_gated / _pieces_gated).  Outputs and all
+    four slabs must be bit-identical to the unfused cache (trimkv_append_gated, then trimkv_decode_attn) over eviction
+    cycles, and log beta equal to materialize()."""
+    from trimkv_amd import LazyLogBeta, TrimKVCache, get_attention_interface
+    from trimkv_amd.gate import RetentionGate
+    attn = get_attention_interface("trimkv_hip")
+    torch.manual_seed(B + G)
+    g = RetentionGate(hidden, H, 512, bias_init=3.0, initializer_range=0.05)
+    g.linear1.bias.data.normal_(0, 0.1)
+    g = g.to(dtype).eval().to(DEV)
+    gen = torch.Generator().manual_seed(B * 10 + G)
+    plain, fused = TrimKVCache(), TrimKVCache()
+    fused.fuse_decode_append = True
+    T, carried = 0, 0
+    for S in [prefill] + [1] * (2 * buf + 3):
+        pos = torch.arange(T, T + S, device=DEV)
+        k, v = draw_kv(gen, B, H, S, dtype=dtype)
+        k, v = k.to(DEV), v.to(DEV)
+        x = torch.randn(B, S, hidden, generator=gen).to(dtype).to(DEV)
+        lazy = g(x).transpose(1, 2)
+        assert isinstance(lazy, LazyLogBeta)
+        Kp, Vp, _, _, kwp = plain.update(k, v, lazy, pos, 0)
+        Kf, Vf, _, _, kwf = fused.update(k, v, lazy, pos, 0)
+        if S == 1:
+            assert "pending_append" in kwf and fused._slabs[0].pending is not None, "a lazy log beta must not switch the fusion off"
+            q = torch.randn(B, H * G, 1, 128, generator=gen).to(dtype).to(DEV)
+            want, _, _ = attn(_Mod(), q, Kp, Vp, None, scaling=128 ** -0.5, flash_attn_kwargs=kwp)
+            got, _, _ = attn(_Mod(), q, Kf, Vf, None, scaling=128 ** -0.5, flash_attn_kwargs=kwf)
+            assert fused._slabs[0].pending is None
+            assert torch.equal(got, want), "gated fused launch differs from append_gated + attend"
+            n = fused.get_cache_length(0)
+            assert torch.equal(fused._slabs[0].lb[:, n - 1].view(B, H), lazy.materialize()[:, :, 0])
+            carried += 1
+        T += S
+        plain.compress("alpha", M, buf)
+        fused.compress("alpha", M, buf)
+        assert fused.get_cache_length(0) == plain.get_cache_length(0)
+        for a, b in zip(fused[0], plain[0]):
+            assert torch.equal(a, b)
+        assert torch.equal(fused._slabs[0].seg_len, plain._slabs[0].seg_len)
+    assert carried == 2 * buf + 3
+
+
+@pytest.mark.parametrize("G", [2, 4, 6])
+def test_ragged_fused_step_with_a_lazy_log_beta(G):
+    """The same on the ragged cache with per-head budgets: planned piece lists, trimkv_append_attend_pieces_gated."""
+    import numpy as np
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, get_attention_interface
+    from trimkv_amd.gate import RetentionGate
+    attn = get_attention_interface("db_attn_flash_batched")
+    B, H, hidden, buf = 4, 4, 1024, 8
+    torch.manual_seed(G)
+    g = RetentionGate(hidden, H, 256, bias_init=3.0, initializer_range=0.05).to(torch.bfloat16).eval().to(DEV)
+    rng = np.random.default_rng(G)
+    budgets = np.clip(np.round(np.exp(rng.normal(np.log(200), 1.2, size=B * H))), 4, 2500).astype(np.int64)
+    gen = torch.Generator().manual_seed(G)
+    plain, fused = BatchedDynamicBudgetTrimKVCache(), BatchedDynamicBudgetTrimKVCache()
+    fused.fuse_decode_append = True
+    for c in (plain, fused):
+        c.set_budgets(budgets)
+    S0 = 2600
+    k, v = draw_kv(gen, B, H, S0)
+    x = torch.randn(B, S0, hidden, generator=gen).to(torch.bfloat16).to(DEV)
+    lazy = g(x).transpose(1, 2)
+    for c in (plain, fused):
+        c.update(k.to(DEV), v.to(DEV), lazy, torch.arange(S0, device=DEV), 0)
+        c.evict_to_budgets(buffer_size=0)
+    T = S0
+    for t in range(3 * buf):
+        pos = torch.arange(T, T + 1, device=DEV)
+        kn, vn = draw_kv(gen, B, H, 1)
+        lazy = g(torch.randn(B, 1, hidden, generator=gen).to(torch.bfloat16).to(DEV)).transpose(1, 2)
+        q = torch.randn(B, H * G, 1, 128, generator=gen).to(torch.bfloat16).to(DEV)
+        op = plain.update(kn.to(DEV), vn.to(DEV), lazy, pos, 0)
+        of = fused.update(kn.to(DEV), vn.to(DEV), lazy, pos, 0)
+        assert "pending_append" in of[4]
+        want, _, _ = attn(_Mod(), q, op[0], op[1], None, flash_attn_kwargs=op[4])
+        got, _, _ = attn(_Mod(), q, of[0], of[1], None, flash_attn_kwargs=of[4])
+        assert torch.equal(got, want) and fused._slabs[0].pending is None
+        T += 1
+        for c in (plain, fused):
+            c.evict_to_budgets(buffer_size=buf)
+        assert torch.equal(fused.head_lens[0], plain.head_lens[0]) and torch.equal(fused.cu_seqlens_k[0], plain.cu_seqlens_k[0])
+    for name in ("key_cache", "value_cache", "retention_weights", "kv_positions"):
+        assert torch.equal(getattr(fused, name)[0], getattr(plain, name)[0])
+
+
+def test_gated_append_attend_refuses_more_than_64_slices():
+    import ctypes
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    one = ctypes.c_void_p(256)
+    call = lambda nslice, part=one: lib.trimkv_append_attend_gated(one, one, one, one, one, one, one, None, None, 8, 2, 64, 128, 4, L.BF16, L.BF16,
+                                                                   one, one, 256, 128, part, nslice, one, one, 0, 0, 0.1, 64, 0, None, 0, None)
+    assert call(65) == -6 and call(0) == -6 and call(32, part=None) == -1
+    pieces = lambda nslice: lib.trimkv_append_attend_pieces_gated(one, one, one, one, one, one, one, None, one, 4, 8, 2, 64, 128, 4, L.BF16, L.BF16,
+                                                                  one, one, 256, 128, one, nslice, one, one, 0, 0, 0.1, 64, one, 1 << 20, None)
+    assert pieces(65) == -6

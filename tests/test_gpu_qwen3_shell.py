@@ -175,3 +175,44 @@ def test_shell_generate_chunked_prompt_and_ragged_cache():
     total = cache.get_total_cached_tokens()
     assert total <= 2 * cfg2.num_hidden_layers * cfg2.num_key_value_heads * (cfg2.memory_size + cfg2.buffer_size)
     assert len(set(cache.head_lens[0].tolist())) > 1                   # the shared budget left the heads ragged
+
+
+@pytest.mark.parametrize("gate", ["rg", "rg2", "rg3"])
+def test_shell_decode_keeps_one_launch_per_layer_with_the_fused_gate(gate):
+    """The model shell switches ``fuse_decode_append`` on, and the fused gates hand update() a LazyLogBeta at every real
+    hidden size: the deferred append must engage all the same (the attention launch finishes the gate), and the logits
+    must equal, bit for bit, those of a run whose cache appends in a launch of its own."""
+    from trimkv_amd import LazyLogBeta, TrimKVCache
+    torch.manual_seed(3)
+    cfg = _tiny_config("qwen3", retention_gate=gate)
+    assert cfg.hidden_size % 512 == 0
+    model = _family("qwen3")[1](cfg).to(torch.bfloat16).to(DEV).eval()
+    B, P, STEPS = 2, 70, 24
+    ids = torch.randint(0, cfg.vocab_size, (B, P + STEPS), generator=torch.Generator().manual_seed(4)).to(DEV)
+    runs = {}
+    for fuse in (True, False):
+        cache = TrimKVCache()
+        cache.fuse_decode_append = fuse
+        deferred = []
+        inner = cache.update
+
+        def update(k, v, rw, pos, l, kw=None, inner=inner, deferred=deferred):
+            out = inner(k, v, rw, pos, l, kw)
+            if k.shape[2] == 1:
+                deferred.append(isinstance(rw, LazyLogBeta) and "pending_append" in out[4])
+            return out
+
+        cache.update = update
+        logits = []
+        with torch.no_grad():
+            out = model(ids[:, :P], past_key_values=cache)
+            for t in range(STEPS):
+                out = model(ids[:, P + t:P + t + 1], past_key_values=cache)
+                logits.append(out.logits)
+                assert all(s is None or s.pending is None for s in cache._slabs)     # every attention call carried its append out
+        runs[fuse] = (torch.cat(logits, dim=1), deferred, [cache.kv_positions[l].clone() for l in range(cfg.num_hidden_layers)])
+    assert len(runs[True][1]) == STEPS * cfg.num_hidden_layers and all(runs[True][1]), "the fused gate switched the one-launch step off"
+    assert not any(runs[False][1])
+    assert torch.equal(runs[True][0], runs[False][0])
+    for a, b in zip(runs[True][2], runs[False][2]):
+        assert torch.equal(a, b)

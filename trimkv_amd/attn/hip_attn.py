@@ -154,24 +154,26 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
     nseg, d = slab.B * slab.H, slab.D
     out = torch.empty_like(query)
     st = _lib.current_stream(query.device)
+    # a log beta that the retention gate left unfinished (LazyLogBeta) is finished by the same launch: the gated entry points
+    gated = not torch.is_tensor(slab.pending[3])
     if pieces is not None:   # ragged lengths: one launch over the (segment, piece) list, merged inside it
         plist, npieces = pieces
         ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(npieces, group), st)
-        rc = lib.trimkv_append_attend_pieces(query.data_ptr(), out.data_ptr(), *slab.ptrs, plist.data_ptr(), npieces,
-                                             nseg, slab.H, slab.cap, d, group, *slab.codes, *slab.pending[0],
-                                             scale, slab.max_len, ws.data_ptr(), ws.numel(), st)
+        fn = lib.trimkv_append_attend_pieces_gated if gated else lib.trimkv_append_attend_pieces
+        rc = fn(query.data_ptr(), out.data_ptr(), *slab.ptrs, plist.data_ptr(), npieces, nseg, slab.H, slab.cap, d, group, *slab.codes,
+                *slab.pending[0], scale, slab.max_len, ws.data_ptr(), ws.numel(), st)
         if rc:
-            _lib.check(rc, "trimkv_append_attend_pieces")
+            _lib.check(rc, "trimkv_append_attend_pieces_gated" if gated else "trimkv_append_attend_pieces")
         slab.pending = None
         return out
     ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, slab.max_len, chunk)
     ws = _workspace(query.device, ws_bytes, st) if ws_bytes else None
     # slab.pending[0] = the new row's addresses and strides, in the order of the entry point's parameters
-    rc = lib.trimkv_append_attend(query.data_ptr(), out.data_ptr(), *slab.ptrs, None if seg_order is None else seg_order.data_ptr(),
-                                  nseg, slab.H, slab.cap, d, group, *slab.codes, *slab.pending[0],
-                                  scale, slab.max_len, chunk, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
+    fn = lib.trimkv_append_attend_gated if gated else lib.trimkv_append_attend
+    rc = fn(query.data_ptr(), out.data_ptr(), *slab.ptrs, None if seg_order is None else seg_order.data_ptr(), nseg, slab.H, slab.cap, d, group,
+            *slab.codes, *slab.pending[0], scale, slab.max_len, chunk, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
     if rc:
-        _lib.check(rc, "trimkv_append_attend")
+        _lib.check(rc, "trimkv_append_attend_gated" if gated else "trimkv_append_attend")
     slab.pending = None
     return out
 

@@ -199,15 +199,25 @@ class _SlabBacked(_CacheBase):
         (``_flush``).  Returns False when this update cannot be deferred (the ordinary append runs then)."""
         if slab.pending is not None:
             self._flush(slab)
-        if isinstance(lb, LazyLogBeta) or not (k.is_cuda and lb.is_cuda):
+        lazy = isinstance(lb, LazyLogBeta)
+        if not k.is_cuda or not (lazy or lb.is_cuda):
             return False
         B, H, D = slab.B, slab.H, slab.D
         if tuple(k.shape) != (B, H, 1, D) or v.shape != k.shape or v.dtype != k.dtype or k.dtype != slab.k.dtype:
             return False
         if tuple(lb.shape) != (B, H, 1) or lb.dtype != slab.lb.dtype:
             return False
-        ks = k.stride()
-        if ks[3] != 1 or (ks[0] | ks[1]) % 8 or v.stride() != ks or (k.data_ptr() | v.data_ptr()) % 16:
+        if lazy:
+            # the gate's partial sums [slices, B, Hkv]: the attention launch finishes them (trimkv_append_attend_gated),
+            # one slice per lane
+            part = lb.part
+            if not lb.transposed or part.shape[0] > 64 or tuple(part.shape[1:]) != (B, H) or not part.is_contiguous():
+                return False
+            lb_args = (part.data_ptr(), part.shape[0], lb.bias_f32.data_ptr())
+        else:
+            lb_args = (lb.data_ptr(), lb.stride(0), lb.stride(1))
+        ks, vs = k.stride(), v.stride()   # the stride over the single new token does not matter
+        if ks[3] != 1 or (ks[0] | ks[1]) % 8 or (vs[0], vs[1], vs[3]) != (ks[0], ks[1], ks[3]) or (k.data_ptr() | v.data_ptr()) % 16:
             return False
         if pos.dtype != torch.int64 or pos.device != k.device:
             return False
@@ -219,9 +229,10 @@ class _SlabBacked(_CacheBase):
             return False
         if slab.max_len + 1 > slab.cap:
             slab.regrow(self._new_capacity(slab, slab.max_len + 1, 1))
-        # [0]: what trimkv_append_attend needs of the new row (addresses, element strides over batch and head);
-        # [1:]: the tensors themselves, kept alive and used by _flush
-        slab.pending = ((k.data_ptr(), v.data_ptr(), ks[0], ks[1], lb.data_ptr(), lb.stride(0), lb.stride(1), pos.data_ptr(), ps[0], ps[1]),
+        # [0]: what trimkv_append_attend(_gated) needs of the new row (addresses, element strides over batch and head; for a
+        # lazy log beta the partial sums, their slice count and the bias); [1:]: the tensors themselves, kept alive and
+        # used by _flush
+        slab.pending = ((k.data_ptr(), v.data_ptr(), ks[0], ks[1], *lb_args, pos.data_ptr(), ps[0], ps[1]),
                         k, v, lb, pos)
         slab.lens += 1
         slab.max_len += 1

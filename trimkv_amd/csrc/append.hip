@@ -21,11 +21,6 @@ struct AppendArgs {
     const int64_t* pos_new; int64_t pos_sb, pos_sh, pos_ss;              // element strides
 };
 
-__device__ __forceinline__ float log_sigmoid(float x) {
-    // min(x, 0) - log1p(exp(-|x|)), the formulation torch uses
-    return fminf(x, 0.0f) - log1pf(__expf(-fabsf(x)));
-}
-
 template <bool GATED>
 __global__ __launch_bounds__(AP_THREADS) void append_kernel(AppendArgs a) {
     const int seg = blockIdx.x;

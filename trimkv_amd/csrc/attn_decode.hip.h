@@ -110,7 +110,21 @@ struct AppendPart {
     const int64_t* pos_new; int64_t pos_sb, pos_sh;
     void* lb_slab; int64_t* pos_slab; int32_t* seg_len; int32_t* cu;
     int kv_heads, lb_dtype;
+    // GATED kernels only: log beta of the new row is finished here from the retention gate's per-slice partial sums
+    // [gate_nslice][batch][kv_heads] (gate_nslice <= 64) and its bias [kv_heads], instead of being read from lb_new
+    const float* gate_part; const float* gate_bias; int gate_nslice;
 };
+
+// log(beta) of one new row from the gate's partial sums, by a whole wavefront: lane j holds the partial of slice j (0 beyond
+// the last slice), a fixed butterfly adds them, then bias and logsigmoid with the roundings of a 16-bit torch module --
+// the same operations in the same order as append_small_kernel<true>, so both paths store the same bits.
+__device__ __forceinline__ float finish_gate(float partial, float bias, int lb_dtype) {
+    float acc = 0.0f + partial;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) acc += __shfl_xor(acc, d, 64);
+    acc = round_to_dtype(acc, lb_dtype);
+    return log_sigmoid(round_to_dtype(acc + bias, lb_dtype));
+}
 
 struct AttnArgs {
     const uint4* q; void* out; const uint4* k; const uint4* v;
@@ -164,7 +178,8 @@ __device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new
 // APPEND: row `new_row` of the segment (-1: none) is this step's token.  It is read from a.ap.k_new / v_new wherever the
 // stream reaches it, and the wavefront that owns it writes it into the slabs (K, V, log beta, position).
 // COHERENT: the partials are read by another workgroup of this same launch (see store_shared_partial).
-template <int G, int ROW16, bool F16, bool APPEND, bool COHERENT = false>
+// GATED (with APPEND): log beta of the new row comes from the retention gate's partial sums (finish_gate), not from lb_new.
+template <int G, int ROW16, bool F16, bool APPEND, bool COHERENT = false, bool GATED = false>
 __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base, int new_row) {
     constexpr int D_REAL = ROW16 * 8;
     using C = AttnCfg<G>;
@@ -206,9 +221,10 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     const uint4* knew = nullptr;
     const uint4* vnew = nullptr;
     uint4 kn = make_uint4(0u, 0u, 0u, 0u), vn = kn;
-    float lbn = 0.0f;
+    float lbn = 0.0f, gate_bias = 0.0f;
     int64_t pn = 0;
     int64_t lb_off = 0, pos_off = 0;
+    const float* gate_src = nullptr;   // GATED: this lane's slice of the gate's partial sums for the new row (clamped to the last slice)
     if (APPEND) {
         const int b = seg / a.ap.kv_heads, h = seg - b * a.ap.kv_heads;
         const int64_t off = (int64_t)b * a.ap.kv_sb + (int64_t)h * a.ap.kv_sh + ((int64_t)cc << 4);
@@ -216,10 +232,12 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         vnew = (const uint4*)(a.ap.v_new + off);
         lb_off = (int64_t)b * a.ap.lb_sb + (int64_t)h * a.ap.lb_sh;
         pos_off = (int64_t)b * a.ap.pos_sb + (int64_t)h * a.ap.pos_sh;
+        if (GATED) gate_src = a.ap.gate_part + ((int64_t)min(lane, a.ap.gate_nslice - 1) * (a.nseg / a.ap.kv_heads) + b) * a.ap.kv_heads + h;
         if (APPEND_EARLY) {
             kn = *knew;
             vn = *vnew;
-            lbn = load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype);
+            if (GATED) { lbn = *gate_src; gate_bias = a.ap.gate_bias[h]; }   // unconditional, like the row itself
+            else lbn = load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype);
             pn = a.ap.pos_new[pos_off];
         }
     }
@@ -389,6 +407,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
                 ((uint4*)a.k)[dst * ROW16 + c] = kn;
                 ((uint4*)a.v)[dst * ROW16 + c] = vn;
             }
+            if (GATED) lbn = finish_gate(lane < a.ap.gate_nslice ? lbn : 0.0f, gate_bias, a.ap.lb_dtype);
             if (lane == 0) {
                 store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
                 a.ap.pos_slab[dst] = pn;
@@ -421,8 +440,13 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             ((uint4*)a.k)[dst * ROW16 + c] = kn;
             ((uint4*)a.v)[dst * ROW16 + c] = vn;
         }
+        if (GATED) {
+            const int h = seg % a.ap.kv_heads;
+            const float partial = *gate_src;
+            lbn = finish_gate(lane < a.ap.gate_nslice ? partial : 0.0f, a.ap.gate_bias[h], a.ap.lb_dtype);
+        }
         if (lane == 0) {
-            store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype));
+            store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, GATED ? lbn : load_as_f32(a.ap.lb_new, lb_off, a.ap.lb_dtype));
             a.ap.pos_slab[dst] = a.ap.pos_new[pos_off];
         }
     }
@@ -485,7 +509,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     }
 }
 
-template <int G, int ROW16, bool F16, bool APPEND>
+template <int G, int ROW16, bool F16, bool APPEND, bool GATED = false>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_kernel(AttnArgs a) {
     // Workgroups are handed to the 8 XCDs round-robin by linear id.  The segment is the fast grid
     // axis so that consecutive ids are different segments: with the split as the fast axis and 8
@@ -510,14 +534,14 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     }
     const int rps = (live + nsp - 1) / nsp;
     const int t0 = first + split * rps, t1 = min(n, t0 + rps);
-    attend_rows<G, ROW16, F16, APPEND>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split, new_row);
+    attend_rows<G, ROW16, F16, APPEND, false, GATED>(a, seg, t0, t1, a.direct != 0, (int64_t)seg * a.nsplit + split, new_row);
 }
 
 // Piece-list launch: one workgroup per entry of a.pieces, in the order of the list (the caller sorts it so that every
 // compute unit receives about the same number of rows), and no second launch: a segment cut into several pieces is
 // merged by whichever of its workgroups finishes last.  Every workgroup of the grid works on a piece, so once a segment's
 // counter is full nobody will read its length again and the merging workgroup may advance it (APPEND).
-template <int G, int ROW16, bool F16, bool APPEND>
+template <int G, int ROW16, bool F16, bool APPEND, bool GATED = false>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_pieces_kernel(AttnArgs a) {
     __shared__ int last_of_segment;
     const int4 e = a.pieces[blockIdx.x];
@@ -541,7 +565,7 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
     const int64_t slot0 = e.w;
     // one instantiation for both cases (a second inlined copy of the streaming loop costs registers): a segment in one
     // piece writes its output itself, the others leave partials
-    attend_rows<G, ROW16, F16, APPEND, true>(a, seg, t0, t1, nsp == 1, slot0 + piece, new_row);
+    attend_rows<G, ROW16, F16, APPEND, true, GATED>(a, seg, t0, t1, nsp == 1, slot0 + piece, new_row);
     if (nsp == 1) return;
     // every thread waits until its own partial stores have been acknowledged (they are write-through stores: the
     // acknowledgement comes from memory), only then may the counter move
@@ -658,50 +682,50 @@ static int pick_chunk(int nseg, int max_len) {
     return chunk < whole ? chunk : whole;
 }
 
-template <int G, int ROW16, bool F16, bool APPEND>
+template <int G, int ROW16, bool F16, bool APPEND, bool GATED>
 static void launch_attn_rows(const AttnArgs& a, hipStream_t st) {
-    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16, F16, APPEND>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
+    hipLaunchKernelGGL((decode_attn_kernel<G, ROW16, F16, APPEND, GATED>), dim3(a.nseg, a.nsplit), dim3(AT_THREADS), 0, st, a);
     if (!a.direct) hipLaunchKernelGGL((decode_attn_merge_kernel<G, ROW16, F16, APPEND>), dim3(a.nseg), dim3(G * AT_D), 0, st, a);
 }
 
-template <int G, bool F16, bool APPEND>
+template <int G, bool F16, bool APPEND, bool GATED>
 static void launch_attn_dtype(const AttnArgs& a, int head_dim, hipStream_t st) {
-    if (head_dim == 128) launch_attn_rows<G, 16, F16, APPEND>(a, st);
-    else if (head_dim == 96) launch_attn_rows<G, 12, F16, APPEND>(a, st);
-    else launch_attn_rows<G, 8, F16, APPEND>(a, st);
+    if (head_dim == 128) launch_attn_rows<G, 16, F16, APPEND, GATED>(a, st);
+    else if (head_dim == 96) launch_attn_rows<G, 12, F16, APPEND, GATED>(a, st);
+    else launch_attn_rows<G, 8, F16, APPEND, GATED>(a, st);
 }
 
-template <int G, bool APPEND>
+template <int G, bool APPEND, bool GATED>
 static void launch_attn(const AttnArgs& a, int head_dim, int dtype, hipStream_t st) {
-    if (dtype == TRIMKV_F16) launch_attn_dtype<G, true, APPEND>(a, head_dim, st);
-    else launch_attn_dtype<G, false, APPEND>(a, head_dim, st);
+    if (dtype == TRIMKV_F16) launch_attn_dtype<G, true, APPEND, GATED>(a, head_dim, st);
+    else launch_attn_dtype<G, false, APPEND, GATED>(a, head_dim, st);
 }
 
-template <int G, bool APPEND>
+template <int G, bool APPEND, bool GATED>
 static void launch_attn_pieces(const AttnArgs& a, int npieces, int head_dim, int dtype, hipStream_t st) {
     const dim3 grid(npieces), block(AT_THREADS);
     if (dtype == TRIMKV_F16) {
-        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, true, APPEND>), grid, block, 0, st, a);
-        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, true, APPEND>), grid, block, 0, st, a);
-        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, true, APPEND>), grid, block, 0, st, a);
+        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, true, APPEND, GATED>), grid, block, 0, st, a);
+        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, true, APPEND, GATED>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, true, APPEND, GATED>), grid, block, 0, st, a);
     } else {
-        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, false, APPEND>), grid, block, 0, st, a);
-        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, false, APPEND>), grid, block, 0, st, a);
-        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, false, APPEND>), grid, block, 0, st, a);
+        if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, false, APPEND, GATED>), grid, block, 0, st, a);
+        else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, false, APPEND, GATED>), grid, block, 0, st, a);
+        else hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 8, false, APPEND, GATED>), grid, block, 0, st, a);
     }
 }
 
-template <bool APPEND>
+template <bool APPEND, bool GATED = false>
 static void launch_attn_pieces_group(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st) {
     switch (group) {
-        case 1: launch_attn_pieces<1, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 2: launch_attn_pieces<2, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 3: launch_attn_pieces<3, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 4: launch_attn_pieces<4, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 5: launch_attn_pieces<5, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 6: launch_attn_pieces<6, APPEND>(a, npieces, head_dim, dtype, st); break;
-        case 7: launch_attn_pieces<7, APPEND>(a, npieces, head_dim, dtype, st); break;
-        default: launch_attn_pieces<8, APPEND>(a, npieces, head_dim, dtype, st); break;
+        case 1: launch_attn_pieces<1, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 2: launch_attn_pieces<2, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 3: launch_attn_pieces<3, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 4: launch_attn_pieces<4, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 5: launch_attn_pieces<5, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 6: launch_attn_pieces<6, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        case 7: launch_attn_pieces<7, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
+        default: launch_attn_pieces<8, APPEND, GATED>(a, npieces, head_dim, dtype, st); break;
     }
 }
 
@@ -733,17 +757,17 @@ static int prepare_pieces(const char* fn, AttnArgs& a, const int32_t* pieces, in
 }
 
 // group = 1..8 -> the matching instantiation
-template <bool APPEND>
+template <bool APPEND, bool GATED = false>
 static void launch_attn_group(const AttnArgs& a, int group, int head_dim, int dtype, hipStream_t st) {
     switch (group) {
-        case 1: launch_attn<1, APPEND>(a, head_dim, dtype, st); break;
-        case 2: launch_attn<2, APPEND>(a, head_dim, dtype, st); break;
-        case 3: launch_attn<3, APPEND>(a, head_dim, dtype, st); break;
-        case 4: launch_attn<4, APPEND>(a, head_dim, dtype, st); break;
-        case 5: launch_attn<5, APPEND>(a, head_dim, dtype, st); break;
-        case 6: launch_attn<6, APPEND>(a, head_dim, dtype, st); break;
-        case 7: launch_attn<7, APPEND>(a, head_dim, dtype, st); break;
-        default: launch_attn<8, APPEND>(a, head_dim, dtype, st); break;
+        case 1: launch_attn<1, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 2: launch_attn<2, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 3: launch_attn<3, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 4: launch_attn<4, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 5: launch_attn<5, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 6: launch_attn<6, APPEND, GATED>(a, head_dim, dtype, st); break;
+        case 7: launch_attn<7, APPEND, GATED>(a, head_dim, dtype, st); break;
+        default: launch_attn<8, APPEND, GATED>(a, head_dim, dtype, st); break;
     }
 }
 

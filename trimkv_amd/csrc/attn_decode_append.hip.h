@@ -17,6 +17,15 @@ static int fill_append_part(const char* fn, AttnArgs& a, void* lb_slab, int64_t*
     return TRIMKV_OK;
 }
 
+// The gated variants: log beta of the new row is finished inside the launch from the retention gate's partial sums.
+static int fill_gate_part(const char* fn, AttnArgs& a, const float* gate_part, int gate_nslice, const float* gate_bias) {
+    if (!gate_part || !gate_bias) return fail(TRIMKV_ERR_NULL, "%s: null gate_part / gate_bias", fn);
+    if (gate_nslice <= 0 || gate_nslice > 64)
+        return fail(TRIMKV_ERR_UNSUPPORTED, "%s: gate_nslice must be in [1, 64] (got %d): one lane per slice finishes the gate", fn, gate_nslice);
+    a.ap.gate_part = gate_part; a.ap.gate_bias = gate_bias; a.ap.gate_nslice = gate_nslice;
+    return TRIMKV_OK;
+}
+
 static int check_append_args(const char* fn, const void* lb_slab, const void* pos_slab, const void* seg_len, const void* k_new, const void* v_new,
                              const void* lb_new, const void* pos_new, int nseg, int kv_heads, int lb_dtype, int64_t kv_stride_b, int64_t kv_stride_h) {
     if (!lb_slab || !pos_slab || !seg_len || !k_new || !v_new || !lb_new || !pos_new) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);

@@ -70,6 +70,11 @@ __device__ __forceinline__ void store_from_f32(void* p, int64_t i, int dt, float
     else ((uint16_t*)p)[i] = f32_to_f16_bits(f);
 }
 
+// min(x, 0) - log1p(exp(-|x|)), the formulation torch uses
+__device__ __forceinline__ float log_sigmoid(float x) {
+    return fminf(x, 0.0f) - log1pf(__expf(-fabsf(x)));
+}
+
 // ---- device: order-preserving key of an fp32 score -------------------------------------------
 // a > b (as floats, -0 == +0) <=> key(a) > key(b); lets a radix select work on unsigned ints.
 __device__ __forceinline__ uint32_t float_key(float s) {
