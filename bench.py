@@ -412,6 +412,97 @@ def ragged_main(args):
     print(json.dumps(out_json))
 
 
+def shell_main(args):
+    """Secondary workload (--shell): decode steps of the thin Qwen3 decoder at the Qwen3-8B layer shape (hidden 4096, 32 query
+    / 8 KV heads, MLP 12288, random bf16 weights, batch 64) on a cache in the steady state of config 3.  It measures what
+    the `rg` retention gate costs a decode step inside a model: gate on a second stream beside the q/k/v projections (the
+    shell's default), gate on the main stream, and no gate at all (log beta a constant tensor), same cache contents."""
+    import torch
+    from trimkv_amd import TrimKVCache
+    from trimkv_amd.qwen3 import TrimKVQwen3Attention, TrimKVQwen3Config, TrimKVQwen3Model
+    c = dict(CONFIGS[3])
+    L = args.layers or c["L"]
+    B, Hkv, Hq, M, buf = c["B"], c["Hkv"], c["Hq"], c["M"], c["buf"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    cfg = TrimKVQwen3Config(vocab_size=1024, hidden_size=args.hidden, intermediate_size=3 * args.hidden, num_hidden_layers=L,
+                            num_attention_heads=Hq, num_key_value_heads=Hkv, head_dim=D, retention_gate="rg",
+                            retention_gate_bias_init=3.0, memory_size=M, buffer_size=buf)
+    torch.manual_seed(0)
+    torch.set_default_dtype(torch.bfloat16)
+    with torch.device(dev):
+        model = TrimKVQwen3Model(cfg)
+    torch.set_default_dtype(torch.float32)
+    for p_ in model.parameters():
+        if p_.dim() > 1:
+            p_.data.normal_(0.0, 0.02)
+    model.eval()
+    gen = torch.Generator(device=dev).manual_seed(0)
+    steps, warm = args.steps, args.warmup
+    n0 = M + max(1, (buf - 6 * (steps + warm) - 2) // 2)     # all runs (three variants, twice) fit inside one eviction cycle
+
+    def fresh_cache():
+        cache = TrimKVCache()
+        cache.fuse_decode_append = True
+        pos0 = torch.arange(n0, device=dev)
+        for l in range(L):
+            k = torch.randn(B, Hkv, n0, D, generator=gen, device=dev).to(torch.bfloat16)
+            v = torch.randn(B, Hkv, n0, D, generator=gen, device=dev).to(torch.bfloat16)
+            lb = torch.nn.functional.logsigmoid(torch.randn(B, Hkv, n0, generator=gen, device=dev) * c["sigma"] + c["mu"]).to(torch.bfloat16)
+            cache.update(k, v, lb, pos0, l)
+            del k, v, lb
+        cache.compress("alpha", M, buf)      # not due: teaches the cache its budget
+        return cache
+
+    cache = fresh_cache()
+    x = torch.randn(B, 1, args.hidden, generator=gen, device=dev).to(torch.bfloat16) * 0.1
+    const_lb = torch.nn.functional.logsigmoid(torch.randn(B, 1, Hkv, generator=gen, device=dev) * c["sigma"] + c["mu"]).to(torch.bfloat16)
+    gates = [layer.self_attn.retention_gate for layer in model.layers]
+
+    class NoGate(torch.nn.Module):
+        def forward(self, hidden):
+            return const_lb
+
+    def run(kind):
+        TrimKVQwen3Attention.gate_on_side_stream = kind == "side"
+        for layer, g in zip(model.layers, gates):
+            layer.self_attn.retention_gate = NoGate() if kind == "none" else g
+        with torch.no_grad():
+            for _ in range(warm):
+                model(inputs_embeds=x, past_key_values=cache)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                model(inputs_embeds=x, past_key_values=cache)
+            enq = time.perf_counter() - t0
+            torch.cuda.synchronize()
+            sec = time.perf_counter() - t0
+        return sec * 1e3 / steps, enq * 1e3 / steps
+
+    res = {}
+    for kind in ("none", "side", "main", "none", "side", "main"):     # two rounds, alternating: the rows grow by one per step
+        ms, enq = run(kind)
+        res.setdefault(kind, []).append((ms, enq))
+    TrimKVQwen3Attention.gate_on_side_stream = True
+    assert cache.get_cache_length(0) < M + buf, "the window must not contain an eviction"
+    best = {k: min(m for m, _ in v) for k, v in res.items()}
+    out = {
+        "metric": "decode ms/step of the thin Qwen3 decoder at the Qwen3-8B layer shape: rg gate beside the projections vs no gate",
+        "value": round(best["side"], 4), "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(best["side"], 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"thin TrimKV Qwen3 decoder, {L} layers of the Qwen3-8B shape (hidden {args.hidden}, {Hq} query / {Hkv} KV heads, "
+                               f"head_dim {D}, MLP {3 * args.hidden}), random bf16 weights, batch {B}, cache of {cache.get_cache_length(0)} rows per head "
+                               f"(memory_size {M}, buffer_size {buf}), fused append + attend, no eviction inside the window",
+                   "note": "secondary workload; the headline metric is the default run"},
+        "gate": {"ms_per_step_gate_on_second_stream": round(best["side"], 4), "ms_per_step_gate_on_main_stream": round(best["main"], 4),
+                 "ms_per_step_without_gate": round(best["none"], 4),
+                 "gate_cost_second_stream_pct": round((best["side"] / best["none"] - 1) * 100, 2),
+                 "gate_cost_main_stream_pct": round((best["main"] / best["none"] - 1) * 100, 2),
+                 "all_runs_ms_and_host_enqueue_ms": {k: [(round(m, 4), round(e, 4)) for m, e in v] for k, v in res.items()}},
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -433,9 +524,15 @@ def main():
                          "kernel) from a random hidden state per layer instead of appending drawn values; reported as a "
                          "variant, the BASELINE configs draw beta directly")
     ap.add_argument("--hidden", type=int, default=4096, help="hidden size for --gate (Qwen3-8B: 4096)")
+    ap.add_argument("--gate-stream", choices=("side", "main"), default="main",
+                    help="with --gate: run the gate's first linear on the main stream in front of the launch that needs it, or on a "
+                         "second stream one layer ahead (overlapping the previous layer's attention launch)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy (a kernel of known traffic) so that rocprofv3 --pmc "
                          "FETCH_SIZE / WRITE_SIZE readings of the same run can be scaled")
+    ap.add_argument("--shell", action="store_true",
+                    help="secondary workload: decode steps of the thin Qwen3 decoder at the Qwen3-8B layer shape, with the rg gate on a "
+                         "second stream, on the main stream and without a gate (defaults: 12 steps, 3 warm-up, per variant)")
     ap.add_argument("--prefill", action="store_true",
                     help="secondary workload: chunked prompt processing at config 5's shape (4096-token chunks); "
                          "with it --steps/--warmup count chunks (defaults 6/2)")
@@ -451,6 +548,10 @@ def main():
         if args.steps == 1024 and args.warmup == 128:
             args.steps, args.warmup = 6, 2
         return prefill_main(args)
+    if args.shell:
+        if args.steps == 1024 and args.warmup == 128:
+            args.steps, args.warmup = 12, 3
+        return shell_main(args)
     if args.config == 4:
         return ragged_main(args)
 
@@ -526,6 +627,21 @@ def main():
 
     scale = D ** -0.5
     use_gate = bool(args.gate)
+    # --gate: where the gate's first linear (trimkv_gate_hidden) runs.  "main": on the main stream, in front of the launch
+    # that needs it (nothing overlaps it).  "side": on a second stream of the same priority, one layer ahead, so that it
+    # may overlap the previous layer's attention launch.
+    gate_side = use_gate and args.gate_stream == "side"
+    main = torch.cuda.current_stream(dev)
+    side = torch.cuda.Stream(device=dev) if gate_side else None
+    gate_done = [torch.cuda.Event() for _ in range(L)] if gate_side else []
+    lazies = [None] * L
+
+    def issue_gate(l):
+        with torch.cuda.stream(side):
+            lazy = gates[l](hidden_pool[l])
+        gate_done[l].record(side)
+        lazy.part.record_stream(main)
+        lazies[l] = lazy.transpose(1, 2)
 
     def layers_pass(sample):
         """Append + attend for every layer: one decode step without its eviction.  Returns the bytes it had to move.
@@ -534,10 +650,18 @@ def main():
         pos = torch.full((1,), T, dtype=torch.int64, device=dev)
         slot = tick % POOL
         update = cache.update
+        if gate_side:   # the first layer's gate: after everything the previous step enqueued
+            side.wait_stream(main)
+            issue_gate(0)
         for l in range(L):
             kn, vn, lbn, q = pool[l][slot]
-            if use_gate:
-                lbn = gates[l](hidden_pool[l]).transpose(1, 2)   # LazyLogBeta: finished inside the append kernel
+            if gate_side:
+                main.wait_event(gate_done[l])
+                lbn = lazies[l]
+                if l + 1 < L:
+                    issue_gate(l + 1)     # runs on the second stream while this layer appends and attends
+            elif use_gate:
+                lbn = gates[l](hidden_pool[l]).transpose(1, 2)   # LazyLogBeta: finished inside the launch that appends
             K, V, _, _, kw = update(kn, vn, lbn, pos, l)
             if sample:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -609,12 +733,13 @@ def main():
         durs = [e0.elapsed_time(e1) * 1e-3 for e0, e1, _ in events]
         lens = [n for _, _, n in events]
         avg_s = sum(durs) / len(durs)
-        fused = cache.fuse_decode_append and not args.gate   # the sampled launch then also writes the new rows
+        fused = cache.fuse_decode_append   # the sampled launch then also writes the new rows
         avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens) + (append_bytes if fused else 0)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
-        targs = f"<{G}, 16, false, {'true' if fused else 'false'}>"
-        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 256 else " + decode_attn_merge_kernel" + targs), "achieved": round(achieved, 1),
+        merge_targs = f"<{G}, 16, false, {'true' if fused else 'false'}>"
+        targs = merge_targs[:-1] + (", true>" if fused and args.gate else ">")    # GATED instantiation when the launch finishes the gate
+        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 256 else " + decode_attn_merge_kernel" + merge_targs), "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "traffic_measured_in_run": False,
@@ -641,8 +766,10 @@ def main():
                                f"head_dim {D}, memory_size {M}, buffer_size {buf}, steady-state decode (append + attend per layer, "
                                f"evict every {buf} steps), log beta = logsigmoid(N({c['mu']},{c['sigma']})) fp32",
                    "segments_per_layer": nseg, "cache_bytes": cache.memory_bytes(),
-                   "launches_per_layer_step": ("1: append + attend in one launch (trimkv_append_attend)" if cache.fuse_decode_append and not args.gate
-                                               else "2: trimkv_append, trimkv_decode_attn") + ("" if B * Hkv >= 256 else " + split-K merge"),
+                   "launches_per_layer_step": (("2: trimkv_gate_hidden, then gate epilogue + append + attend in one launch (trimkv_append_attend_gated)" if args.gate
+                                                else "1: append + attend in one launch (trimkv_append_attend)") if cache.fuse_decode_append
+                                               else ("3: trimkv_gate_hidden, trimkv_append_gated, trimkv_decode_attn" if args.gate else "2: trimkv_append, trimkv_decode_attn"))
+                                              + ("" if B * Hkv >= 256 else " + split-K merge"),
                    **timing},
         "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
                      "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
@@ -655,7 +782,10 @@ def main():
         out["cpu_baseline"] = cpu_baseline(c)
     if args.gate:
         out["config"]["variant"] = (f"log beta from the fused rg gate (hidden {args.hidden}, intermediate 512, bf16) "
-                                    "instead of drawn values: not the BASELINE configuration")
+                                    "instead of drawn values: not the BASELINE configuration; "
+                                    + ("the gate's first linear runs on a second stream one layer ahead, beside the previous layer's "
+                                       "attention launch" if gate_side else
+                                       "the gate's first linear runs on the main stream in front of the launch that needs it"))
     if args.layers:
         out["config"]["note"] = "layer count overridden: not the BASELINE configuration"
     print(json.dumps(out))

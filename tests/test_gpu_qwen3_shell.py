@@ -211,6 +211,18 @@ def test_shell_decode_keeps_one_launch_per_layer_with_the_fused_gate(gate):
                 logits.append(out.logits)
                 assert all(s is None or s.pending is None for s in cache._slabs)     # every attention call carried its append out
         runs[fuse] = (torch.cat(logits, dim=1), deferred, [cache.kv_positions[l].clone() for l in range(cfg.num_hidden_layers)])
+    if gate == "rg":   # the gate beside the projections on a second stream (opt-in) or in front of them (default): the same bits
+        from trimkv_amd.qwen3 import TrimKVQwen3Attention
+        TrimKVQwen3Attention.gate_on_side_stream = True
+        try:
+            cache = TrimKVCache()
+            cache.fuse_decode_append = True
+            with torch.no_grad():
+                model(ids[:, :P], past_key_values=cache)
+                forked = torch.cat([model(ids[:, P + t:P + t + 1], past_key_values=cache).logits for t in range(STEPS)], dim=1)
+        finally:
+            TrimKVQwen3Attention.gate_on_side_stream = False
+        assert torch.equal(forked, runs[True][0])
     assert len(runs[True][1]) == STEPS * cfg.num_hidden_layers and all(runs[True][1]), "the fused gate switched the one-launch step off"
     assert not any(runs[False][1])
     assert torch.equal(runs[True][0], runs[False][0])

@@ -25,7 +25,7 @@ from torch import nn
 import torch.nn.functional as F
 
 from .attn import get_attention_interface
-from .cache_utils import TrimKVCache
+from .cache_utils import LazyLogBeta, TrimKVCache
 from .gate import RetentionGate, RetentionGate2, RetentionGate3
 
 
@@ -133,6 +133,20 @@ def apply_rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.T
     return out if rd == x.shape[-1] else torch.cat([out, x[..., rd:]], dim=-1)
 
 
+_SIDE_STREAMS: dict = {}
+
+
+def _side_stream(device) -> "torch.cuda.Stream":
+    """One extra stream per device (default priority), shared by all layers: the gates of consecutive layers are ordered
+    on it, which they are anyway through the hidden state."""
+    key = torch.device(device).index
+    key = torch.cuda.current_device() if key is None else key
+    st = _SIDE_STREAMS.get(key)
+    if st is None:
+        st = _SIDE_STREAMS[key] = torch.cuda.Stream(device=key)
+    return st
+
+
 class TrimKVQwen3Attention(nn.Module):
     gate_kinds = ("rg", "rg2", "rg3")   # the gates the reference's Qwen3 attention accepts (qwen3:295-302)
 
@@ -175,16 +189,51 @@ class TrimKVQwen3Attention(nn.Module):
         v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
         return q, k, v
 
+    # `rg` depends on nothing but the normed hidden state, as the q/k/v projections do.  With this flag its first linear
+    # (trimkv_gate_hidden) is issued on a second stream of the same priority and joined by an event before update(), so that
+    # it runs beside the projections, the head norms and RoPE instead of in front of them.  Off by default: the fork and
+    # join cost the host about 45 us per layer (stream switch, two events) to hide an 11 us kernel, which only pays when the
+    # host runs far ahead of the GPU; this eager decoder is host-bound at decode batch sizes (measured at the Qwen3-8B
+    # shape, batch 64: 18.9 ms per step with the gate on the main stream, 23.6 ms with the fork, 18.1 ms without a gate).
+    gate_on_side_stream = False
+
+    def _gate_beside_projections(self, hidden_states):
+        """The `rg` gate of this layer on the side stream; returns (log beta, event to wait for before it is read)."""
+        dev = hidden_states.device
+        cur = torch.cuda.current_stream(dev)
+        side = _side_stream(dev)
+        side.wait_stream(cur)                       # the normed hidden state is ready
+        with torch.cuda.stream(side):
+            retention = self.retention_gate(hidden_states)
+        done = getattr(self, "_gate_done", None)
+        if done is None:
+            done = self._gate_done = torch.cuda.Event()
+        done.record(side)
+        # Both tensors cross streams; instead of record_stream (allocator events on every free) they are kept alive until this
+        # layer's next call.  By then the main stream has waited for `done` (so whatever re-uses the hidden state's block on the
+        # main stream runs after the gate has read it) and the side stream has waited for the main stream again (so the next
+        # gate's partial sums, which may re-use this block on the side stream, are written after the attention launch read these).
+        self._gate_keep = (hidden_states, retention)
+        return retention, done
+
     def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
         B, S, _ = hidden_states.shape
-        q, k, v = self._qkv(hidden_states)
         # `rg` sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
-        retention = self.retention_gate(hidden_states).transpose(1, 2) if self.config.retention_gate == "rg" else None
+        retention, gate_done = None, None
+        if self.config.retention_gate == "rg":
+            if self.gate_on_side_stream and hidden_states.is_cuda and not self.training:
+                retention, gate_done = self._gate_beside_projections(hidden_states)
+            else:
+                retention = self.retention_gate(hidden_states)
+            retention = retention.transpose(1, 2)
+        q, k, v = self._qkv(hidden_states)
         cos, sin = position_embeddings
         q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
         if self.config.retention_gate in ("rg2", "rg3"):   # these see concat(K, V) after RoPE (qwen3:345-347)
             retention = self.retention_gate(torch.cat([k, v], dim=-1)).transpose(1, 2)
         offset = past_key_values.get_seq_length(self.layer_idx)
+        if gate_done is not None:
+            torch.cuda.current_stream(hidden_states.device).wait_event(gate_done)
         k, v, retention, kv_positions, fa_kwargs = past_key_values.update(
             k, v, retention, cache_position, self.layer_idx,
             {"sin": sin, "cos": cos, "cache_position": cache_position, "attention_mask": attention_mask})
