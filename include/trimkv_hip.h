@@ -407,6 +407,38 @@ int trimkv_append_attend_pieces(const void* q, void* out,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * Equal segments -- trimkv_decode_attn_uniform, trimkv_append_attend_uniform(_gated): the calls above for a cache whose
+ * segments all hold the same number of rows, which is every step of TrimKVCache (src/trimkv/cache_utils.py:62-110 keeps
+ * one length per layer; its attention is HF flash_attention_2 through src/trimkv/attn/__init__.py:15-26).  The length
+ * (len, resp. len_before the append) and the cut are launch arguments: every segment is attended in pieces_per_segment
+ * equal pieces (1: whole, one workgroup per segment), workgroup (segment, piece) comes from the grid, so a workgroup
+ * requests its first K tile without having loaded a list entry or a length first.  Pieces are merged inside the launch
+ * as in trimkv_decode_attn_pieces; workspace: trimkv_decode_attn_pieces_workspace(nseg * pieces_per_segment, group) bytes
+ * with the same zero-counter contract (not needed, may be NULL, when pieces_per_segment == 1).  K/V rows are the slab
+ * layout (segment seg at row seg*cap).  The appending forms advance seg_len (and cu_seqlens) like trimkv_append_attend and
+ * store bit-identical rows and outputs; seg_len itself is not read.  seg_first as in trimkv_decode_attn.
+ */
+int trimkv_decode_attn_uniform(const void* q, void* out, const void* k_slab, const void* v_slab, const int32_t* seg_first,
+                               int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                               int len, int pieces_per_segment, void* workspace, size_t workspace_bytes, void* stream);
+int trimkv_append_attend_uniform(const void* q, void* out,
+                                 void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                 int nseg, int kv_heads, int cap, int head_dim, int group, int kv_dtype, int lb_dtype,
+                                 const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                 const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
+                                 const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                 float scale, int len_before, int pieces_per_segment,
+                                 void* workspace, size_t workspace_bytes, void* stream);
+int trimkv_append_attend_uniform_gated(const void* q, void* out,
+                                       void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                       int nseg, int kv_heads, int cap, int head_dim, int group, int kv_dtype, int lb_dtype,
+                                       const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                       const float* gate_part, int gate_nslice, const float* gate_bias,
+                                       const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                       float scale, int len_before, int pieces_per_segment,
+                                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * trimkv_append_attend_gated / trimkv_append_attend_pieces_gated -- trimkv_append_attend(_pieces) whose new row takes its
  * log beta from the retention gate's partial sums instead of a finished tensor: the second linear's slice sum, the bias,
  * the logsigmoid (src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:177-179, called at :332-333 before update at :353) and
@@ -414,7 +446,8 @@ int trimkv_append_attend_pieces(const void* q, void* out,
  * stored bits are the same as that call's.  gate_part: [gate_nslice][nseg / kv_heads][kv_heads] fp32 as written by
  * trimkv_gate_hidden(_swiglu) for ONE token per batch element, gate_nslice = trimkv_gate_slices(inter) <= 64
  * (TRIMKV_ERR_UNSUPPORTED beyond: use trimkv_append_gated + trimkv_decode_attn); gate_bias: [kv_heads] fp32.  The other
- * arguments are those of trimkv_append_attend / trimkv_append_attend_pieces without lb_new and its strides.
+ * arguments are those of trimkv_append_attend / trimkv_append_attend_pieces (/ _uniform, declared above) without lb_new
+ * and its strides.
  */
 int trimkv_append_attend_gated(const void* q, void* out,
                                void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,

@@ -62,6 +62,11 @@ SIGNATURES = {
                                         _p, _i, _p, _p, _i64, _i64, _f, _i, _i, _p, _sz, _p]),
     "trimkv_append_attend_pieces_gated": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64,
                                                _p, _i, _p, _p, _i64, _i64, _f, _i, _p, _sz, _p]),
+    "trimkv_decode_attn_uniform": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p]),
+    "trimkv_append_attend_uniform": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64,
+                                          _p, _i64, _i64, _p, _i64, _i64, _f, _i, _i, _p, _sz, _p]),
+    "trimkv_append_attend_uniform_gated": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64,
+                                                _p, _i, _p, _p, _i64, _i64, _f, _i, _i, _p, _sz, _p]),
     "trimkv_plan_attn_pieces": (_i, [_p, _i, _i, _i, _p, _i]),
     "trimkv_decode_attn_static": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "trimkv_prefill_attn": (_i, [_p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p]),

@@ -71,29 +71,16 @@ def _workspace_zeroed(device, nbytes: int, stream: int) -> torch.Tensor:
     return ws
 
 
-_UNIFORM_PIECES: Dict[Tuple[str, int, int], torch.Tensor] = {}
-
-
-def _uniform_pieces(device, nseg: int, max_len: int):
-    """Piece list for segments of (nearly) equal length -- the dense cache.  With fewer than 256 segments each is cut so
+def _uniform_cut(nseg: int, max_len: int) -> int:
+    """Pieces per segment for segments of equal length -- the dense cache.  With fewer than 256 segments each is cut so
     that about 256 workgroups exist (a compute unit pulls about 50 GB/s whatever it runs, so all 256 are needed), but not
-    below 512 rows apiece; the pieces are merged inside the launch (``trimkv_decode_attn_pieces``), which saves the second
-    launch of the grid-split path.  None when the segments are attended whole (256 segments or more, or short ones)."""
+    below 512 rows apiece; the pieces are merged inside the launch (``trimkv_decode_attn_uniform``), which saves the second
+    launch of the grid-split path.  1 when the segments are attended whole (256 segments or more, or short ones)."""
     if nseg >= 256 or nseg > 8192:
-        return None
+        return 1
     want = (dense_workgroups + nseg - 1) // nseg
     chunk = max(dense_min_rows, (((max_len + want - 1) // want + 63) // 64) * 64)
-    nsp = (max_len + chunk - 1) // chunk
-    if nsp <= 1:
-        return None
-    key = (str(device), nseg, nsp)
-    t = _UNIFORM_PIECES.get(key)
-    if t is None:
-        seg = torch.arange(nseg, dtype=torch.int32).repeat(nsp)                        # piece-major: consecutive workgroups are
-        which = torch.arange(nsp, dtype=torch.int32).repeat_interleave(nseg)           # different segments (they spread over the XCDs)
-        t = torch.stack([seg, which, torch.full_like(seg, nsp), seg * nsp], dim=1).contiguous().to(device)
-        _UNIFORM_PIECES[key] = t
-    return t, nseg * nsp
+    return max(1, (max_len + chunk - 1) // chunk)
 
 
 def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[torch.Tensor]:
@@ -111,21 +98,31 @@ def _workspace(device, nbytes: int, stream: Optional[int] = None) -> Optional[to
 def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Tensor, nseg: int, group: int,
                      seg_len: Optional[torch.Tensor], seg_start: Optional[torch.Tensor], cap: int, max_len: int,
                      scale: float, chunk: int = 0, seg_order: Optional[torch.Tensor] = None,
-                     seg_first: Optional[torch.Tensor] = None, pieces=None) -> torch.Tensor:
+                     seg_first: Optional[torch.Tensor] = None, pieces=None, uniform_pps: int = 0) -> torch.Tensor:
     """``query`` [nseg*group, D] (contiguous) -> [nseg*group, D]; K/V rows at ``seg_start[seg]`` or ``seg*cap``.
     ``seg_order``: optional int32 permutation of the segments, longest first (dispatch order only).
-    ``seg_first``: optional int32 [nseg], the first attended row of every segment (rows before it are masked)."""
+    ``seg_first``: optional int32 [nseg], the first attended row of every segment (rows before it are masked).
+    ``uniform_pps`` > 0: every segment holds exactly ``max_len`` rows at ``seg*cap`` (a dense cache): length and cut travel
+    as launch arguments (``trimkv_decode_attn_uniform``), each segment in that many equal pieces merged inside the launch."""
     if not query.is_cuda:
         raise _lib.TrimKVLibraryError("decode attention runs on the GPU through libtrimkv_hip.so only (no CPU path)")
     if group > _MAX_GROUP:   # more query heads per KV head than one launch takes: several launches over slices of the group
         g1 = _group_slice(group)
         q3 = query.view(nseg, group, -1)
         outs = [decode_attention(q3[:, a:a + g1].reshape(nseg * g1, -1), k_rows, v_rows, nseg, g1, seg_len, seg_start, cap, max_len,
-                                 scale, chunk, seg_order, seg_first, pieces).view(nseg, g1, -1) for a in range(0, group, g1)]
+                                 scale, chunk, seg_order, seg_first, pieces, uniform_pps).view(nseg, g1, -1) for a in range(0, group, g1)]
         return torch.cat(outs, dim=1).view(nseg * group, -1)
     lib = _lib.load()
     d = query.shape[-1]
     out = torch.empty_like(query)
+    if uniform_pps > 0:
+        st = _lib.current_stream(query.device)
+        ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(nseg * uniform_pps, group), st) if uniform_pps > 1 else None
+        rc = lib.trimkv_decode_attn_uniform(query.data_ptr(), out.data_ptr(), k_rows.data_ptr(), v_rows.data_ptr(), _lib.ptr(seg_first),
+                                            nseg, cap, d, group, _lib.dtype_code(query.dtype), float(scale), max_len, uniform_pps,
+                                            _lib.ptr(ws), 0 if ws is None else ws.numel(), st)
+        _lib.check(rc, "trimkv_decode_attn_uniform")
+        return out
     if pieces is not None:   # (device piece list, count): one launch, pieces merged inside it
         st = _lib.current_stream(query.device)
         ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(pieces[1], group), st)
@@ -146,7 +143,7 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
 
 
 def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: int = 0,
-                  seg_order: Optional[torch.Tensor] = None, pieces=None) -> torch.Tensor:
+                  seg_order: Optional[torch.Tensor] = None, pieces=None, uniform_pps: int = 0) -> torch.Tensor:
     """The deferred one-token append of ``slab`` (a cache layer whose ``update`` ran with ``fuse_decode_append``) and the
     attention over the layer including that token, in one launch: ``trimkv_append_attend``.  ``query`` [nseg*group, D]
     contiguous -> [nseg*group, D].  Clears the pending append."""
@@ -156,6 +153,15 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
     st = _lib.current_stream(query.device)
     # a log beta that the retention gate left unfinished (LazyLogBeta) is finished by the same launch: the gated entry points
     gated = not torch.is_tensor(slab.pending[3])
+    if uniform_pps > 0:      # a dense cache: every segment holds max_len - 1 rows before this token; length and cut are launch arguments
+        ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(nseg * uniform_pps, group), st) if uniform_pps > 1 else None
+        fn = lib.trimkv_append_attend_uniform_gated if gated else lib.trimkv_append_attend_uniform
+        rc = fn(query.data_ptr(), out.data_ptr(), *slab.ptrs, nseg, slab.H, slab.cap, d, group, *slab.codes, *slab.pending[0], scale,
+                slab.max_len - 1, uniform_pps, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
+        if rc:
+            _lib.check(rc, "trimkv_append_attend_uniform_gated" if gated else "trimkv_append_attend_uniform")
+        slab.pending = None
+        return out
     if pieces is not None:   # ragged lengths: one launch over the (segment, piece) list, merged inside it
         plist, npieces = pieces
         ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(npieces, group), st)
@@ -323,15 +329,20 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     causal = bool(getattr(module, "is_causal", True)) if is_causal is None else bool(is_causal)
     window = int(sliding_window) if sliding_window is not None and n > int(sliding_window) else None
     plain = not dropout and softcap is None        # what the kernels compute: softmax(q k^T * scale) v
-    dense_pieces = None
-    if Q == 1 and not dense_chunk and G in _DENSE_PIECES_GROUPS:
-        dense_pieces = _uniform_pieces(query.device, B * Hkv, n)
-    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None and window is None and plain, dense_pieces)
+    # every segment of a dense cache holds n rows: length and cut go to the kernel as launch arguments (pps pieces per segment)
+    pps = 0
+    if Q == 1 and not dense_chunk and G <= _MAX_GROUP:
+        pps = _uniform_cut(B * Hkv, n)
+        if pps > 1 and G not in _DENSE_PIECES_GROUPS:
+            pps = 0    # wide groups in pieces: the grid launch + merge kernel
+    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None and window is None and plain, True if pps > 1 else None)
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
-        return append_attend(slab, q2, G, scale, chunk=dense_chunk, pieces=dense_pieces).view(B, 1, Hq, D), None, None
+        if slab.cu is not None:
+            pps = 0
+        return append_attend(slab, q2, G, scale, chunk=dense_chunk, uniform_pps=pps).view(B, 1, Hq, D), None, None
     kernel_ok = plain and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128)
     seg_first = None
     if kernel_ok and Q == 1:
@@ -352,7 +363,7 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
-        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first, pieces=dense_pieces)
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first, uniform_pps=pps)
         return out.view(B, 1, Hq, D), None, None
     if kernel_ok and Q > 1 and attention_mask is None and window is None and causal:
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)

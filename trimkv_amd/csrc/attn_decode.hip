@@ -30,6 +30,23 @@ extern "C" int trimkv_decode_attn(const void* q, void* out, const void* k_slab, 
                               dtype, scale, max_len, chunk, workspace, workspace_bytes, stream);
 }
 
+// ---- equal segments (a dense cache): lengths and cuts as launch arguments ---------------------------------------------
+extern "C" int trimkv_decode_attn_uniform(const void* q, void* out, const void* k_slab, const void* v_slab, const int32_t* seg_first,
+                                          int nseg, int cap, int head_dim, int group, int dtype, float scale,
+                                          int len, int pieces_per_segment, void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_decode_attn_uniform";
+    AttnArgs a;
+    if (len <= 0) return fail(TRIMKV_ERR_SHAPE, "%s: len=%d", fn, len);
+    int rc = prepare_attn(fn, a, q, out, k_slab, v_slab, nullptr, nullptr, nullptr, seg_first, nseg, cap, head_dim, group, dtype, scale,
+                          len, ((len + 63) / 64) * 64, nullptr, 0);
+    if (rc) return rc;
+    const int npieces = prepare_uniform(fn, a, len, pieces_per_segment, nseg, group, workspace, workspace_bytes);
+    if (npieces < 0) return npieces;
+    if (pieces_per_segment == 1) launch_attn_group<false>(a, group, head_dim, dtype, (hipStream_t)stream);
+    else launch_pieces_plain(a, npieces, group, head_dim, dtype, (hipStream_t)stream);
+    return launch_status(fn);
+}
+
 // ---- the same call for callers that cannot allocate ------------------------------------------------------------------
 // The split-K partials live in a fixed array inside the library's code object instead of a caller workspace.  In host code
 // the array's name is only a handle: the device address is looked up once per device and that address is what the

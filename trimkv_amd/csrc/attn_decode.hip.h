@@ -137,6 +137,10 @@ struct AttnArgs {
     // piece-list launches (decode_attn_pieces_kernel): one workgroup per entry {segment, piece, pieces of the segment,
     // first partial slot of the segment}; counters[seg] counts the finished pieces of a segment (zero between launches)
     const int4* pieces; uint32_t* counters; int npieces;
+    // Equal segments (a dense cache): uniform_len >= 0 is the stored length of EVERY segment (seg_len is then not read, only
+    // advanced by APPEND kernels), and uniform_nsp > 0 replaces the piece list by the grid: workgroup (x, y) is piece y of
+    // uniform_nsp equal pieces of segment x, partial slots x*uniform_nsp + y.  Nothing is loaded before the first K tile.
+    int uniform_len, uniform_nsp;
 };
 
 // Row bounds of a piece inside its segment are fractions with this denominator (trimkv_hip.h: TRIMKV_PIECE_FRACTION).
@@ -159,7 +163,7 @@ __device__ __forceinline__ float load_shared_partial(const float* p) { return __
 // *first: the first attended row (0 unless the caller masks a prefix of the segment).
 template <bool APPEND>
 __device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new_row, int* first) {
-    int n = a.seg_len ? a.seg_len[seg] : a.max_len;
+    int n = a.uniform_len >= 0 ? a.uniform_len : (a.seg_len ? a.seg_len[seg] : a.max_len);
     *new_row = -1;
     if (APPEND) {
         n = max(n, 0);
@@ -544,16 +548,25 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
 template <int G, int ROW16, bool F16, bool APPEND, bool GATED = false>
 __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIMKV_AT_WPE))) void decode_attn_pieces_kernel(AttnArgs a) {
     __shared__ int last_of_segment;
-    const int4 e = a.pieces[blockIdx.x];
-    // entry = {segment, piece | begin << 16, pieces of the segment | end << 16, first partial slot}
-    const uint32_t ey = (uint32_t)e.y, ez = (uint32_t)e.z;
-    const int seg = min(max(e.x, 0), a.nseg - 1), nsp = max((int)(ez & 0xffffu), 1), piece = min((int)(ey & 0xffffu), nsp - 1);
-    if (nsp > 1 && (e.w < 0 || e.w + nsp > a.npieces)) return;   // a list whose partial slots do not fit the workspace: touch nothing
+    int seg, nsp, piece;
+    int64_t slot0;
+    uint32_t f0 = 0, f1 = 0;
+    if (a.uniform_nsp > 0) {   // equal segments in equal pieces: everything comes from the launch arguments
+        seg = blockIdx.x; piece = blockIdx.y; nsp = a.uniform_nsp;
+        slot0 = (int64_t)seg * nsp;
+    } else {
+        const int4 e = a.pieces[blockIdx.x];
+        // entry = {segment, piece | begin << 16, pieces of the segment | end << 16, first partial slot}
+        const uint32_t ey = (uint32_t)e.y, ez = (uint32_t)e.z;
+        seg = min(max(e.x, 0), a.nseg - 1); nsp = max((int)(ez & 0xffffu), 1); piece = min((int)(ey & 0xffffu), nsp - 1);
+        if (nsp > 1 && (e.w < 0 || e.w + nsp > a.npieces)) return;   // a list whose partial slots do not fit the workspace: touch nothing
+        f1 = min(ez >> 16, (uint32_t)AT_PIECE_FRACTION); f0 = min(ey >> 16, f1);
+        slot0 = e.w;
+    }
     int new_row, first;
     const int n = segment_rows<APPEND>(a, seg, &new_row, &first);
     const int live = n - first;
     int t0, t1;   // may be empty: the piece then contributes nothing
-    const uint32_t f1 = min(ez >> 16, (uint32_t)AT_PIECE_FRACTION), f0 = min(ey >> 16, f1);
     if (f1 == 0) {           // equal pieces
         const int rps = (live + nsp - 1) / nsp;
         t0 = min(n, first + piece * rps);
@@ -562,7 +575,6 @@ __global__ __launch_bounds__(AT_THREADS) __attribute__((amdgpu_waves_per_eu(TRIM
         t0 = first + (int)(((int64_t)live * f0) >> AT_PIECE_FRACTION_BITS);
         t1 = first + (int)(((int64_t)live * f1) >> AT_PIECE_FRACTION_BITS);
     }
-    const int64_t slot0 = e.w;
     // one instantiation for both cases (a second inlined copy of the streaming loop costs registers): a segment in one
     // piece writes its output itself, the others leave partials
     attend_rows<G, ROW16, F16, APPEND, true, GATED>(a, seg, t0, t1, nsp == 1, slot0 + piece, new_row);
@@ -703,7 +715,7 @@ static void launch_attn(const AttnArgs& a, int head_dim, int dtype, hipStream_t 
 
 template <int G, bool APPEND, bool GATED>
 static void launch_attn_pieces(const AttnArgs& a, int npieces, int head_dim, int dtype, hipStream_t st) {
-    const dim3 grid(npieces), block(AT_THREADS);
+    const dim3 grid = a.uniform_nsp > 0 ? dim3(a.nseg, a.uniform_nsp) : dim3(npieces), block(AT_THREADS);
     if (dtype == TRIMKV_F16) {
         if (head_dim == 128) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 16, true, APPEND, GATED>), grid, block, 0, st, a);
         else if (head_dim == 96) hipLaunchKernelGGL((decode_attn_pieces_kernel<G, 12, true, APPEND, GATED>), grid, block, 0, st, a);
@@ -756,6 +768,35 @@ static int prepare_pieces(const char* fn, AttnArgs& a, const int32_t* pieces, in
     return TRIMKV_OK;
 }
 
+// Completes `a` (already through prepare_attn with a chunk that covers max_len, i.e. direct) for a launch over equal
+// segments: every segment holds `len` rows (before the append, if any) and is cut into `pps` equal pieces.  pps == 1 runs
+// the grid kernel (one workgroup per segment writes the output); pps > 1 the piece-list kernel in grid mode, merged in
+// the launch.  Returns the number of pieces (> 0), or a negative status.
+static int prepare_uniform(const char* fn, AttnArgs& a, int len, int pps, int nseg, int group, void* workspace, size_t workspace_bytes) {
+    if (len < 0 || len > a.cap) return fail(TRIMKV_ERR_SHAPE, "%s: length %d outside [0, capacity %d]", fn, len, a.cap);
+    if (pps < 1 || pps > 65535) return fail(TRIMKV_ERR_SHAPE, "%s: pieces_per_segment must be in [1, 65535] (got %d)", fn, pps);
+    a.uniform_len = len;
+    if (pps == 1) return 1;
+    if (nseg > AT_PIECE_MAX_SEGMENTS) return fail(TRIMKV_ERR_UNSUPPORTED, "%s: at most %d segments in pieces (got %d)", fn, AT_PIECE_MAX_SEGMENTS, nseg);
+    if ((int64_t)nseg * pps > 0x7fffffff) return fail(TRIMKV_ERR_SHAPE, "%s: too many pieces", fn);
+    const int npieces = nseg * pps;
+    const size_t need = pieces_workspace_bytes(npieces, group);
+    if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);
+    if ((uintptr_t)workspace & 15) return fail(TRIMKV_ERR_SHAPE, "%s: workspace must be 16-byte aligned", fn);
+    a.uniform_nsp = pps;
+    a.npieces = npieces;
+    a.counters = (uint32_t*)workspace;
+    a.ws_o = (float*)((char*)workspace + AT_PIECE_COUNTER_BYTES);
+    a.ws_ml = a.ws_o + (size_t)npieces * group * AT_D;
+    a.direct = 0;
+    return npieces;
+}
+
+// The piece-list kernels are instantiated in their own translation units; these let the entry points of the others reach them.
+void launch_pieces_plain(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st);
+void launch_pieces_append(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st);
+void launch_pieces_append_gated(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st);
+
 // group = 1..8 -> the matching instantiation
 template <bool APPEND, bool GATED = false>
 static void launch_attn_group(const AttnArgs& a, int group, int head_dim, int dtype, hipStream_t st) {
@@ -794,6 +835,7 @@ static int prepare_attn(const char* fn, AttnArgs& a, const void* q, void* out, c
     a.ws_o = nullptr; a.ws_ml = nullptr;
     a.ap = AppendPart{};
     a.pieces = nullptr; a.counters = nullptr; a.npieces = 0;
+    a.uniform_len = -1; a.uniform_nsp = 0;
     if (!a.direct) {
         const size_t need = (size_t)nseg * a.nsplit * group * (AT_D + 2) * sizeof(float);   // partial rows are padded to 128 features
         if (!workspace || workspace_bytes < need) return fail(TRIMKV_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, got %zu", fn, need, workspace_bytes);

@@ -33,3 +33,31 @@ extern "C" int trimkv_append_attend(const void* q, void* out,
     return launch_status(fn);
 }
 
+
+// The dense cache's decode step: every segment holds len_before rows, so the length and the cut of each workgroup are
+// launch arguments and a workgroup requests its first K tile without loading anything first (a piece list costs two
+// dependent loads -- entry, then length -- before it, the grid launch one).
+extern "C" int trimkv_append_attend_uniform(const void* q, void* out,
+                                            void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                            int nseg, int kv_heads, int cap, int head_dim, int group, int kv_dtype, int lb_dtype,
+                                            const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                            const void* lb_new, int64_t lb_stride_b, int64_t lb_stride_h,
+                                            const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                            float scale, int len_before, int pieces_per_segment,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_append_attend_uniform";
+    int rc = check_append_args(fn, lb_slab, pos_slab, seg_len, k_new, v_new, lb_new, pos_new, nseg, kv_heads, lb_dtype, kv_stride_b, kv_stride_h);
+    if (rc) return rc;
+    if (len_before < 0 || len_before >= cap) return fail(TRIMKV_ERR_CAPACITY, "%s: no room for a row after %d rows (capacity %d)", fn, len_before, cap);
+    AttnArgs a;
+    rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, nullptr, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
+                      len_before + 1, ((len_before + 1 + 63) / 64) * 64, nullptr, 0);
+    if (rc) return rc;
+    const int npieces = prepare_uniform(fn, a, len_before, pieces_per_segment, nseg, group, workspace, workspace_bytes);
+    if (npieces < 0) return npieces;
+    fill_append_part(fn, a, lb_slab, pos_slab, seg_len, cu_seqlens, nseg, kv_heads, lb_dtype, k_new, v_new, kv_stride_b, kv_stride_h,
+                     lb_new, lb_stride_b, lb_stride_h, pos_new, pos_stride_b, pos_stride_h);
+    if (pieces_per_segment == 1) launch_attn_group<true>(a, group, head_dim, kv_dtype, (hipStream_t)stream);
+    else launch_pieces_append(a, npieces, group, head_dim, kv_dtype, (hipStream_t)stream);
+    return launch_status(fn);
+}

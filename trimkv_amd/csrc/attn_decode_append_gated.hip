@@ -34,3 +34,30 @@ extern "C" int trimkv_append_attend_gated(const void* q, void* out,
     launch_attn_group<true, true>(a, group, head_dim, kv_dtype, (hipStream_t)stream);
     return launch_status(fn);
 }
+
+extern "C" int trimkv_append_attend_uniform_gated(const void* q, void* out,
+                                                  void* k_slab, void* v_slab, void* lb_slab, int64_t* pos_slab, int32_t* seg_len, int32_t* cu_seqlens,
+                                                  int nseg, int kv_heads, int cap, int head_dim, int group, int kv_dtype, int lb_dtype,
+                                                  const void* k_new, const void* v_new, int64_t kv_stride_b, int64_t kv_stride_h,
+                                                  const float* gate_part, int gate_nslice, const float* gate_bias,
+                                                  const int64_t* pos_new, int64_t pos_stride_b, int64_t pos_stride_h,
+                                                  float scale, int len_before, int pieces_per_segment,
+                                                  void* workspace, size_t workspace_bytes, void* stream) {
+    const char* fn = "trimkv_append_attend_uniform_gated";
+    int rc = check_append_args(fn, lb_slab, pos_slab, seg_len, k_new, v_new, gate_part, pos_new, nseg, kv_heads, lb_dtype, kv_stride_b, kv_stride_h);
+    if (rc) return rc;
+    if (len_before < 0 || len_before >= cap) return fail(TRIMKV_ERR_CAPACITY, "%s: no room for a row after %d rows (capacity %d)", fn, len_before, cap);
+    AttnArgs a;
+    rc = prepare_attn(fn, a, q, out, k_slab, v_slab, seg_len, nullptr, nullptr, nullptr, nseg, cap, head_dim, group, kv_dtype, scale,
+                      len_before + 1, ((len_before + 1 + 63) / 64) * 64, nullptr, 0);
+    if (rc) return rc;
+    const int npieces = prepare_uniform(fn, a, len_before, pieces_per_segment, nseg, group, workspace, workspace_bytes);
+    if (npieces < 0) return npieces;
+    fill_append_part(fn, a, lb_slab, pos_slab, seg_len, cu_seqlens, nseg, kv_heads, lb_dtype, k_new, v_new, kv_stride_b, kv_stride_h,
+                     nullptr, 0, 0, pos_new, pos_stride_b, pos_stride_h);
+    rc = fill_gate_part(fn, a, gate_part, gate_nslice, gate_bias);
+    if (rc) return rc;
+    if (pieces_per_segment == 1) launch_attn_group<true, true>(a, group, head_dim, kv_dtype, (hipStream_t)stream);
+    else launch_pieces_append_gated(a, npieces, group, head_dim, kv_dtype, (hipStream_t)stream);
+    return launch_status(fn);
+}

@@ -31,3 +31,7 @@ extern "C" int trimkv_append_attend_pieces_gated(const void* q, void* out,
     launch_attn_pieces_group<true, true>(a, npieces, group, head_dim, kv_dtype, (hipStream_t)stream);
     return launch_status(fn);
 }
+
+void trimkv::launch_pieces_append_gated(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st) {
+    launch_attn_pieces_group<true, true>(a, npieces, group, head_dim, dtype, st);
+}

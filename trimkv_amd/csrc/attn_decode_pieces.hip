@@ -27,3 +27,7 @@ extern "C" int trimkv_decode_attn_pieces(const void* q, void* out, const void* k
     return launch_status(fn);
 }
 
+void trimkv::launch_pieces_plain(const AttnArgs& a, int npieces, int group, int head_dim, int dtype, hipStream_t st) {
+    launch_attn_pieces_group<false>(a, npieces, group, head_dim, dtype, st);
+}
+
