@@ -68,6 +68,26 @@ def measured_traffic_ratio(config=3):
     return None, None
 
 
+def profile_kernel_figures(config=3):
+    """Average duration of the dominant kernel and its algorithmic bytes per launch as the committed rocprofv3 kernel trace
+    of this workload has them (lines `profile_kernel_us:` and `profile_bytes_per_launch:` of the summary under profiles/),
+    so that the roofline fraction can be reproduced from profiles/ to the digit next to the figure timed in this run."""
+    path = os.path.join(ROOT, "profiles", f"decode_step_config{config}_kernel_trace.md")
+    us = nbytes = None
+    try:
+        for line in open(path):
+            if line.startswith("profile_kernel_us:"):
+                us = float(line.split(":")[1])
+            elif line.startswith("profile_bytes_per_launch:"):
+                nbytes = int(line.split(":")[1])
+    except OSError:
+        pass
+    if us is None or nbytes is None:
+        return None
+    return {"profile_kernel_us": us, "profile_bytes_per_launch": nbytes, "profile_frac": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+            "profile_source": os.path.relpath(path, ROOT)}
+
+
 def cpu_baseline(c, budget_s=20.0):
     """The oracle (the reference's pure-PyTorch CPU path restated) on ONE layer at full shape,
     extrapolated to the full step: t_step = L * (B / b) * (t_append_attend + t_evict / buffer)."""
@@ -511,6 +531,10 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=sorted(list(CONFIGS) + [4]),
                     help="BASELINE config: 3 = headline; 2, 5 = other dense shapes; 4 = ragged per-head budgets (secondary workload)")
     ap.add_argument("--chunk", type=int, default=0, help="split-K rows per workgroup for decode attention (0 = library default)")
+    ap.add_argument("--dense-workgroups", type=int, default=0,
+                    help="tuning knob: workgroups wanted per dense decode-attention launch (segments are cut into equal pieces to reach it)")
+    ap.add_argument("--dense-groups", type=str, default="",
+                    help="tuning knob: comma-separated group sizes that attend a split dense segment in one launch (pieces merged inside it)")
     ap.add_argument("--layers", type=int, default=0, help="override the number of layers (smoke runs only; makes the result invalid)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fuse", action="store_true",
@@ -576,6 +600,10 @@ def main():
     attn_fn = get_attention_interface("trimkv_hip")
     if args.chunk:
         hip_attn.dense_chunk = args.chunk
+    if args.dense_workgroups:
+        hip_attn.dense_workgroups = args.dense_workgroups
+    if args.dense_groups:
+        hip_attn._DENSE_PIECES_GROUPS = tuple(int(g) for g in args.dense_groups.split(","))
 
     # Cycle of the steady state: an eviction takes every head to M rows, the next buf steps attend M+1 .. M+buf rows and the
     # last of them evicts again.  The cache starts one row short of the trigger, so the first warm-up step evicts.
@@ -737,17 +765,28 @@ def main():
         avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens) + (append_bytes if fused else 0)
         achieved = avg_bytes / avg_s / 1e9
         ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
-        merge_targs = f"<{G}, 16, false, {'true' if fused else 'false'}>"
-        targs = merge_targs[:-1] + (", true>" if fused and args.gate else ">")    # GATED instantiation when the launch finishes the gate
-        roof = {"bound": "hbm", "kernel": "decode_attn_kernel" + targs + ("" if B * Hkv >= 256 else " + decode_attn_merge_kernel" + merge_targs), "achieved": round(achieved, 1),
+        tf = lambda b: "true" if b else "false"
+        targs = f"<{G}, 16, false, {tf(fused)}, {tf(fused and args.gate)}>"   # group, 16-byte pieces per row, fp16, APPEND, GATED
+        pps = hip_attn._uniform_cut(nseg, M + buf) if not args.chunk else 0
+        if pps > 1 and G in hip_attn._DENSE_PIECES_GROUPS:
+            kernel = "decode_attn_pieces_kernel" + targs + f" ({pps} equal pieces per segment from the grid, merged inside the launch)"
+        elif nseg >= 256 or pps == 1:
+            kernel = "decode_attn_kernel" + targs
+        else:
+            kernel = "decode_attn_kernel" + targs + f" + decode_attn_merge_kernel<{G}, 16, false, {tf(fused)}>"
+        roof = {"bound": "hbm", "kernel": kernel, "achieved": round(achieved, 1),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_bytes * ratio), "traffic_source": src,
                 "traffic_measured_in_run": False,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(durs),
+                "frac_basis": "HIP events recorded around the sampled calls on the launch stream: they include the dispatch gap in front "
+                              "of the kernel, so frac is a little below the kernel's own (profile_frac, from the committed trace)",
                 "algorithmic_bytes_per_launch": int(avg_bytes),
                 "mfma_utilisation": 0.0,
                 "mfma_note": f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
                              "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
+    if roof is not None and args.config == 3 and not args.gate:
+        roof.update(profile_kernel_figures(3) or {})
     parity = attention_gate(cache, c, attn_fn, mod, T)
     parity.update(evict_parity)
     timing = {"host_enqueue_ms_per_step": round(enqueue_seconds * 1e3 / args.steps, 4), "ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}

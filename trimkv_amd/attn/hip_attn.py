@@ -33,9 +33,9 @@ _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
 # KV head (one spilled dword at five) and spills badly at eight.  Ragged caches, whose alternative is the append as a
 # launch of its own in front of the unfused piece-list kernel: 43.0 against 45.1 us per layer at a group of 5, 44.0 against
 # 46.0 at 6, 63.9 against 59.9 at 8 (256 lognormal segments).  Dense cache, whose alternative is the fused grid launch +
-# merge kernel: equal at a group of 5 (2.044 against 2.039 ms per step at Qwen3-14B's shape), so it stays there.
+# merge kernel: 50.2 us in one launch against 46.8 + 5.2 us in two at a group of 5 (64 segments of 8448 rows in 4 pieces).
 _FUSED_PIECES_GROUPS = (1, 2, 3, 4, 5, 6)
-_DENSE_PIECES_GROUPS = (1, 2, 3, 4)
+_DENSE_PIECES_GROUPS = (1, 2, 3, 4, 5, 6)
 _WARNED = set()
 dense_workgroups, dense_min_rows = 256, 512   # piece-list launches of the dense cache: workgroups wanted, fewest rows apiece
 dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)
