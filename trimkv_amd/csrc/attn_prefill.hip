@@ -320,7 +320,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int b = seg / a.kv_heads, h = seg - b * a.kv_heads;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform by construction; saying so keeps what derives from it in scalar registers
     const int j = lane & 31, hl = lane >> 5;    // MFMA column (query) and lane half
     const int G = a.group, Q = a.q_len;
     const int BT = (PF2_WAVES * 32) / G;        // query times per workgroup; rows BT * G .. 255 are padding
@@ -330,18 +331,27 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int t_q = t_wg0 + r / G;              // this lane's query time
     const bool q_ok = r < BT * G && t_q < Q;
     const int t_w_first = t_wg0 + (w * 32) / G;
-    const int t_w_last = t_wg0 + min(w * 32 + 31, BT * G - 1) / G;
     const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
 
-    // Q fragments (B operand of S^T): 8 d of step ks at d = ks * 16 + hl * 8
+    // Q fragments (B operand of S^T): 8 d of step ks at d = ks * 16 + hl * 8, multiplied by scale * log2(e) and rounded back
+    // to 16 bits once, here: the score MFMAs then deliver exponents of two directly and the loop never multiplies a score.
     pf_bf16x8 qf[8];
     {
         const uint16_t* qrow = a.q + (int64_t)b * a.q_sb + (int64_t)(h * G + g) * a.q_sh + (int64_t)min(t_q, Q - 1) * a.q_st;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const int e0 = ks * 16 + hl * 8;
-            qf[ks] = *(const pf_bf16x8*)(qrow + min(e0, a.hd - 8));
-            if (e0 >= a.hd) qf[ks] = pf_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};   // padded features: whatever K holds there counts for nothing
+            const pf_u32x4 raw = *(const pf_u32x4*)(qrow + min(e0, a.hd - 8));
+            pf_u32x4 sc;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                float lo, hi;
+                if (F16) { lo = f16_bits_to_f32((uint16_t)(raw[x] & 0xffffu)); hi = f16_bits_to_f32((uint16_t)(raw[x] >> 16)); }
+                else { lo = __uint_as_float(raw[x] << 16); hi = __uint_as_float(raw[x] & 0xffff0000u); }
+                sc[x] = pack_kv<F16>(lo * a.scale_log2, hi * a.scale_log2);
+            }
+            if (e0 >= a.hd) sc = pf_u32x4{0u, 0u, 0u, 0u};   // padded features: whatever K holds there counts for nothing
+            qf[ks] = __builtin_bit_cast(pf_bf16x8, sc);
         }
     }
 
@@ -350,16 +360,19 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o[db][v] = 0.0f;
-    // exponent reference (scaled log2 units) and this lane's share of the row sum.  A query that sees no key at all
+    // Exponent reference (log2 units) and this lane's share of the row sum.  The score MFMAs start from -m_ref in their
+    // accumulator (negm, all 16 registers alike: a lane is one query), so what they deliver is already s - m_ref.  The
+    // reference starts at 0 and is moved onto the row maximum by the first block.  A query that sees no key at all
     // (segment shorter than the chunk) keeps reference 0: its masked scores give exp2(-huge) = 0, never exp2(0).
-    float m_ref = PF_NEG, l_run = 0.0f;
+    float m_ref = 0.0f, l_run = 0.0f;
+    pf_f32x16 negm;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) negm[v] = 0.0f;
 
     const int t_last = min(Q - 1, t_wg0 + BT - 1);
     const int k_end = max(0, min(n, n - Q + t_last + 1));     // keys the workgroup visits
     const int vis_j = n - Q + t_q;                            // last key this lane's query sees
-    if (vis_j < 0) m_ref = 0.0f;
     const int vis_lo = n - Q + t_w_first;                     // ... the wavefront's first query
-    const int vis_hi = t_w_first < Q ? n - Q + min(Q - 1, t_w_last) : -1;   // ... its last real query (none: skip every tile)
     const int last_row = max(n - 1, 0);
 
     // ---- staging: global -> registers -> LDS (K row-major, V transposed) ----
@@ -426,11 +439,9 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int k_off = j * PF2_KROW + hl * 16;
     const int v_off = PF2_KBYTES + j * PF2_VROW + hl * 16;
 
-    // S^T = K . Q^T of one 32-key block (raw, unscaled scores)
+    // S^T = K . Q^T of one 32-key block, relative to the exponent reference: s - m_ref in log2 units
     auto qk = [&](const char* buf, int kb) __attribute__((always_inline)) {
-        pf_f32x16 s;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.0f;
+        pf_f32x16 s = negm;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
@@ -439,9 +450,13 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         return s;
     };
     // Mask (diagonal blocks only), row maximum, and the lazy move of the exponent reference: O and l are
-    // rescaled only when some row of the wavefront outgrows its reference by 2^PF2_LAZY.
-    auto prepare = [&](pf_f32x16& s, int blk) __attribute__((always_inline)) {
+    // rescaled only when some row of the wavefront outgrows its reference by 2^PF2_LAZY.  FIRST: the wavefront's first
+    // block puts the reference on the row maximum wherever it lies (O and l are still zero: nothing to rescale).
+    auto prepare = [&](pf_f32x16& s, int blk, auto first_c) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(first_c)::value;
         if (blk * 32 + 31 > vis_lo) {   // wave-uniform: some query of the wavefront does not see the whole block
+            // (the empty volatile statement keeps this a branch: as 48 speculated selects it would run for every block)
+            asm volatile("" ::: );
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int key = blk * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
@@ -450,24 +465,28 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         }
         float tmax = s[0];
 #pragma unroll
-        for (int v = 1; v < 16; ++v) tmax = fmaxf(tmax, s[v]);
-        tmax *= a.scale_log2;
-        if (__builtin_amdgcn_ballot_w64(tmax > m_ref + PF2_LAZY) != 0) {
-            const float t2 = fmaxf(tmax, __shfl_xor(tmax, 32, 64));   // both halves of a query agree on the reference
-            const float m_new = fmaxf(m_ref, t2);
-            const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-            m_ref = m_new;
-            l_run *= alpha;
+        for (int v = 1; v < 16; ++v) tmax = __builtin_fmaxf(tmax, s[v]);
+        if (FIRST || __builtin_amdgcn_ballot_w64(tmax > PF2_LAZY) != 0) {
+            const float t2 = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, 64));   // both halves of a query agree on the reference
+            // how far the reference moves: onto the maximum (first block; not at all for a row that sees nothing), else up only
+            const float d = FIRST ? (t2 > 0.5f * PF_NEG ? t2 : 0.0f) : __builtin_fmaxf(t2, 0.0f);
+            m_ref += d;
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+            for (int v = 0; v < 16; ++v) { s[v] -= d; negm[v] = -m_ref; }
+            if (!FIRST) {
+                const float alpha = __builtin_amdgcn_exp2f(-d);
+                l_run *= alpha;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+            }
         }
     };
-    // P = exp2(S * scale - ref) as bf16 (two scores -> one dword) and the row sum of the rounded P
+    // P = exp2(s - ref) as bf16 (two scores -> one dword) and the row sum of the rounded P
     auto p_pair = [&](const pf_f32x16& s, int x) __attribute__((always_inline)) {
-        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x], a.scale_log2, -m_ref));
-        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(s[2 * x + 1], a.scale_log2, -m_ref));
+        const float p0 = __builtin_amdgcn_exp2f(s[2 * x]);
+        const float p1 = __builtin_amdgcn_exp2f(s[2 * x + 1]);
         const uint32_t pw = pack_kv<F16>(p0, p1);
         l_run = add_pair<F16>(pw, l_run);
         return pw;
@@ -477,9 +496,10 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     };
     // One pipeline step, in issue order (the fences keep the compiler from regrouping it): the 8 MFMAs of the next
     // block's scores, each followed by one eighth of this block's exponentials; then the 8 MFMAs of P.V.  Operand
-    // reads from LDS are issued well ahead of the MFMA that consumes them.
+    // reads from LDS are issued well ahead of the MFMA that consumes them.  s_cur and s_nxt are two register blocks that
+    // swap roles from step to step (no copy).
     //   HAS_NEXT = false: last block of the wavefront, no scores to compute.
-    auto step = [&](pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
+    auto step = [&](const pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
                     __attribute__((always_inline)) {
         constexpr bool HAS_NEXT = decltype(has_next)::value;
         // The 16 MFMA operands of a step (8 K fragments, then 8 V fragments) are one stream of LDS reads, each requested
@@ -494,10 +514,6 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
                 frag[m] = v_frag(vbuf, vkb, (m - 8) >> 2, (m - 8) & 3);
             }
         };
-        if (HAS_NEXT) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) s_nxt[v] = 0.0f;
-        }
 #pragma unroll
         for (int m = 0; m < PD; ++m) request(m);
         __builtin_amdgcn_sched_barrier(0);
@@ -505,7 +521,7 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         for (int ks = 0; ks < 8; ++ks) {
             request(ks + PD);
             pw[ks] = p_pair(s_cur, ks);
-            if (HAS_NEXT) s_nxt = mfma_32x32x16<F16>(frag[ks], qf[ks], s_nxt);
+            if (HAS_NEXT) s_nxt = mfma_32x32x16<F16>(frag[ks], qf[ks], ks == 0 ? negm : s_nxt);
             __builtin_amdgcn_sched_barrier(0);
         }
         pf_bf16x8 pfrag[2];
@@ -527,46 +543,37 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     // written at the top of iteration t into the buffer tile t - 2 used (every wavefront left it before the barrier of
     // iteration t - 1) and becomes visible at the barrier in the middle of iteration t, in time for the scores of its
     // first block.
+    // Every wavefront walks all blocks of the workgroup's tiles: the blocks that lie wholly above a wavefront's diagonal
+    // (at most two of up to several hundred, the workgroup spans BT query times) are masked like the diagonal ones
+    // and contribute zeros, which keeps the loop free of per-wavefront branches.
     const int ntiles = (k_end + PF2_BN - 1) / PF2_BN;
-    const int nb_w = vis_hi >= 0 ? min(vis_hi / 32 + 1, 2 * ntiles) : 0;   // blocks this wavefront visits
     if (ntiles > 0) {
-        pf_f32x16 s_cur;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) s_cur[v] = 0.0f;
+        pf_f32x16 s_a, s_b;   // scores of the current and of the next block, roles swapping every step
         fetch(0);
         publish(pf2_lds);
         fetch(PF2_BN);
         __syncthreads();
-        if (nb_w > 0) {
-            s_cur = qk(pf2_lds, 0);
-            prepare(s_cur, 0);
-        }
+        s_a = qk(pf2_lds, 0);
+        prepare(s_a, 0, std::true_type{});
         int i0 = 0, i1 = 1;   // buffer index of tile t and of tile t + 1
-        for (int t = 0; t < ntiles; ++t) {
+        for (int t = 0; t + 1 < ntiles; ++t) {
             const char* b0 = pf2_lds + i0 * PF2_BUF;
             char* b1 = pf2_lds + i1 * PF2_BUF;
             publish(b1);
             fetch((t + 2) * PF2_BN);          // unconditional (rows clamped)
-            int blk = 2 * t;
-            pf_f32x16 s_nxt;
-            if (blk + 1 < nb_w) {
-                step(s_cur, s_nxt, b0, 1, b0, 0, std::true_type{});
-                prepare(s_nxt, blk + 1);
-                s_cur = s_nxt;
-            } else if (blk < nb_w) {
-                step(s_cur, s_nxt, b0, 1, b0, 0, std::false_type{});
-            }
+            step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
+            prepare(s_b, 2 * t + 1, std::false_type{});
             __syncthreads();
-            blk = 2 * t + 1;
-            if (blk + 1 < nb_w) {
-                step(s_cur, s_nxt, b1, 0, b0, 1, std::true_type{});
-                prepare(s_nxt, blk + 1);
-                s_cur = s_nxt;
-            } else if (blk < nb_w) {
-                step(s_cur, s_nxt, b1, 0, b0, 1, std::false_type{});
-            }
+            step(s_b, s_a, b1, 0, b0, 1, std::true_type{});
+            prepare(s_a, 2 * t + 2, std::false_type{});
             i0 = i1;
             i1 = i1 == 2 ? 0 : i1 + 1;
+        }
+        {   // the last tile: its second block has no successor
+            const char* b0 = pf2_lds + i0 * PF2_BUF;
+            step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
+            prepare(s_b, 2 * ntiles - 1, std::false_type{});
+            step(s_b, s_a, b0, 0, b0, 1, std::false_type{});
         }
     }
 
@@ -589,9 +596,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
 
 template <int G, bool F16>
 static int launch_prefill(const PrefillArgs& a, int nseg, hipStream_t st) {
-    // short chunks: 16 queries per wavefront waste fewer MFMA columns; a non-positive scale: the large kernel takes
-    // row maxima before scaling, which needs scale > 0
-    if (a.q_len < 64 || !(a.scale_log2 > 0.0f)) {
+    // short chunks: 16 queries per wavefront waste fewer MFMA columns
+    if (a.q_len < 64) {
         using C = SmallCfg<G>;
         const int tiles = (a.q_len + C::BT - 1) / C::BT;
         hipLaunchKernelGGL((prefill_small_kernel<G, F16>), dim3(tiles, nseg), dim3(C::THREADS), 0, st, a);
