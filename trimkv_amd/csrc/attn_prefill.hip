@@ -278,6 +278,7 @@ constexpr int PF2_VROW = PF2_BN * 2 + 16;           // bytes per V^T row (one d,
 constexpr int PF2_VBYTES = PF_D * PF2_VROW;         // 16384
 constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
 constexpr int PF2_LDS = 3 * PF2_BUF;                // three tiles in rotation
+constexpr int PF2_PD = 3;                           // LDS operand reads in flight ahead of the MFMA that consumes them
 constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a row maximum grows by more than 2^6
 
 // A workgroup is always 8 wavefronts (two per SIMD, 256 registers each) and owns 256 / G consecutive query times
@@ -452,8 +453,16 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     // Mask (diagonal blocks only), row maximum, and the lazy move of the exponent reference: O and l are
     // rescaled only when some row of the wavefront outgrows its reference by 2^PF2_LAZY.  FIRST: the wavefront's first
     // block puts the reference on the row maximum wherever it lies (O and l are still zero: nothing to rescale).
-    auto prepare = [&](pf_f32x16& s, int blk, auto first_c) __attribute__((always_inline)) {
+    // tmax: the maximum of s before masking, as the step computed it under its P.V MFMAs (ignored by FIRST).
+    auto max16 = [&](const pf_f32x16& s) __attribute__((always_inline)) {
+        float t = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) t = __builtin_fmaxf(t, s[v]);
+        return t;
+    };
+    auto prepare = [&](pf_f32x16& s, int blk, float tmax, auto first_c) __attribute__((always_inline)) {
         constexpr bool FIRST = decltype(first_c)::value;
+        if (FIRST) tmax = max16(s);
         if (blk * 32 + 31 > vis_lo) {   // wave-uniform: some query of the wavefront does not see the whole block
             // (the empty volatile statement keeps this a branch: as 48 speculated selects it would run for every block)
             asm volatile("" ::: );
@@ -462,10 +471,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
                 const int key = blk * 32 + 8 * (v >> 2) + 4 * hl + (v & 3);
                 s[v] = key <= vis_j ? s[v] : PF_NEG;
             }
+            tmax = max16(s);
         }
-        float tmax = s[0];
-#pragma unroll
-        for (int v = 1; v < 16; ++v) tmax = __builtin_fmaxf(tmax, s[v]);
         if (FIRST || __builtin_amdgcn_ballot_w64(tmax > PF2_LAZY) != 0) {
             const float t2 = __builtin_fmaxf(tmax, __shfl_xor(tmax, 32, 64));   // both halves of a query agree on the reference
             // how far the reference moves: onto the maximum (first block; not at all for a row that sees nothing), else up only
@@ -499,12 +506,13 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     // reads from LDS are issued well ahead of the MFMA that consumes them.  s_cur and s_nxt are two register blocks that
     // swap roles from step to step (no copy).
     //   HAS_NEXT = false: last block of the wavefront, no scores to compute.
+    // Returns the row maximum of s_nxt (this lane's 16 scores), computed in the shadow of the P.V MFMAs.
     auto step = [&](const pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
-                    __attribute__((always_inline)) {
+                    __attribute__((always_inline)) -> float {
         constexpr bool HAS_NEXT = decltype(has_next)::value;
         // The 16 MFMA operands of a step (8 K fragments, then 8 V fragments) are one stream of LDS reads, each requested
         // PD MFMAs before the one that consumes it: no burst of reads at the start of a step, a few registers in flight.
-        constexpr int PD = 3;
+        constexpr int PD = PF2_PD;
         pf_bf16x8 frag[16];
         uint32_t pw[8];
         auto request = [&](int m) __attribute__((always_inline)) {
@@ -530,12 +538,22 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
             const pf_u32x4 pq = {pw[4 * st], pw[4 * st + 1], pw[4 * st + 2], pw[4 * st + 3]};
             pfrag[st] = __builtin_bit_cast(pf_bf16x8, pq);
         }
+        // the maximum of the next block's scores as a tree of three-input maxima, one or two per P.V MFMA from the third
+        // on (the last score MFMA has landed by then): after the step only the comparison with the reference is left
+        float mt[7];
+        auto max3 = [](float x, float y, float z) __attribute__((always_inline)) { return __builtin_fmaxf(__builtin_fmaxf(x, y), z); };
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             request(8 + i + PD);
             o[i & 3] = mfma_32x32x16<F16>(frag[8 + i], pfrag[i >> 2], o[i & 3]);
+            if (HAS_NEXT) {
+                if (i >= 2 && i <= 6) mt[i - 2] = max3(s_nxt[3 * (i - 2)], s_nxt[3 * (i - 2) + 1], s_nxt[3 * (i - 2) + 2]);
+                if (i == 6) mt[5] = max3(mt[0], mt[1], s_nxt[15]);
+                if (i == 7) mt[6] = max3(mt[2], mt[3], mt[4]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        return HAS_NEXT ? __builtin_fmaxf(mt[5], mt[6]) : 0.0f;
     };
 
     // Pipeline over 32-key blocks: while the exponentials of block b run on the VALU, the MFMA unit computes the scores
@@ -554,25 +572,25 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         fetch(PF2_BN);
         __syncthreads();
         s_a = qk(pf2_lds, 0);
-        prepare(s_a, 0, std::true_type{});
+        prepare(s_a, 0, 0.0f, std::true_type{});
         int i0 = 0, i1 = 1;   // buffer index of tile t and of tile t + 1
         for (int t = 0; t + 1 < ntiles; ++t) {
             const char* b0 = pf2_lds + i0 * PF2_BUF;
             char* b1 = pf2_lds + i1 * PF2_BUF;
             publish(b1);
             fetch((t + 2) * PF2_BN);          // unconditional (rows clamped)
-            step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
-            prepare(s_b, 2 * t + 1, std::false_type{});
+            const float ma = step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
+            prepare(s_b, 2 * t + 1, ma, std::false_type{});
             __syncthreads();
-            step(s_b, s_a, b1, 0, b0, 1, std::true_type{});
-            prepare(s_a, 2 * t + 2, std::false_type{});
+            const float mb = step(s_b, s_a, b1, 0, b0, 1, std::true_type{});
+            prepare(s_a, 2 * t + 2, mb, std::false_type{});
             i0 = i1;
             i1 = i1 == 2 ? 0 : i1 + 1;
         }
         {   // the last tile: its second block has no successor
             const char* b0 = pf2_lds + i0 * PF2_BUF;
-            step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
-            prepare(s_b, 2 * ntiles - 1, std::false_type{});
+            const float ma = step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
+            prepare(s_b, 2 * ntiles - 1, ma, std::false_type{});
             step(s_b, s_a, b0, 0, b0, 1, std::false_type{});
         }
     }
