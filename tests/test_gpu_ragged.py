@@ -248,6 +248,54 @@ def test_single_sequence_floor_branch_credit_skips_an_empty_head():
     _same(d.cache, d.ref)
 
 
+@pytest.mark.parametrize("strategy", ["alpha", "layer_wise_alpha"])
+def test_shared_budget_eviction_enqueues_without_synchronisation(strategy):
+    """The reference's default ragged strategies (one budget per batch element over all layers, cache_utils.py:836-945, or per
+    layer, :740-834) through fused decode steps with torch's synchronisation debugging set to "error": an implicit
+    synchronisation anywhere in update / attention / compress would raise.  The new lengths travel to the host through a
+    pinned buffer in stream order; ``sync_waits`` counts the times a reader had to wait for them (none here: they land
+    long before the next eviction needs them).  The final state must equal the oracle's, fed the same inputs."""
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, get_attention_interface
+    attn = get_attention_interface("db_attn_flash_batched")
+    B, H, L, G, M, buf, P = 2, 4, 3, 2, 48, 8, 80
+    gen = torch.Generator().manual_seed(21)
+    cache, ref = BatchedDynamicBudgetTrimKVCache(), BatchedRaggedCacheRef()
+    cache.fuse_decode_append = True
+    steps = 3 * buf + 3
+    feed = []
+    for S in [P] + [1] * steps:
+        feed.append([(draw_kv(gen, B, H, S), draw_log_beta(gen, B, H, S, sigma=1.5), torch.randn(B, H * G, 1, 128, generator=gen).to(torch.bfloat16))
+                     for _ in range(L)])
+    on_dev = [[(k.to(DEV), v.to(DEV), lb.to(DEV), q.to(DEV)) for (k, v), lb, q in step] for step in feed]
+    pos_dev = [torch.arange(0, P, device=DEV)] + [torch.arange(P + t, P + t + 1, device=DEV) for t in range(steps)]
+    kw = dict(strategy=strategy, memory_size=M, buffer_size=buf)
+    for l in range(L):
+        cache.update(*on_dev[0][l][:3], pos_dev[0], l)
+    cache.compress(**kw)                          # first eviction: builds the device tables (uploads)
+    torch.cuda.synchronize()
+    evictions = 0
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        for t in range(1, steps + 1):
+            for l in range(L):
+                k, v, lb, q = on_dev[t][l]
+                K, V, _, _, fa = cache.update(k, v, lb, pos_dev[t], l)
+                attn(None, q, K, V, None, flash_attn_kwargs=fa)
+            before = cache._lens_inflight
+            cache.compress(**kw)
+            evictions += cache._lens_inflight is not None and cache._lens_inflight is not before
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    assert evictions >= 2 and cache.sync_waits == 0
+    T = 0
+    for (S, step) in zip([P] + [1] * steps, feed):
+        for l, ((k, v), lb, _) in enumerate(step):
+            ref.update(k, v, lb, torch.arange(T, T + S), l)
+        T += S
+        ref.compress(**kw)
+    _same(cache, ref)
+
+
 def test_bf16_log_beta_scores_stay_bf16_in_the_ragged_classes():
     """int64 age * bf16 log beta -> bf16 (age rounded to bf16 first); ties are common, so the kept
     SCORES are compared: the multiset of kept scores must equal the oracle's."""

@@ -90,7 +90,7 @@ class _Slab:
     """Device storage of one layer."""
 
     __slots__ = ("k", "v", "lb", "pos", "seg_len", "cu", "B", "H", "D", "cap", "lens", "max_len", "k4", "v4", "lb3", "pos3", "ptrs", "order",
-                 "pending", "codes", "total", "pieces", "pieces_total", "pieces_age", "pieces_buf")
+                 "pending", "codes", "total", "pieces", "pieces_total", "pieces_age", "pieces_buf", "order_host")
 
     def __init__(self, B, H, D, cap, kv_dtype, lb_dtype, device, ragged: bool):
         nseg = B * H
@@ -105,6 +105,7 @@ class _Slab:
         self.max_len = 0
         self.total = 0  # sum of lens (kept by the ragged caches, which size their split-K chunk from it)
         self.order = None  # ragged caches: segments by decreasing length/budget (dispatch order of the attention launch)
+        self.order_host = None  # the pinned copy it was uploaded from (kept until the next one replaces it)
         self.pending = None  # a one-token append that the next attention call will carry out (see _SlabBacked._defer)
         self.pieces = None   # ragged caches: (device piece list, number of pieces) of the decode-attention launch
         self.pieces_total, self.pieces_age = 0, 0
@@ -638,7 +639,7 @@ class TrimKVCache(_SlabBacked):
                 lo, hi = i * slab.H, (i + nb) * slab.H
                 new.k, new.v, new.lb, new.pos = slab.k[lo:hi], slab.v[lo:hi], slab.lb[lo:hi], slab.pos[lo:hi]
                 new.seg_len, new.cu = slab.seg_len[lo:hi], None
-                new.lens, new.max_len, new.order = slab.lens[lo:hi].copy(), slab.max_len, None
+                new.lens, new.max_len, new.order, new.order_host = slab.lens[lo:hi].copy(), slab.max_len, None, None
                 new.pending, new.total = None, int(new.lens.sum())
                 new.pieces, new.pieces_total, new.pieces_age, new.pieces_buf = None, 0, 0, None
                 new._refresh_views()
@@ -674,7 +675,7 @@ class TrimKVCache(_SlabBacked):
             c.B, c.H, c.D, c.cap = slab.B, slab.H, slab.D, slab.cap
             c.k, c.v, c.lb, c.pos = (t.to(device, copy=True) for t in (slab.k, slab.v, slab.lb, slab.pos))
             c.seg_len, c.cu = slab.seg_len.to(device, copy=True), None
-            c.lens, c.max_len, c.order = slab.lens.copy(), slab.max_len, None
+            c.lens, c.max_len, c.order, c.order_host = slab.lens.copy(), slab.max_len, None, None
             c.pending, c.total = None, slab.total
             c.pieces, c.pieces_total, c.pieces_age, c.pieces_buf = None, 0, 0, None
             c._refresh_views()
@@ -726,6 +727,13 @@ class _RaggedCache(_SlabBacked):
         self.attention_compute_units = 0     # what the piece lists of the decode-attention launches are balanced for; 0: ask the device
         self.attention_replan_steps = 32     # a layer's piece list is rebuilt at least this often
         self._replans = 0
+        # Lengths after a shared-budget eviction come to the host through an asynchronous copy (see _refresh): until it has
+        # landed the host mirrors are upper bounds.  sync_waits counts the times a host reader had to wait for it.
+        self._lens_inflight = None
+        self._lens_pinned: Dict[Any, list] = {}
+        self._analytic_total: Optional[int] = None       # exact grand total of cached tokens while lengths are in flight
+        self._analytic_layer: Optional[Dict[int, int]] = None   # ... and per layer, where the strategy fixes it
+        self.sync_waits = 0
 
     # plain attributes in the reference; a property here because newer HF Cache classes define a
     # read-only `batch_size` of their own
@@ -747,17 +755,38 @@ class _RaggedCache(_SlabBacked):
         return [_EMPTY() if s is None else s.cu for s in self._slabs]
 
     def get_total_cached_tokens(self) -> int:  # cache_utils.py:253-254, 593-594
+        if self._lens_inflight is not None and self._analytic_total is not None:
+            return self._analytic_total       # the eviction's strategy fixes the total: no need to wait for the lengths
+        self._settle(True)
         return int(sum(int(s.lens.sum()) for s in self._slabs if s is not None))
 
     def _layer_tokens(self, layer: int) -> int:
+        inf = self._lens_inflight
+        if inf is not None and layer in inf[2]:      # a layer whose lengths are on their way
+            if self._analytic_layer is not None and layer in self._analytic_layer:
+                return self._analytic_layer[layer]
+            self._settle(True)
         s = self._slabs[layer]
         return 0 if s is None else int(s.lens.sum())
+
+    def _kept_under_shared_budget(self, layers: List[int], segs_per_group: int, budget: int, per_layer: bool):
+        """Token counts after a top-k under a shared budget, from the exact mirrors before it: every budget group keeps
+        min(budget, what it holds).  ``per_layer``: one budget per (layer, group) -> (grand total, {layer: total}); else one
+        budget per group across ``layers`` -> (grand total, None).  Layers outside ``layers`` are counted as they are."""
+        self._settle(True)
+        others = sum(int(s.lens.sum()) for i, s in enumerate(self._slabs) if s is not None and i not in layers)
+        held = np.stack([self._slabs[l].lens.reshape(-1, segs_per_group).sum(axis=1) for l in layers])   # [L, groups]
+        if per_layer:
+            kept = np.minimum(held, budget).sum(axis=1)
+            return others + int(kept.sum()), {l: int(kept[i]) for i, l in enumerate(layers)}
+        return others + int(np.minimum(held.sum(axis=0), budget).sum()), None
 
     def _packed(self, slab: _Slab):
         """The layer in the reference's own layout (cache_utils.py:682-689): ``[sum(n), D]`` rows packed segment after
         segment, indexed by ``cu_seqlens_k``.  A copy, gathered on the device without a host synchronisation (the row
         count comes from the host mirror of the lengths); for readers that index the returned K with the returned
         ``cu_seqlens_k`` themselves, as flash_attn_varlen_func does (attn/flash_attn.py:135-145)."""
+        self._settle(True)
         dev = slab.k.device
         r = torch.arange(slab.total, device=dev, dtype=torch.int32)
         seg = torch.searchsorted(slab.cu[1:], r, right=True)
@@ -769,12 +798,23 @@ class _RaggedCache(_SlabBacked):
 
     def _update(self, key_states, value_states, retention_weights, cache_positions, layer_idx: int, packed: bool = False):
         packed = packed or self.return_packed
+        if self._lens_inflight is not None:
+            self._settle(False)
         if key_states is not None:
             S = key_states.shape[2]
             if layer_idx == 0:
                 self._seen_tokens += S
             self._ensure_layer(layer_idx)
             slab = self._slabs[layer_idx]
+            if self._lens_inflight is not None and slab is not None:
+                if slab.max_len + S > slab.cap:
+                    self._settle(True)    # the bound, not necessarily the cache, has outgrown the slab: get the real lengths first
+                else:
+                    nseg = key_states.shape[0] * key_states.shape[1]
+                    if self._analytic_total is not None:
+                        self._analytic_total += S * nseg
+                    if self._analytic_layer is not None and layer_idx in self._analytic_layer:
+                        self._analytic_layer[layer_idx] += S * nseg
             if not (S == 1 and self.fuse_decode_append and not packed and slab is not None
                     and self._defer(slab, key_states, value_states, retention_weights, cache_positions)):
                 self._append(layer_idx, key_states, value_states, retention_weights, cache_positions)
@@ -980,10 +1020,17 @@ class _RaggedCache(_SlabBacked):
         _lib.check(rc, "trimkv_evict")
         self._keepalive2 = keep_dev
 
-    def _refresh(self, layers: List[int]) -> None:
-        """After an eviction: rebuild cu_seqlens on the device and bring the new lengths to the
-        host -- the one synchronisation an eviction costs (the reference pays O(B*L*Hkv))."""
+    def _refresh(self, layers: List[int], total_after: Optional[int] = None, layer_totals: Optional[Dict[int, int]] = None) -> None:
+        """After a shared-budget eviction: rebuild cu_seqlens on the device and start the new lengths on their way to the
+        host -- a copy into pinned memory in stream order, no synchronisation (the reference pays O(B*L*Hkv) ``.item()``
+        calls here).  Until the copy has landed (``_settle``) the host mirrors keep their old values, which are upper bounds:
+        good enough to launch appends and attention (the kernels read the real lengths on the device; a piece list planned
+        for the old lengths is scaled to them).  ``total_after`` / ``layer_totals``: the exact token counts after the
+        eviction where the strategy fixes them (a budget that was binding is spent exactly), so that the next trigger
+        decision does not have to wait for the lengths either."""
         lib = _lib.load()
+        if not layers:
+            return
         if len(layers) > 1 and self._layers_alike(layers):
             t = self._device_tables(layers)
             s0 = self._slabs[layers[0]]
@@ -994,15 +1041,63 @@ class _RaggedCache(_SlabBacked):
                 slab = self._slabs[l]
                 rc = lib.trimkv_build_cu_seqlens(slab.seg_len.data_ptr(), slab.nseg, slab.cu.data_ptr(), _lib.current_stream(slab.k.device))
                 _lib.check(rc, "trimkv_build_cu_seqlens")
-        if layers:
-            lens = torch.stack([self._slabs[l].seg_len for l in layers]).cpu().numpy().astype(np.int64)
-            for i, l in enumerate(layers):
-                self._slabs[l].lens = lens[i].copy()
-                self._slabs[l].max_len = int(lens[i].max())
-                self._slabs[l].total = int(lens[i].sum())
-                self._slabs[l].pieces = None
-                if getattr(self, "_budgets_host", None) is None:
-                    self._set_dispatch_order(self._slabs[l], lens[i])
+        if self._lens_inflight is not None and not self._settle(False):
+            # an older copy that has not landed is superseded by this one (the newer lengths are the truth) -- unless it
+            # carries layers that this eviction did not touch: those must not be lost
+            if not set(self._lens_inflight[2]) <= set(layers):
+                self._settle(True)
+        nseg = self._slabs[layers[0]].nseg
+        ragged_shapes = any(self._slabs[l].nseg != nseg for l in layers)
+        if ragged_shapes:                  # layers of different shapes: rare, take the simple road
+            for l in layers:
+                self._install_lens(l, self._slabs[l].seg_len.cpu().numpy().astype(np.int64))
+            self._lens_inflight, self._analytic_total, self._analytic_layer = None, None, None
+            return
+        dev_lens = torch.stack([self._slabs[l].seg_len for l in layers])
+        key = (len(layers), nseg)
+        ring = self._lens_pinned.get(key)
+        if ring is None:
+            ring = self._lens_pinned[key] = [[torch.empty(len(layers), nseg, dtype=torch.int32, pin_memory=True) for _ in range(2)], 0]
+        host = ring[0][ring[1]]
+        ring[1] ^= 1
+        host.copy_(dev_lens, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        # baseline: the (upper-bound) mirrors at this moment; appends until the copy lands add to both sides alike
+        base = {l: self._slabs[l].lens.copy() for l in layers}
+        self._lens_inflight = (ev, host, list(layers), base, dev_lens)
+        self._analytic_total, self._analytic_layer = total_after, layer_totals
+        for l in layers:
+            self._slabs[l].pieces = None   # lengths changed wholesale: plan afresh (for the bounds now, exactly once settled)
+
+    def _install_lens(self, layer: int, lens: np.ndarray) -> None:
+        slab = self._slabs[layer]
+        slab.lens = lens
+        slab.max_len = int(lens.max()) if lens.size else 0
+        slab.total = int(lens.sum())
+        slab.pieces = None
+        if getattr(self, "_budgets_host", None) is None:
+            self._set_dispatch_order(slab, lens)
+
+    def _settle(self, block: bool) -> bool:
+        """Bring the host mirrors up to date with lengths that are on their way from the device.  ``block`` False: only if
+        the copy has landed already (the usual case one decode step after the eviction).  Returns whether the mirrors are
+        exact now."""
+        inf = self._lens_inflight
+        if inf is None:
+            return True
+        ev, host, layers, base, _ = inf
+        if not ev.query():
+            if not block:
+                return False
+            self.sync_waits += 1
+            ev.synchronize()
+        fresh = host.numpy().astype(np.int64)
+        for i, l in enumerate(layers):
+            slab = self._slabs[l]
+            self._install_lens(l, fresh[i] + (slab.lens - base[l]))   # + what was appended since the eviction
+        self._lens_inflight, self._analytic_total, self._analytic_layer = None, None, None
+        return True
 
     @staticmethod
     def _set_dispatch_order(slab: _Slab, key) -> None:
@@ -1011,8 +1106,9 @@ class _RaggedCache(_SlabBacked):
         key = np.asarray(key, dtype=np.int64)
         if key.size < 16 or int(key.max()) * key.size <= 1.5 * max(1, int(key.sum())):
             slab.order = None
-        else:
-            slab.order = torch.from_numpy(np.argsort(-key, kind="stable").astype(np.int32)).to(slab.k.device)
+        else:   # through pinned memory, in stream order: a copy from pageable memory would wait for the whole stream
+            host = torch.from_numpy(np.argsort(-key, kind="stable").astype(np.int32)).pin_memory()
+            slab.order, slab.order_host = host.to(slab.k.device, non_blocking=True), host
 
     def set_budgets(self, budgets) -> None:
         """Give every segment its own token budget: ``budgets`` is ``[nseg]`` (all layers alike) or
@@ -1031,6 +1127,7 @@ class _RaggedCache(_SlabBacked):
         (cache_utils.py:508-521).  The trigger is evaluated on the host mirror of the lengths and
         again per segment on the device; no host synchronisation happens here."""
         self._flush_all()
+        self._settle(True)
         every = [l for l in range(len(self._slabs)) if self._slabs[l] is not None]
         layers = every if layers is None else list(layers)
         if not layers:
@@ -1099,6 +1196,7 @@ class _RaggedCache(_SlabBacked):
     def segment_positions(self):
         """Per layer, per segment: retained absolute positions (host tensors)."""
         self._flush_all()
+        self._settle(True)
         out = []
         for s in self._slabs:
             pos = s.pos.cpu()
@@ -1129,6 +1227,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
     def get_cache_length(self, layer_idx: int = 0, batch_idx: int = 0, head_idx: int = 0) -> int:
         if layer_idx >= len(self._slabs) or self._slabs[layer_idx] is None:
             return 0
+        self._settle(True)
         return int(self._slabs[layer_idx].lens[batch_idx * self.num_kv_heads + head_idx])
 
     @torch.inference_mode()
@@ -1139,7 +1238,7 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
         num_layers = len(self._slabs) if num_layers is None else num_layers
         H = self.num_kv_heads if num_key_value_heads is None else num_key_value_heads
         B = self.batch_size
-        if self.get_total_cached_tokens() <= B * H * (memory_size + buffer_size) * num_layers and "threshold" not in strategy:
+        if "threshold" not in strategy and self.get_total_cached_tokens() <= B * H * (memory_size + buffer_size) * num_layers:
             return  # cache_utils.py:714-717
         if "layer_wise" in strategy:  # cache_utils.py:719-729, 740-834
             base = strategy.replace("layer_wise_", "")
@@ -1148,6 +1247,8 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
             todo = [l for l in range(num_layers) if self._layer_tokens(l) > B * H * (memory_size + buffer_size)]
             if not todo:
                 return
+            # what the layers hold afterwards is fixed by the budget unless the floor tops heads up: known without a read-back
+            after = self._kept_under_shared_budget(todo, H, memory_size * H, True) if floor_budget_ratio <= 0 else (None, None)
             alike = self._layers_alike(todo)
             for part in ([todo] if alike else [[l] for l in todo]):   # layers of one shape go through together
                 if floor_budget_ratio > 0:
@@ -1164,20 +1265,22 @@ class BatchedDynamicBudgetTrimKVCache(_RaggedCache):
                 else:
                     thr, take, tie_base, _ = self._group_select_each(part, H, memory_size * H, base)
                     self._compact_layers(part, H, thr, take, tie_base, base)
-            self._refresh(todo)
+            self._refresh(todo, *after)
         else:  # cache_utils.py:836-945; floor_budget_ratio is not used by this variant
-            tokens_per_batch = sum(self._layer_tokens(l) for l in range(num_layers)) // B
-            if tokens_per_batch <= num_layers * H * (memory_size + buffer_size) and "threshold" not in strategy:
-                return
+            if "threshold" not in strategy:
+                held = self.get_total_cached_tokens() if num_layers == len(self._slabs) else sum(self._layer_tokens(l) for l in range(num_layers))
+                if held // B <= num_layers * H * (memory_size + buffer_size):
+                    return
             if strategy not in ("alpha", "knorm_alpha", "alpha_threshold", "knorm_alpha_threshold"):
                 raise ValueError(f"Unknown compression strategy: {strategy}")
             layers = list(range(num_layers))
             threshold = None
             if "threshold" in strategy:
                 threshold = self._log_threshold(alpha_threshold, self._slabs[layers[0]].lb.dtype)
+            after = self._kept_under_shared_budget(layers, H, num_layers * H * memory_size, False) if threshold is None else (None, None)
             thr, take, tie_base, _ = self._group_select(layers, H, num_layers * H * memory_size, strategy, threshold)
             self._compact_layers(layers, H, thr, take, tie_base, strategy)
-            self._refresh(layers)
+            self._refresh(layers, *after)
 
     def log(self):
         positions = self.segment_positions()
@@ -1201,6 +1304,7 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
     def get_cache_length(self, layer_idx: int = 0, head_idx: int = 0) -> int:
         if layer_idx >= len(self._slabs) or self._slabs[layer_idx] is None:
             return 0
+        self._settle(True)
         return int(self._slabs[layer_idx].lens[head_idx])
 
     @torch.inference_mode()
@@ -1216,15 +1320,16 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             if todo and base not in ("alpha", "knorm_alpha"):
                 raise ValueError(f"Unknown compression strategy: {base}")
             if todo:
+                after = self._kept_under_shared_budget(todo, H, H * memory_size, True)
                 alike = self._layers_alike(todo)
                 for part in ([todo] if alike else [[l] for l in todo]):
                     thr, take, tie_base, _ = self._group_select_each(part, H, H * memory_size, base)
                     self._compact_layers(part, H, thr, take, tie_base, base)
-                self._refresh(todo)
+                self._refresh(todo, *after)
             return
         # all layers at once, cache_utils.py:418-536
         total_budget = num_layers * H * memory_size
-        if num_layers * H * (memory_size + buffer_size) > self.get_total_cached_tokens() and "threshold" not in strategy:
+        if "threshold" not in strategy and num_layers * H * (memory_size + buffer_size) > self.get_total_cached_tokens():
             return
         if strategy not in ("alpha", "knorm_alpha", "alpha_threshold", "knorm_alpha_threshold"):
             raise ValueError(f"Unknown compression strategy: {strategy}")
@@ -1233,9 +1338,10 @@ class DynamicBudgetTrimKVCache(_RaggedCache):
             threshold = None
             if "threshold" in strategy:
                 threshold = self._log_threshold(alpha_threshold, self._slabs[layers[0]].lb.dtype)
+            after = self._kept_under_shared_budget(layers, H, total_budget, False) if threshold is None else (None, None)
             thr, take, tie_base, _ = self._group_select(layers, H, total_budget, strategy, threshold)
             self._compact_layers(layers, H, thr, take, tie_base, strategy)
-            self._refresh(layers)
+            self._refresh(layers, *after)
             return
         assert "threshold" not in strategy, "Thresholding strategy is not compatible with floor_budget_ratio > 0"
         adaptive = int(total_budget * (1 - floor_budget_ratio))

@@ -206,28 +206,26 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
     const int piece = threadIdx.x & (lpr - 1), rl = threadIdx.x >> lpr_shift;
     const bool piece_ok = (piece << 4) < row_bytes;   // rows that are not a power of two long (head_dim 96) leave lanes idle
     const int tile_rows = rpp * EV_ROW_PASSES;
-    for (int base = (first_moved / tile_rows) * tile_rows; base < kept; base += tile_rows) {
-        uint4 kk[EV_ROW_PASSES], vv[EV_ROW_PASSES];
-        bool mv[EV_ROW_PASSES];
+    // Two tiles of rows are in flight: while tile t waits at the barrier and is stored, the loads of tile t + 1 are already
+    // under way.  That is safe in place: the sources of tile t + 1 lie at or behind its own destinations, i.e. behind every
+    // destination of tile t.  Loads are unconditional (rows past the end and idle lanes re-read a valid piece) so that the
+    // wait for tile t is exact and leaves the loads of tile t + 1 outstanding; only the stores are predicated.
+    const int piece_off = piece_ok ? (piece << 4) : 0;
+    auto issue = [&](int base, uint4 (&kk)[EV_ROW_PASSES], uint4 (&vv)[EV_ROW_PASSES], bool (&mv)[EV_ROW_PASSES]) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < EV_ROW_PASSES; ++p) {
             const int r = base + p * rpp + rl;
-            mv[p] = false;
-            kk[p] = make_uint4(0, 0, 0, 0);
-            vv[p] = make_uint4(0, 0, 0, 0);
-            if (r < kept && piece_ok) {
-                const int src = (int)idx[r];
-                if (src != r) {
-                    mv[p] = true;
-                    const int64_t o = (int64_t)src * row_bytes + (piece << 4);
-                    kk[p] = load_stream(kseg + o);   // rows move once and are next read a whole decode step later:
-                    vv[p] = load_stream(vseg + o);   // streaming (non-temporal) loads and stores
-                }
-            }
+            const int src = (int)idx[min(r, kept - 1)];
+            mv[p] = r < kept && piece_ok && src != r;
+            const int64_t o = (int64_t)src * row_bytes + piece_off;
+            kk[p] = load_stream(kseg + o);   // rows move once and are next read a whole decode step later:
+            vv[p] = load_stream(vseg + o);   // streaming (non-temporal) loads and stores
         }
+    };
+    auto retire = [&](int base, uint4 (&kk)[EV_ROW_PASSES], uint4 (&vv)[EV_ROW_PASSES], const bool (&mv)[EV_ROW_PASSES]) __attribute__((always_inline)) {
 #pragma unroll
         for (int p = 0; p < EV_ROW_PASSES; ++p) { land(kk[p]); land(vv[p]); }
-        __syncthreads();
+        __syncthreads();   // every thread holds its rows of this tile: the tile's destinations may be overwritten
 #pragma unroll
         for (int p = 0; p < EV_ROW_PASSES; ++p) {
             if (mv[p]) {
@@ -236,6 +234,23 @@ __device__ __forceinline__ void move_segment(char* kseg, char* vseg, void* lbseg
                 store_stream(kseg + o, kk[p]);
                 store_stream(vseg + o, vv[p]);
             }
+        }
+    };
+    {
+        uint4 ka[EV_ROW_PASSES], va[EV_ROW_PASSES], kb[EV_ROW_PASSES], vb[EV_ROW_PASSES];
+        bool ma[EV_ROW_PASSES], mb[EV_ROW_PASSES];
+        int base = (first_moved / tile_rows) * tile_rows;
+        if (base < kept) issue(base, ka, va, ma);
+        while (base < kept) {
+            const bool more = base + tile_rows < kept;          // uniform across the workgroup
+            if (more) issue(base + tile_rows, kb, vb, mb);
+            retire(base, ka, va, ma);
+            base += tile_rows;
+            if (!more) break;
+            const bool more2 = base + tile_rows < kept;
+            if (more2) issue(base + tile_rows, ka, va, ma);
+            retire(base, kb, vb, mb);
+            base += tile_rows;
         }
     }
     __syncthreads();
