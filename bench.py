@@ -764,7 +764,7 @@ def main():
         fused = cache.fuse_decode_append   # the sampled launch then also writes the new rows
         avg_bytes = sum(attn_bytes(n) for n in lens) / len(lens) + (append_bytes if fused else 0)
         achieved = avg_bytes / avg_s / 1e9
-        ratio, src = measured_traffic_ratio() if args.config == 3 else (None, None)
+        ratio, src = measured_traffic_ratio(args.config) if not args.gate else (None, None)
         tf = lambda b: "true" if b else "false"
         targs = f"<{G}, 16, false, {tf(fused)}, {tf(fused and args.gate)}>"   # group, 16-byte pieces per row, fp16, APPEND, GATED
         pps = hip_attn._uniform_cut(nseg, M + buf) if not args.chunk else 0
