@@ -7,8 +7,8 @@
 // plus the chunk's own tokens <= t, i.e. keys j <= n - Q_LEN + t.
 //
 // Two kernels share the formulation below.  prefill_attn_kernel (chunks of 64 queries and more) gives
-// a wavefront 32 queries of one head and uses v_mfma_f32_32x32x16_bf16 on 64-key tiles that are
-// rotating through three LDS buffers, V stored transposed; prefill_small_kernel (short chunks) gives a wavefront
+// a wavefront 32 queries and uses v_mfma_f32_32x32x16_bf16 on 64-key tiles that LDS-direct loads
+// rotate through four LDS buffers; prefill_small_kernel (short chunks) gives a wavefront
 // 16 queries and uses v_mfma_f32_16x16x32_bf16 on 32-key tiles.
 //
 // A workgroup owns BT consecutive query times of one segment for all G query heads of its KV head,
@@ -20,10 +20,9 @@
 // per-query quantity (running max, sum, rescale factor) lives in the lane that needs it, and the
 // probabilities a lane holds after the first product are exactly the keys its B operand of the
 // second product wants -- P never crosses lanes.  V is row-major in memory, so its A operand
-// (8 keys at one d) needs a transposition: the large kernel transposes while it stages the tile
-// (key pairs merged with v_perm_b32, written as dwords into a [d][key slot] array whose slot order
-// is the order in which the MFMA output hands a lane its keys); the small kernel gathers 8 dwords
-// (d, d+1) per lane and splits them into an even-d and an odd-d operand.
+// (8 keys at one d) needs a transposition: the large kernel reads it with the transposing LDS read
+// (ds_read_b64_tr_b16); the small kernel gathers 8 dwords (d, d+1) per lane and splits them into an
+// even-d and an odd-d operand.
 #include "common.hip.h"
 #include <type_traits>
 
@@ -266,18 +265,31 @@ __global__ __launch_bounds__(SmallCfg<G>::THREADS) void prefill_small_kernel(Pre
 //   C (32 x 32): column l % 32, register v holds row 8 * (v / 4) + 4 * hl + v % 4
 // S^T = K . Q^T per 32-key block: after it a lane holds, for its query, keys 8c + 4hl + i (c, i in 0..3).
 // The second product consumes 16 keys per MFMA; step st takes from lane half hl the keys of c = 2st and
-// 2st + 1, i.e. registers v = 8st .. 8st + 7 in order.  The V^T tile is stored so that exactly those
-// 8 keys are 16 contiguous bytes: slot(key) = 16 * (key / 16) + 8 * hl(key) + e(key).
+// 2st + 1, i.e. registers v = 8st .. 8st + 7 in order: keys 16 st + 4 hl + 0..3 and 16 st + 8 + 4 hl + 0..3.
+//
+// K and V tiles are staged by LDS-direct loads (global_load_lds_dwordx4): a tile never passes through registers and
+// no VALU instruction takes part in staging.
+// LDS: four K tiles [64 rows][256 B] in the low 64 KB, four V tiles (also row-major) in the next 64 KB.  A wavefront's
+// load instruction fills 1 KB (lane l lands at +16 l), i.e. four whole rows; which 16-byte piece of global memory a
+// lane fetches is free, and that is where the bank swizzle comes from:
+//   K: piece c of row r sits at position c ^ (r & 15): the 16 rows a b128 fragment read touches (one piece index,
+//      consecutive rows) fall on all 64 banks.
+//   V: the 32-byte pair p of row r sits at pair position p ^ (2 (r & 3)).  The A operand of O^T += V^T.P^T (8 keys at
+//      one d per lane) is read with two ds_read_b64_tr_b16: within 16 lanes, lane i supplies 8 bytes (4 d of one key,
+//      key = base + i / 4, d = d0 + 4 (i % 4) ..) and receives the four keys base .. base + 3 at d = d0 + i.
+// The compiler does not see the LDS-direct loads (inline assembly: the builtin would make it wait for all of them before
+// every LDS read), so it neither counts them nor waits for them: every wait is written out in the kernel, including
+// the one before the wavefront ends.
 // ---------------------------------------------------------------------------------------------
 typedef float pf_f32x16 __attribute__((ext_vector_type(16)));
+typedef short pf_s16x4 __attribute__((ext_vector_type(4)));
+#define PF_LDS3 __attribute__((address_space(3)))
 
 constexpr int PF2_BN = 64;                          // keys per tile (two 32-key blocks)
-constexpr int PF2_KROW = 272;                       // bytes per staged K row
-constexpr int PF2_KBYTES = PF2_BN * PF2_KROW;       // 17408
-constexpr int PF2_VROW = PF2_BN * 2 + 16;           // bytes per V^T row (one d, 64 key slots): 9 x 16 bytes, so 16 consecutive rows cover all banks
-constexpr int PF2_VBYTES = PF_D * PF2_VROW;         // 16384
-constexpr int PF2_BUF = PF2_KBYTES + PF2_VBYTES;    // 33792
-constexpr int PF2_LDS = 3 * PF2_BUF;                // three tiles in rotation
+constexpr int PF2_NBUF = 4;                         // tiles in rotation: two being read, two on their way
+constexpr int PF2_TILE = PF2_BN * 256;              // bytes of one K (or V) tile
+constexpr int PF2_VBASE = PF2_NBUF * PF2_TILE;      // 65536: K tiles below, V tiles above
+constexpr int PF2_LDS = 2 * PF2_NBUF * PF2_TILE;    // 131072
 constexpr int PF2_PD = 3;                           // LDS operand reads in flight ahead of the MFMA that consumes them
 constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a row maximum grows by more than 2^6
 
@@ -287,37 +299,32 @@ constexpr float PF2_LAZY = 6.0f;                    // O is rescaled only when a
 // spread of a wavefront's causal limits small.
 constexpr int PF2_WAVES = 8;
 constexpr int PF2_THREADS = PF2_WAVES * 64;
-constexpr int PF2_KPIECES = PF2_BN * 16 / PF2_THREADS;          // 16-byte pieces of K per thread (2)
-constexpr int PF2_VPIECES = (PF2_BN / 2) * 16 / PF2_THREADS;    // (key pair, 8 d) pieces of V per thread (1)
-static_assert(PF2_KPIECES * PF2_THREADS == PF2_BN * 16 && PF2_VPIECES * PF2_THREADS == (PF2_BN / 2) * 16, "tile must divide over the workgroup");
+static_assert(PF2_THREADS * 2 * 16 == PF2_TILE, "a thread stages two 16-byte pieces of K and two of V per tile");
 
-// V staging piece p of a tile -> (key-slot pair, 16-byte chunk of d).  A wavefront takes 16 slot pairs x 4 chunks:
-// its dword writes into V^T (row stride 36 words) then fall on 32 different banks, and its loads are 64-byte runs.
-__device__ __forceinline__ int pf2_vpiece_sp(int p) { return (p & 15) + 16 * ((p >> 6) & 1); }
-__device__ __forceinline__ int pf2_vpiece_dchunk(int p) { return ((p >> 4) & 3) + 4 * (p >> 7); }
-// key (0..63) of the tile that sits in V^T slot `slot`
-__device__ __forceinline__ int pf2_key_of_slot(int slot) {
-    const int kb = slot >> 5, st = (slot >> 4) & 1, hl = (slot >> 3) & 1, e = slot & 7;
-    return kb * 32 + st * 16 + hl * 4 + (e & 3) + ((e >> 2) << 3);
+// One LDS-direct load of 16 bytes per lane: lane l's bytes land at LDS address lds_addr + 16 l.
+__device__ __forceinline__ void pf2_load_to_lds(const char* sbase, uint32_t voff, uint32_t lds_addr) {
+    uint32_t saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved) : "v"(voff), "s"(sbase), "s"(lds_addr) : "memory");
 }
 
 template <bool F16>
 __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) char pf2_lds[];
+    PF_LDS3 char* const lds3 = (PF_LDS3 char*)pf2_lds;
+    const uint32_t lds0 = (uint32_t)(uintptr_t)lds3;
 
     // Workgroups are handed to the 8 XCDs round robin in dispatch order (x fastest), and each XCD has its own L2.  All
     // query tiles of a segment read the same K/V, so they are mapped to one XCD (segment s on XCD s % 8, its tiles in
     // consecutive turns of that XCD, later times first: they see more keys): the K/V tiles that several of them walk at
     // about the same time are then fetched into one L2 instead of eight.
     int seg = blockIdx.y, tile = (int)gridDim.x - 1 - (int)blockIdx.x;
-#ifndef TRIMKV_PF_NO_XCD_MAP
     if ((gridDim.y & 7) == 0) {
         const int lin = (int)blockIdx.y * (int)gridDim.x + (int)blockIdx.x;
         const int turn = lin >> 3;
         seg = (lin & 7) + 8 * (turn / (int)gridDim.x);
         tile = (int)gridDim.x - 1 - turn % (int)gridDim.x;
     }
-#endif
     const int b = seg / a.kv_heads, h = seg - b * a.kv_heads;
     int n = a.seg_len ? a.seg_len[seg] : a.max_len;
     n = max(0, min(n, a.max_len));
@@ -376,80 +383,65 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
     const int vis_lo = n - Q + t_w_first;                     // ... the wavefront's first query
     const int last_row = max(n - 1, 0);
 
-    // ---- staging: global -> registers -> LDS (K row-major, V transposed) ----
-    // Per-thread pieces are fixed; only the tile base moves.  Rows are addressed as 32-bit byte offsets from the
-    // segment's (wave-uniform) base and clamped to the last row, so every load is unconditional.
-    pf_u32x4 kst[PF2_KPIECES], vst[PF2_VPIECES][2];
+    // ---- staging: global -> LDS ----
+    // Thread tid fetches, for K and for V, one 16-byte piece of row tid / 16 and one of row 32 + tid / 16 of the tile; the
+    // piece it fetches is the one whose swizzled position is tid % 16 (hd < 128: pieces past the row re-read its last one,
+    // q is zero there and those columns of O are not stored).
     const uint32_t row_bytes = (uint32_t)a.hd * 2u;
     const char* kseg = a.k + row0 * (int64_t)row_bytes;
     const char* vseg = a.v + row0 * (int64_t)row_bytes;
-    int k_row[PF2_KPIECES], v_row[PF2_VPIECES];
-    uint32_t k_col[PF2_KPIECES], v_col[PF2_VPIECES];
-#pragma unroll
-    for (int i = 0; i < PF2_KPIECES; ++i) {
-        const int p = tid + i * PF2_THREADS;
-        k_row[i] = p >> 4;
-        k_col[i] = min((uint32_t)(p & 15) * 16u, row_bytes - 16u);   // pieces past a short row re-read its last one
-    }
-#pragma unroll
-    for (int i = 0; i < PF2_VPIECES; ++i) {
-        const int p = tid + i * PF2_THREADS;
-        v_row[i] = pf2_key_of_slot(pf2_vpiece_sp(p) * 2);      // slots 2sp, 2sp + 1 hold keys key, key + 1
-        v_col[i] = min((uint32_t)pf2_vpiece_dchunk(p) * 16u, row_bytes - 16u);
-    }
-    auto fetch = [&](int kbase) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < PF2_KPIECES; ++i) {
-            const uint32_t off = (uint32_t)min(kbase + k_row[i], last_row) * row_bytes + k_col[i];
-            kst[i] = *(const pf_u32x4*)(kseg + off);
-        }
-#pragma unroll
-        for (int i = 0; i < PF2_VPIECES; ++i) {
-            const uint32_t o0 = (uint32_t)min(kbase + v_row[i], last_row) * row_bytes + v_col[i];
-            const uint32_t o1 = (uint32_t)min(kbase + v_row[i] + 1, last_row) * row_bytes + v_col[i];
-            vst[i][0] = *(const pf_u32x4*)(vseg + o0);
-            vst[i][1] = *(const pf_u32x4*)(vseg + o1);
-        }
-    };
-    auto publish = [&](char* buf) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < PF2_KPIECES; ++i) {
-            const int p = tid + i * PF2_THREADS;
-            *(pf_u32x4*)(buf + (p >> 4) * PF2_KROW + (p & 15) * 16) = kst[i];
-        }
-#pragma unroll
-        for (int i = 0; i < PF2_VPIECES; ++i) {
-            const int p = tid + i * PF2_THREADS;
-            {
-                const int sp = pf2_vpiece_sp(p), dchunk = pf2_vpiece_dchunk(p);
-                const pf_u32x4 lo = vst[i][0], hi = vst[i][1];
-                char* vt = buf + PF2_KBYTES;
-#pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const int d0 = dchunk * 8 + 2 * x;
-                    const uint32_t ev = __builtin_amdgcn_perm(hi[x], lo[x], 0x05040100u);   // (key, key + 1) at d0
-                    const uint32_t od = __builtin_amdgcn_perm(hi[x], lo[x], 0x07060302u);   // ... at d0 + 1
-                    *(uint32_t*)(vt + d0 * PF2_VROW + sp * 4) = ev;
-                    *(uint32_t*)(vt + (d0 + 1) * PF2_VROW + sp * 4) = od;
-                }
-            }
+    const int st_row = tid >> 4, st_pos = tid & 15;
+    const uint32_t st_kcol = min((uint32_t)(st_pos ^ (st_row & 15)) * 16u, row_bytes - 16u);
+    const uint32_t st_vcol = min((uint32_t)((((st_pos >> 1) ^ (2 * (st_row & 3))) << 1) | (st_pos & 1)) * 16u, row_bytes - 16u);
+    const uint32_t st_koff = (uint32_t)st_row * row_bytes + st_kcol;     // offsets inside a tile whose 64 rows all exist
+    const uint32_t st_voff = (uint32_t)st_row * row_bytes + st_vcol;
+    auto request_tile = [&](int tt, int buf) __attribute__((always_inline)) {
+        const int kbase = tt * PF2_BN;
+        const uint32_t dk = lds0 + buf * PF2_TILE + w * 1024, dv = dk + PF2_VBASE;
+        if (kbase + PF2_BN <= n) {   // wave-uniform; the tile's base goes into the scalar base address
+            const char* kt = kseg + (uint32_t)kbase * row_bytes;
+            const char* vt = vseg + (uint32_t)kbase * row_bytes;
+            pf2_load_to_lds(kt, st_koff, dk);
+            pf2_load_to_lds(kt + 32 * row_bytes, st_koff, dk + PF2_TILE / 2);
+            pf2_load_to_lds(vt, st_voff, dv);
+            pf2_load_to_lds(vt + 32 * row_bytes, st_voff, dv + PF2_TILE / 2);
+        } else {                     // rows past the segment's end are replaced by its last row (finite values, masked keys)
+            const uint32_t r0 = (uint32_t)min(kbase + st_row, last_row) * row_bytes;
+            const uint32_t r1 = (uint32_t)min(kbase + st_row + 32, last_row) * row_bytes;
+            pf2_load_to_lds(kseg, r0 + st_kcol, dk);
+            pf2_load_to_lds(kseg, r1 + st_kcol, dk + PF2_TILE / 2);
+            pf2_load_to_lds(vseg, r0 + st_vcol, dv);
+            pf2_load_to_lds(vseg, r1 + st_vcol, dv + PF2_TILE / 2);
         }
     };
 
-    // per-lane LDS read offsets
-    const int k_off = j * PF2_KROW + hl * 16;
-    const int v_off = PF2_KBYTES + j * PF2_VROW + hl * 16;
-
-    // S^T = K . Q^T of one 32-key block, relative to the exponent reference: s - m_ref in log2 units
-    auto qk = [&](const char* buf, int kb) __attribute__((always_inline)) {
-        pf_f32x16 s = negm;
+    // per-lane LDS read offsets; the buffer, the 32-key block and the step are immediates on top of them
+    PF_LDS3 char* k_ptr[8];
+    PF_LDS3 char* v_ptr[4];
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            const pf_bf16x8 kf = *(const pf_bf16x8*)(buf + k_off + kb * 32 * PF2_KROW + ks * 32);
-            s = mfma_32x32x16<F16>(kf, qf[ks], s);
+    for (int ks = 0; ks < 8; ++ks) {
+        k_ptr[ks] = lds3 + (j * 256 + (((2 * ks + hl) ^ (j & 15)) << 4));
+        asm volatile("" : "+v"(k_ptr[ks]));          // a value in a register from here on, not an expression to recompute in the loop
+    }
+    {
+        const int i = lane & 15, jhalf = (lane >> 4) & 1;
+        const int kx = 4 * hl + (i >> 2);            // key (within its group of 8) this lane supplies to the transposing read
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+            v_ptr[db] = lds3 + (PF2_VBASE + kx * 256 + (((2 * db + jhalf) ^ (2 * (kx & 3))) << 5) + (i & 3) * 8);
+            asm volatile("" : "+v"(v_ptr[db]));
         }
-        return s;
+    }
+    auto k_frag = [&](int imm, int ks) __attribute__((always_inline)) {
+        return *(const PF_LDS3 pf_bf16x8*)(k_ptr[ks] + imm);
     };
+    auto v_frag = [&](int imm, int st, int db) __attribute__((always_inline)) {
+        PF_LDS3 char* p = v_ptr[db] + imm + st * 16 * 256;
+        const pf_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PF_LDS3 pf_s16x4*)p);                // keys 16 st + 4 hl + 0..3
+        const pf_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((PF_LDS3 pf_s16x4*)(p + 8 * 256));    // ... + 8
+        return __builtin_bit_cast(pf_bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+
     // Mask (diagonal blocks only), row maximum, and the lazy move of the exponent reference: O and l are
     // rescaled only when some row of the wavefront outgrows its reference by 2^PF2_LAZY.  FIRST: the wavefront's first
     // block puts the reference on the row maximum wherever it lies (O and l are still zero: nothing to rescale).
@@ -498,38 +490,44 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
         l_run = add_pair<F16>(pw, l_run);
         return pw;
     };
-    auto v_frag = [&](const char* buf, int kb, int st, int db) __attribute__((always_inline)) {
-        return *(const pf_bf16x8*)(buf + v_off + db * 32 * PF2_VROW + (kb * 4 + st * 2) * 16);
-    };
     // One pipeline step, in issue order (the fences keep the compiler from regrouping it): the 8 MFMAs of the next
-    // block's scores, each followed by one eighth of this block's exponentials; then the 8 MFMAs of P.V.  Operand
-    // reads from LDS are issued well ahead of the MFMA that consumes them.  s_cur and s_nxt are two register blocks that
-    // swap roles from step to step (no copy).
-    //   HAS_NEXT = false: last block of the wavefront, no scores to compute.
-    // Returns the row maximum of s_nxt (this lane's 16 scores), computed in the shadow of the P.V MFMAs.
-    auto step = [&](const pf_f32x16& s_cur, pf_f32x16& s_nxt, const char* kbuf, int kkb, const char* vbuf, int vkb, auto has_next)
-                    __attribute__((always_inline)) -> float {
-        constexpr bool HAS_NEXT = decltype(has_next)::value;
-        // The 16 MFMA operands of a step (8 K fragments, then 8 V fragments) are one stream of LDS reads, each requested
-        // PD MFMAs before the one that consumes it: no burst of reads at the start of a step, a few registers in flight.
+    // block's scores, each followed by one eighth of this block's exponentials; then the 8 MFMAs of P.V, with the maximum
+    // of the next block's scores computed in their shadow.  s_cur and s_nxt are two register blocks that swap roles from
+    // step to step (no copy).  The 16 MFMA operands of a step (8 K fragments, then 8 V fragments) belong to one stream of
+    // LDS reads that runs across steps: each is requested PD MFMAs before the one that consumes it, so the first PD K
+    // fragments of a step were requested by the step before it (pre[], in and out).
+    //   kimm, vimm: byte offsets of this step's K block and V block; nkimm: of the next step's K block
+    //   HAS_NEXT = false: last block of the wavefront, no scores to compute.  FEEDS_NEXT = false: no step follows that wants K.
+    //   SYNC: the iteration's barrier, between the two groups of MFMAs (the score MFMAs drain while the wavefront waits).
+    // Returns the row maximum of s_nxt (this lane's 16 scores).
+    auto step = [&](const pf_f32x16& s_cur, pf_f32x16& s_nxt, pf_bf16x8 (&pre)[PF2_PD], auto kimm_c, auto vimm_c, auto nkimm_c, auto has_next,
+                    auto feeds_next, auto sync_c) __attribute__((always_inline)) -> float {
+        constexpr bool HAS_NEXT = decltype(has_next)::value, FEEDS_NEXT = decltype(feeds_next)::value, SYNC = decltype(sync_c)::value;
+        const int KIMM = kimm_c, VIMM = vimm_c, NKIMM = nkimm_c;   // integral constants in the main loop (instruction immediates), plain ints in the tail
         constexpr int PD = PF2_PD;
-        pf_bf16x8 frag[16];
+        pf_bf16x8 frag[16 + PD];
         uint32_t pw[8];
         auto request = [&](int m) __attribute__((always_inline)) {
             if (m < 8) {
-                if (HAS_NEXT) frag[m] = *(const pf_bf16x8*)(kbuf + k_off + kkb * 32 * PF2_KROW + m * 32);
+                if (HAS_NEXT) frag[m] = k_frag(KIMM, m);
             } else if (m < 16) {
-                frag[m] = v_frag(vbuf, vkb, (m - 8) >> 2, (m - 8) & 3);
+                frag[m] = v_frag(VIMM, (m - 8) >> 2, (m - 8) & 3);
+            } else if (FEEDS_NEXT) {
+                frag[m] = k_frag(NKIMM, m - 16);
             }
         };
 #pragma unroll
-        for (int m = 0; m < PD; ++m) request(m);
-        __builtin_amdgcn_sched_barrier(0);
+        for (int m = 0; m < PD; ++m) frag[m] = pre[m];
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
             request(ks + PD);
             pw[ks] = p_pair(s_cur, ks);
             if (HAS_NEXT) s_nxt = mfma_32x32x16<F16>(frag[ks], qf[ks], ks == 0 ? negm : s_nxt);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (SYNC) {   // behind the barrier the next tile is visible: every thread has waited for its own four loads of it
+            asm volatile("s_waitcnt vmcnt(4)" ::: "memory");   // (the four of the tile after it may still be in flight)
+            __syncthreads();
             __builtin_amdgcn_sched_barrier(0);
         }
         pf_bf16x8 pfrag[2];
@@ -539,7 +537,8 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
             pfrag[st] = __builtin_bit_cast(pf_bf16x8, pq);
         }
         // the maximum of the next block's scores as a tree of three-input maxima, one or two per P.V MFMA from the third
-        // on (the last score MFMA has landed by then): after the step only the comparison with the reference is left
+        // on (the last score MFMA has landed by then); the empty volatile statements fix where each is computed: between
+        // these two MFMAs, not after the last one
         float mt[7];
         auto max3 = [](float x, float y, float z) __attribute__((always_inline)) { return __builtin_fmaxf(__builtin_fmaxf(x, y), z); };
 #pragma unroll
@@ -547,52 +546,73 @@ __global__ __launch_bounds__(PF2_THREADS) void prefill_attn_kernel(PrefillArgs a
             request(8 + i + PD);
             o[i & 3] = mfma_32x32x16<F16>(frag[8 + i], pfrag[i >> 2], o[i & 3]);
             if (HAS_NEXT) {
-                if (i >= 2 && i <= 6) mt[i - 2] = max3(s_nxt[3 * (i - 2)], s_nxt[3 * (i - 2) + 1], s_nxt[3 * (i - 2) + 2]);
-                if (i == 6) mt[5] = max3(mt[0], mt[1], s_nxt[15]);
-                if (i == 7) mt[6] = max3(mt[2], mt[3], mt[4]);
+                if (i >= 2 && i <= 6) { mt[i - 2] = max3(s_nxt[3 * (i - 2)], s_nxt[3 * (i - 2) + 1], s_nxt[3 * (i - 2) + 2]); asm volatile("" : "+v"(mt[i - 2])); }
+                if (i == 6) { mt[5] = max3(mt[0], mt[1], s_nxt[15]); asm volatile("" : "+v"(mt[5])); }
+                if (i == 7) { mt[6] = max3(mt[2], mt[3], mt[4]); asm volatile("" : "+v"(mt[6])); }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        return HAS_NEXT ? __builtin_fmaxf(mt[5], mt[6]) : 0.0f;
+        if (FEEDS_NEXT) {
+#pragma unroll
+            for (int m = 0; m < PD; ++m) pre[m] = frag[16 + m];
+        }
+        float mx = HAS_NEXT ? __builtin_fmaxf(mt[5], mt[6]) : 0.0f;
+        // both values are wanted here, at the end of the step: without this the compiler moves the maxima and the row-sum
+        // additions behind the branch that follows, out of the shadow of the MFMAs
+        asm volatile("" : "+v"(mx), "+v"(l_run));
+        return mx;
     };
 
     // Pipeline over 32-key blocks: while the exponentials of block b run on the VALU, the MFMA unit computes the scores
-    // of block b + 1 and then P.V of block b.  Tiles (two blocks) rotate through three LDS buffers: tile t + 1 is
-    // written at the top of iteration t into the buffer tile t - 2 used (every wavefront left it before the barrier of
-    // iteration t - 1) and becomes visible at the barrier in the middle of iteration t, in time for the scores of its
-    // first block.
-    // Every wavefront walks all blocks of the workgroup's tiles: the blocks that lie wholly above a wavefront's diagonal
-    // (at most two of up to several hundred, the workgroup spans BT query times) are masked like the diagonal ones
-    // and contribute zeros, which keeps the loop free of per-wavefront branches.
+    // of block b + 1 and then P.V of block b.  Every wavefront walks all blocks of the workgroup's tiles: the blocks that
+    // lie wholly above a wavefront's diagonal (at most two of up to several hundred, the workgroup spans BT query times)
+    // are masked like the diagonal ones and contribute zeros, which keeps the loop free of per-wavefront branches.
     const int ntiles = (k_end + PF2_BN - 1) / PF2_BN;
     if (ntiles > 0) {
         pf_f32x16 s_a, s_b;   // scores of the current and of the next block, roles swapping every step
-        fetch(0);
-        publish(pf2_lds);
-        fetch(PF2_BN);
+        pf_bf16x8 pre[PF2_PD];
+        request_tile(0, 0);
+        request_tile(1, 1);
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         __syncthreads();
-        s_a = qk(pf2_lds, 0);
+        {
+            s_a = negm;
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) s_a = mfma_32x32x16<F16>(k_frag(0, ks), qf[ks], s_a);
+#pragma unroll
+            for (int m = 0; m < PF2_PD; ++m) pre[m] = k_frag(PF2_TILE / 2, m);
+        }
         prepare(s_a, 0, 0.0f, std::true_type{});
-        int i0 = 0, i1 = 1;   // buffer index of tile t and of tile t + 1
-        for (int t = 0; t + 1 < ntiles; ++t) {
-            const char* b0 = pf2_lds + i0 * PF2_BUF;
-            char* b1 = pf2_lds + i1 * PF2_BUF;
-            publish(b1);
-            fetch((t + 2) * PF2_BN);          // unconditional (rows clamped)
-            const float ma = step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
+        // Iteration t (tile t in the buffer at off0, tile t + 1 at off1): blocks 2t and 2t + 1, and the scores of block 2t + 2.
+        // Tile t + 2 is requested first, into the buffer tile t - 2 used (every wavefront left it before the barrier of
+        // iteration t - 1).  The one barrier of an iteration sits inside its first step, between the score MFMAs and the
+        // P.V MFMAs: behind it tile t + 1 is visible, in time for the K fragments that the end of that step requests.
+        auto iteration = [&](int t, int b2, auto off0, auto off1) __attribute__((always_inline)) {
+            constexpr std::integral_constant<int, PF2_TILE / 2> half{};
+            request_tile(t + 2, b2);          // unconditional (rows clamped): the count of loads in flight stays fixed
+            const float ma = step(s_a, s_b, pre, off0 + half, off0, off1, std::true_type{}, std::true_type{}, std::true_type{});
             prepare(s_b, 2 * t + 1, ma, std::false_type{});
-            __syncthreads();
-            const float mb = step(s_b, s_a, b1, 0, b0, 1, std::true_type{});
+            const float mb = step(s_b, s_a, pre, off1, off0 + half, off1 + half, std::true_type{}, std::true_type{}, std::false_type{});
             prepare(s_a, 2 * t + 2, mb, std::false_type{});
-            i0 = i1;
-            i1 = i1 == 2 ? 0 : i1 + 1;
+        };
+        using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, PF2_TILE>;
+        using I2 = std::integral_constant<int, 2 * PF2_TILE>; using I3 = std::integral_constant<int, 3 * PF2_TILE>;
+        int t = 0;
+        for (; t + 4 < ntiles; t += 4) {      // four tiles per turn: buffer offsets are immediates of the LDS reads
+            iteration(t, 2, I0{}, I1{});
+            iteration(t + 1, 3, I1{}, I2{});
+            iteration(t + 2, 0, I2{}, I3{});
+            iteration(t + 3, 1, I3{}, I0{});
         }
+        for (; t + 1 < ntiles; ++t)           // up to three more, offsets computed
+            iteration(t, (t + 2) & 3, (t & 3) * PF2_TILE, ((t + 1) & 3) * PF2_TILE);
         {   // the last tile: its second block has no successor
-            const char* b0 = pf2_lds + i0 * PF2_BUF;
-            const float ma = step(s_a, s_b, b0, 1, b0, 0, std::true_type{});
-            prepare(s_b, 2 * ntiles - 1, ma, std::false_type{});
-            step(s_b, s_a, b0, 0, b0, 1, std::false_type{});
+            const int off = (t & 3) * PF2_TILE;
+            const float ma = step(s_a, s_b, pre, off + PF2_TILE / 2, off, 0, std::true_type{}, std::false_type{}, std::false_type{});
+            prepare(s_b, 2 * t + 1, ma, std::false_type{});
+            step(s_b, s_a, pre, 0, off + PF2_TILE / 2, 0, std::false_type{}, std::false_type{}, std::false_type{});
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the look-ahead tiles were requested too: nothing may land after the wavefront has gone
     }
 
     // the two halves of a query hold disjoint keys: add their sums, then normalise and store
