@@ -371,6 +371,8 @@ def test_uncompressed_long_context_decode_and_chunk():
     ("config3", 64, 8, 4, 4096, 128, 3.0, 1.5),     # 512 segments: one workgroup per segment, the append rides in the attention launch
     ("config2", 16, 8, 2, 2048, 128, 3.0, 1.0),     # 128 segments: fused piece list, two pieces per segment merged in the launch
     ("config5", 8, 8, 5, 8192, 512, 2.0, 2.0),      # 64 segments: fused grid launch (4 splits) + merge kernel, which advances the lengths
+    ("group8", 32, 8, 8, 4096, 128, 3.0, 1.5),      # Qwen3-32B's group width (64 query heads on 8 KV heads): q read from LDS, 256 segments
+    ("group8_split", 4, 8, 8, 4096, 128, 3.0, 1.5), # the same in pieces: 32 segments, fused grid launch + merge kernel
 ])
 def test_fused_decode_step_at_full_shape_across_an_eviction(name, B, H, G, M, buf, mu, sigma):
     """The launches the benchmark times, at their own shapes: ``fuse_decode_append`` on, one layer, four decode steps that

@@ -37,7 +37,7 @@ def _fp32(q, k, v, lens, G, segs):
     return torch.stack(outs)
 
 
-@pytest.mark.parametrize("G,D,order", [(4, 128, "desc"), (1, 128, "shuffled"), (5, 128, "shuffled"), (2, 64, "desc"), (8, 96, "shuffled")])
+@pytest.mark.parametrize("G,D,order", [(4, 128, "desc"), (1, 128, "shuffled"), (5, 128, "shuffled"), (2, 64, "desc"), (8, 96, "shuffled"), (7, 128, "desc"), (8, 128, "shuffled")])
 def test_piece_list_launch_matches_fp32_and_the_grid_launch(G, D, order):
     from trimkv_amd import _lib as L
     lib = L.load()

@@ -53,6 +53,10 @@ struct AttnCfg {
     static constexpr int TILE_ROWS = NJ * 4;
     static constexpr int NT = AT_BLOCK_ROWS / TILE_ROWS;       // tiles per block
     static constexpr int PSTRIDE = NV <= 8 ? 8 : 16;           // bf16 slots per (tile, row group) in LDS
+    // Eight query heads: q (32 registers per lane) would push the streaming loop over its 256 registers, and a loop that
+    // spills waits for its own prefetches (scratch traffic counts as loads).  q then lives in LDS, one copy per wavefront,
+    // and a score step reads the head it is working on.
+    static constexpr bool Q_LDS = G >= 8;
 #ifndef TRIMKV_AT_RING
     static constexpr int RING = (NJ >= 4 || G >= 6) ? 4 : 8;   // register tile buffers: RING-1 tiles in flight per wavefront
 #else
@@ -194,6 +198,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
     __shared__ float so[AT_WAVES][G][AT_D];
     __shared__ float sm[AT_WAVES][8];
     __shared__ float sl[AT_WAVES][8];
+    __shared__ uint4 sq[C::Q_LDS ? AT_WAVES : 1][C::Q_LDS ? G : 1][16];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int c = lane & 15, r = lane >> 4;
@@ -291,15 +296,24 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
             float part[16];
 #pragma unroll
             for (int x = 0; x < 16; ++x) part[x] = 0.0f;
-#pragma unroll
-            for (int j = 0; j < NJ; ++j) {
+            auto dot_row = [&](const uint4& krow, const uint4& qg) __attribute__((always_inline)) {
+                float acc = dot2_kv<F16>(krow.x, qg.x, 0.0f);
+                acc = dot2_kv<F16>(krow.y, qg.y, acc);
+                acc = dot2_kv<F16>(krow.z, qg.z, acc);
+                return dot2_kv<F16>(krow.w, qg.w, acc);
+            };
+            if constexpr (C::Q_LDS) {   // head by head, so that one head's q is live at a time
 #pragma unroll
                 for (int g = 0; g < G; ++g) {
-                    float acc = dot2_kv<F16>(kt[j].x, qv[g].x, 0.0f);
-                    acc = dot2_kv<F16>(kt[j].y, qv[g].y, acc);
-                    acc = dot2_kv<F16>(kt[j].z, qv[g].z, acc);
-                    acc = dot2_kv<F16>(kt[j].w, qv[g].w, acc);
-                    part[j * G + g] = acc;
+                    const uint4 qg = sq[w][g][c];
+#pragma unroll
+                    for (int j = 0; j < NJ; ++j) part[j * G + g] = dot_row(kt[j], qg);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+                    for (int g = 0; g < G; ++g) part[j * G + g] = dot_row(kt[j], qv[g]);
                 }
             }
             const float val = reduce16_transposed(part, c);
@@ -405,6 +419,11 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         for (int sl = 0; sl < PD; ++sl) load_tile(kp, knew, w0 + sl * TILE_ROWS, ring[sl % RING]);
 #pragma unroll
         for (int g = 0; g < G; ++g) asm volatile("" : "+v"(qv[g].x), "+v"(qv[g].y), "+v"(qv[g].z), "+v"(qv[g].w));
+        if constexpr (C::Q_LDS) {   // every lane holds column c of all heads: row group r parks heads r, r + 4, ... for its wavefront
+#pragma unroll
+            for (int g = 0; g < G; ++g)
+                if ((g & 3) == r) sq[w][g][c] = qv[g];
+        }
         if (APPEND_EARLY && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
             const int64_t dst = row0 + new_row;
             if (r == 0 && c < ROW16) {
