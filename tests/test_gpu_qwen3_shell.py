@@ -164,7 +164,26 @@ def test_shell_generate_chunked_prompt_and_ragged_cache():
     assert dense.shape == (2, 172) and torch.equal(dense[:, :160], ids)
     agree = lambda a, b: (a[:, 160:] == b[:, 160:]).float().mean().item()
     assert agree(dense, ragged) == 1.0                                 # same kernels underneath, same keys
-    assert agree(dense, whole) >= 0.75                                 # chunked vs one-shot prompt: bf16 summation order only
+    # Chunked against one-shot prompt: only the bf16 summation order differs.  Greedy tokens of a random model are near-ties
+    # and part ways for good after the first flip, so the comparison is on the logits, with the same tokens fed to both.
+    model.config._attn_implementation = "trimkv_hip"
+
+    def logits_along(prefill_chunk):
+        cache, chunk, rows = TrimKVCache(), prefill_chunk or ids.shape[1], []
+        for s0 in range(0, ids.shape[1], chunk):
+            out = model(ids[:, s0:s0 + chunk], past_key_values=cache, logits_to_keep=1)
+        rows.append(out.logits[:, -1].float())
+        for t in range(160, 171):
+            rows.append(model(dense[:, t:t + 1], past_key_values=cache, logits_to_keep=1).logits[:, -1].float())
+        return torch.stack(rows, dim=1)
+    la, lw = logits_along(64), logits_along(0)
+    assert torch.equal(la.argmax(-1), dense[:, 160:])                  # the teacher-forced pass reproduces the generation
+    err, scale = (la - lw).abs().max().item(), lw.abs().max().item()
+    print(f"chunked vs one-shot prompt: max logit difference {err:.4f} on a scale of {scale:.3f}; first token agreement {agree(dense, whole):.2f}", flush=True)
+    assert err <= 0.05 * scale, (err, scale)
+    margin = (lw.topk(2, dim=-1).values[..., 0] - lw.topk(2, dim=-1).values[..., 1])
+    clear = margin > 2 * err                                           # where the one-shot pass has a clear winner, both passes name it
+    assert torch.equal(la.argmax(-1)[clear], lw.argmax(-1)[clear])
 
     cfg2 = _tiny_config(memory_size=32, buffer_size=16)
     model2 = TrimKVQwen3ForCausalLM(cfg2).to(torch.bfloat16).to(DEV).eval()

@@ -29,14 +29,13 @@ from .. import _lib
 
 _WS: Dict[Tuple[str, int], torch.Tensor] = {}
 _MAX_GROUP = 8   # query heads per KV head that one kernel launch handles
-# Group sizes that use the fused (append + attend) piece-list kernel.  Ragged caches, whose alternative is the append as a
-# launch of its own in front of the unfused piece-list kernel: 43.0 against 45.1 us per layer at a group of 5, 44.0 against
-# 46.0 at 6, 47.3 against 48.3 at 7, 51.1 against 50.8 at 8 (256 lognormal segments; at 8 the kernels keep q in LDS, which
-# ended the register spills that had cost both forms 15-20 %).  Dense cache, whose alternative is the fused grid launch +
-# merge kernel: 50.2 us in one launch against 46.8 + 5.2 us in two at a group of 5 (64 segments of 8448 rows in 4 pieces);
-# 53.9 against 52.5-53.6 at 7 and 8.
-_FUSED_PIECES_GROUPS = (1, 2, 3, 4, 5, 6, 7)
-_DENSE_PIECES_GROUPS = (1, 2, 3, 4, 5, 6)
+# Group sizes that use the fused (append + attend) piece-list kernel, and those for which the dense cache merges its equal
+# pieces inside the launch: all of them.  (Before the wide groups ran on MFMA the dot-product kernel spilled registers
+# from six or seven query heads per KV head on, and these lists stopped there.)  Ragged cache, 256 lognormal segments, per
+# layer: 42.2 us fused against 44.4 us with the append as a launch of its own at a group of 8.  Dense cache, 64 segments of
+# 8448 rows in 4 pieces: 48.2-48.8 us in one launch against 47.7-48.4 us + a 5 us merge launch.
+_FUSED_PIECES_GROUPS = (1, 2, 3, 4, 5, 6, 7, 8)
+_DENSE_PIECES_GROUPS = (1, 2, 3, 4, 5, 6, 7, 8)
 _WARNED = set()
 dense_workgroups, dense_min_rows = 256, 512   # piece-list launches of the dense cache: workgroups wanted, fewest rows apiece
 dense_chunk = 0   # split-K rows per workgroup for the dense cache's decode attention; 0 = the library's choice (tuning knob)

@@ -178,6 +178,298 @@ __device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new
     return n;
 }
 
+// The end of attend_rows, after every wavefront has left its accumulator (so), maximum (sm) and sum (sl) in LDS and the
+// workgroup has met at a barrier: the four wavefronts are merged, and the result is normalised and written (direct) or
+// left as a partial in slot `slot_base` of the workspace.
+template <int G, int ROW16, bool F16, bool APPEND, bool COHERENT>
+__device__ __forceinline__ void finish_workgroup(const AttnArgs& a, int seg, bool direct, int64_t slot_base, int new_row,
+                                                 const float (*so)[G][AT_D], const float (*sm)[8], const float (*sl)[8]) {
+    constexpr int D_REAL = ROW16 * 8;
+    const int tid = threadIdx.x;
+    if (APPEND && direct && tid == 0 && new_row >= 0) {
+        // one workgroup per segment: every wavefront read the old length before the barrier above, nobody else reads it
+        a.ap.seg_len[seg] = new_row + 1;
+        if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;     // cu[i] += i per appended token (cache_utils.py:678-680)
+    }
+    for (int i = tid; i < G * AT_D; i += AT_THREADS) {
+        const int g = i / AT_D, d = i - g * AT_D;
+        float mx = AT_NEG;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) mx = fmaxf(mx, sm[ww][g]);
+        float acc = 0.0f, lsum = 0.0f;
+#pragma unroll
+        for (int ww = 0; ww < AT_WAVES; ++ww) {
+            const float f = __builtin_amdgcn_exp2f(sm[ww][g] - mx);
+            acc += f * so[ww][g][d];
+            lsum += f * sl[ww][g];
+        }
+        if (direct) {
+            const float y = lsum > 0.0f ? acc / lsum : 0.0f;
+            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = to_kv_bits<F16>(y);
+        } else {
+            const int64_t slot = slot_base * G + g;
+            if (COHERENT) {
+                store_shared_partial(&a.ws_o[slot * AT_D + d], acc);
+                if (d == 0) { store_shared_partial(&a.ws_ml[slot * 2], mx); store_shared_partial(&a.ws_ml[slot * 2 + 1], lsum); }
+            } else {
+                a.ws_o[slot * AT_D + d] = acc;
+                if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// The same attention for rows of 128 features, built on LDS-direct loads and MFMA.
+//
+// The stream: a wavefront still reads whole rows, 1 KiB (4 rows) per load instruction, but the loads write LDS themselves
+// (global_load_lds_dwordx4, non-temporal) instead of registers: a ring of 16 KiB per wavefront holds the K rows and the V
+// rows of one 32-row step, and 8-16 KiB of it are in flight at any time.  On this part that form streams faster than
+// register loads (measured on 512 workgroups: 7.1 against 6.9 TB/s at 528 MB per launch, 7.3 against 6.4 at 240 MB,
+// 6.3 against 5.5 at 96 MB) and costs no registers.  The compiler does not see these loads (inline assembly), so every
+// wait for them is written out: s_waitcnt vmcnt(8) = "all but the newest eight loads have landed".
+//
+// The arithmetic: v_mfma_f32_16x16x32 with the query heads (padded to 16) as the column index.
+//   S^T[key][head] = K . q^T     A = 16 K rows from LDS (lane l: key l % 16, 8 features of group l / 16 per k-step),
+//                                B = q held in registers; a lane ends up with 4 keys (4 (l / 16) + v) of head l % 16
+//   O^T[d][head]  += V^T . P^T   A = V^T read with the transposing LDS read (8 keys at one feature per lane: the same 4 + 4
+//                                keys of two 16-row tiles that the lane holds probabilities for), B = P as packed pairs
+// so P never crosses lanes and the softmax is per lane (one maximum exchange across the four lane groups per step).
+// Which 16-byte piece of a row a lane's load fetches is free (the destination is lane-linear), and that is where the
+// bank swizzle comes from: K piece c of row r (within its tile) sits at position c ^ r, V 32-byte pair p at p ^ (r & 7).
+// ---------------------------------------------------------------------------------------------------------------------
+typedef __bf16 at_bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 at_f16x8 __attribute__((ext_vector_type(8)));
+typedef float at_f32x4 __attribute__((ext_vector_type(4)));
+typedef short at_s16x4 __attribute__((ext_vector_type(4)));
+#define AT_LDS3 __attribute__((address_space(3)))
+
+#ifndef TRIMKV_AT_MFMA
+#define TRIMKV_AT_MFMA 1
+#endif
+constexpr int ATM_STEP = 32;             // rows per step: two 16-row tiles of K and of V
+constexpr int ATM_TILE_BYTES = 4096;     // 16 rows x 256 B
+constexpr int ATM_RING_BYTES = 16384;    // per wavefront: K tiles 0, 1, then V tiles 0, 1
+
+template <bool F16>
+__device__ __forceinline__ at_f32x4 atm_mfma(at_bf16x8 a, at_bf16x8 b, at_f32x4 c) {
+    if constexpr (F16) return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(at_f16x8, a), __builtin_bit_cast(at_f16x8, b), c, 0, 0, 0);
+    else return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+// One LDS-direct, non-temporal load of 16 bytes per lane: lane l's bytes land at LDS address lds_addr + 16 l.
+__device__ __forceinline__ void atm_load_to_lds(const char* src, uint32_t lds_addr) {
+    uint32_t saved;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt\n\ts_mov_b32 m0, %0"
+                 : "=&s"(saved) : "v"(src), "s"(lds_addr) : "memory");
+}
+template <bool F16>
+__device__ __forceinline__ uint32_t atm_pack(float lo, float hi) {
+    return (uint32_t)to_kv_bits<F16>(lo) | ((uint32_t)to_kv_bits<F16>(hi) << 16);
+}
+
+template <int G, bool F16, bool APPEND, bool COHERENT, bool GATED>
+__device__ __forceinline__ void attend_rows_mfma(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base, int new_row) {
+    // the rings; once every wavefront has left its loop, the merge buffers of finish_workgroup live in the same memory
+    __shared__ __attribute__((aligned(1024))) char ring_all[AT_WAVES * ATM_RING_BYTES];
+    static_assert(AT_WAVES * G * AT_D * 4 + 2 * AT_WAVES * 8 * 4 <= AT_WAVES * ATM_RING_BYTES, "merge buffers must fit into the rings");
+    float (*so)[G][AT_D] = (float (*)[G][AT_D])ring_all;
+    float (*sm)[8] = (float (*)[8])(ring_all + AT_WAVES * G * AT_D * 4);
+    float (*sl)[8] = sm + AT_WAVES;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int h = lane & 15, gq = lane >> 4;       // MFMA column (query head) / row index inside a tile, and lane group
+    const int pw = (t1 - t0 + AT_WAVES - 1) / AT_WAVES;
+    const int w0 = t0 + w * pw, w1 = min(t1, w0 + pw);
+    const int64_t row0 = a.seg_start ? (int64_t)a.seg_start[seg] : (int64_t)seg * a.cap;
+    const char* kseg = (const char*)a.k + row0 * 256;
+    const char* vseg = (const char*)a.v + row0 * 256;
+
+    // APPEND: this step's token comes from the caller's tensors (row pointers, then the loads)
+    const char* knew = nullptr;
+    const char* vnew = nullptr;
+    int ap_b = 0, ap_h = 0;
+    if (APPEND) {
+        ap_b = seg / a.ap.kv_heads; ap_h = seg - ap_b * a.ap.kv_heads;
+        const int64_t off = (int64_t)ap_b * a.ap.kv_sb + (int64_t)ap_h * a.ap.kv_sh;
+        knew = a.ap.k_new + off;
+        vnew = a.ap.v_new + off;
+    }
+    // q as the B operand of the score product: lane (head h, group gq) holds features 32 s + 8 gq .. + 7 of k-step s.
+    // These loads (and the new row's) are issued ahead of the stream's first requests: loads return in order, so the
+    // first use of q waits for nothing that the first step would not wait for anyway.
+    at_bf16x8 qb[4];
+    {
+        const uint4* qrow = a.q + ((int64_t)seg * G + min(h, G - 1)) * 16;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            uint4 t = qrow[4 * s + gq];
+            if (h >= G) t = make_uint4(0u, 0u, 0u, 0u);   // padding columns
+            qb[s] = __builtin_bit_cast(at_bf16x8, t);
+        }
+    }
+    uint4 kn = make_uint4(0u, 0u, 0u, 0u), vn = kn;
+    float lbn = 0.0f, gate_bias = 0.0f;
+    int64_t pn = 0;
+    if (APPEND) {   // fetched by every wavefront (unconditional loads), stored by the wavefront that owns the row
+        kn = *(const uint4*)(knew + (h << 4));
+        vn = *(const uint4*)(vnew + (h << 4));
+        if (GATED) {
+            lbn = a.ap.gate_part[((int64_t)min(lane, a.ap.gate_nslice - 1) * (a.nseg / a.ap.kv_heads) + ap_b) * a.ap.kv_heads + ap_h];
+            gate_bias = a.ap.gate_bias[ap_h];
+        } else {
+            lbn = load_as_f32(a.ap.lb_new, (int64_t)ap_b * a.ap.lb_sb + (int64_t)ap_h * a.ap.lb_sh, a.ap.lb_dtype);
+        }
+        pn = a.ap.pos_new[(int64_t)ap_b * a.ap.pos_sb + (int64_t)ap_h * a.ap.pos_sh];
+    }
+    at_f32x4 o[8];     // O^T: o[db][v] = feature 16 db + 4 gq + v of head h
+#pragma unroll
+    for (int db = 0; db < 8; ++db) o[db] = at_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = AT_NEG, l_run = 0.0f;
+
+    if (w0 < w1) {
+        AT_LDS3 char* const ring = (AT_LDS3 char*)ring_all + w * ATM_RING_BYTES;
+        const uint32_t ring_addr = (uint32_t)(uintptr_t)ring;
+        // per-lane constants of the loads: instruction j of a tile covers its rows 4j .. 4j + 3, lane (gq, h) fetches of
+        // row 4j + gq the piece whose swizzled position is h
+        uint32_t kcol[4], vcol[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int rt = 4 * j + gq;
+            kcol[j] = (uint32_t)(h ^ rt) << 4;
+            vcol[j] = (uint32_t)(((((h >> 1) ^ (rt & 7)) << 1) | (h & 1)) << 4);
+        }
+        const int last = w1 - 1;
+        // the 4 loads of one 16-row tile: K (or V) rows sb + 16 t .. + 15 into tile slot t of the K (or V) half of the ring
+        auto request = [&](int sb, int t, auto is_v_c) __attribute__((always_inline)) {
+            constexpr bool IS_V = decltype(is_v_c)::value;
+            const char* base = IS_V ? vseg : kseg;
+            const char* fresh = IS_V ? vnew : knew;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = min(sb + 16 * t + 4 * j + gq, last);   // rows past the end re-read the last one (weight 0)
+                const uint32_t col = IS_V ? vcol[j] : kcol[j];
+                const char* src = base + ((int64_t)row << 8) + col;
+                if (APPEND) src = row == new_row ? fresh + col : src;   // this step's token comes from the caller's tensor
+                atm_load_to_lds(src, ring_addr + (IS_V ? 2 * ATM_TILE_BYTES : 0) + t * ATM_TILE_BYTES + j * 1024);
+            }
+        };
+        // per-lane LDS read offsets
+        AT_LDS3 char* kfa[4];
+        AT_LDS3 char* vfa[8];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) kfa[s] = ring + h * 256 + (((4 * s + gq) ^ h) << 4);
+        {
+            const int row = 4 * gq + (h >> 2);           // the key this lane supplies to the transposing read
+#pragma unroll
+            for (int db = 0; db < 8; ++db) vfa[db] = ring + 2 * ATM_TILE_BYTES + row * 256 + ((db ^ (row & 7)) << 5) + (h & 3) * 8;
+        }
+
+        // The stream of a wavefront: per 32-row step the tiles K0 K1 V0 V1, four loads each, into their own quarter of the
+        // ring.  Sixteen loads are in flight at the top of a step; a tile is awaited ("all but the newest twelve loads have
+        // landed"), read into registers, and its quarter is refilled with the same tile of the next step at once, so 12-16
+        // KiB stay in flight.  The last step refills nothing and its waits count down instead.
+        request(w0, 0, std::false_type{});
+        request(w0, 1, std::false_type{});
+        request(w0, 0, std::true_type{});
+        request(w0, 1, std::true_type{});
+        if (APPEND && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
+            const int64_t dst = row0 + new_row;
+            if (gq == 0) {
+                ((uint4*)a.k)[dst * 16 + h] = kn;
+                ((uint4*)a.v)[dst * 16 + h] = vn;
+            }
+            if (GATED) lbn = finish_gate(lane < a.ap.gate_nslice ? lbn : 0.0f, gate_bias, a.ap.lb_dtype);
+            if (lane == 0) {
+                store_from_f32(a.ap.lb_slab, dst, a.ap.lb_dtype, lbn);
+                a.ap.pos_slab[dst] = pn;
+            }
+        }
+#pragma unroll 1
+        for (int sb = w0; sb < w1; sb += ATM_STEP) {
+            const bool more = sb + ATM_STEP < w1;   // wave-uniform
+            // tile `left` tiles before the end of the step's stream has landed
+            auto await = [&](auto left_c) __attribute__((always_inline)) {
+                constexpr int LEFT = decltype(left_c)::value;
+                if (more) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+                else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(4 * LEFT) : "memory");
+            };
+            // the tile just read is in registers: its quarter of the ring takes the same tile of the next step
+            auto refill = [&](int t, auto is_v_c) __attribute__((always_inline)) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (more) request(sb + ATM_STEP, t, is_v_c);
+            };
+            at_bf16x8 kf[2][4];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                if (t == 0) await(std::integral_constant<int, 3>{}); else await(std::integral_constant<int, 2>{});
+#pragma unroll
+                for (int s = 0; s < 4; ++s) kf[t][s] = *(const AT_LDS3 at_bf16x8*)(kfa[s] + t * ATM_TILE_BYTES);
+                refill(t, std::false_type{});
+            }
+            at_f32x4 sc[2];
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                sc[t] = at_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int s = 0; s < 4; ++s) sc[t] = atm_mfma<F16>(kf[t][s], qb[s], sc[t]);
+            }
+            // ---- softmax of the step: this lane holds keys sb + 16 t + 4 gq + v of head h ----
+            float x[8];
+            float mx = AT_NEG;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int row = sb + 16 * t + 4 * gq + v;
+                    x[4 * t + v] = row < w1 ? sc[t][v] * a.scale_log2 : AT_NEG;
+                    mx = fmaxf(mx, x[4 * t + v]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            m_run = m_new;
+            float p[8], psum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { p[i] = __builtin_amdgcn_exp2f(x[i] - m_new); psum += p[i]; }
+            l_run = l_run * alpha + psum;
+#pragma unroll
+            for (int db = 0; db < 8; ++db)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) o[db][v] *= alpha;
+            const at_u32x4 pq = {atm_pack<F16>(p[0], p[1]), atm_pack<F16>(p[2], p[3]), atm_pack<F16>(p[4], p[5]), atm_pack<F16>(p[6], p[7])};
+            const at_bf16x8 pfrag = __builtin_bit_cast(at_bf16x8, pq);
+            // ---- V^T operands: keys 4 gq + 0..3 of tile 0 and of tile 1 at one feature per lane ----
+            at_s16x4 vlo[8], vhi[8];
+            await(std::integral_constant<int, 1>{});
+#pragma unroll
+            for (int db = 0; db < 8; ++db) vlo[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AT_LDS3 at_s16x4*)vfa[db]);
+            refill(0, std::true_type{});
+            await(std::integral_constant<int, 0>{});
+#pragma unroll
+            for (int db = 0; db < 8; ++db) vhi[db] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((AT_LDS3 at_s16x4*)(vfa[db] + ATM_TILE_BYTES));
+            refill(1, std::true_type{});
+#pragma unroll
+            for (int db = 0; db < 8; ++db)
+                o[db] = atm_mfma<F16>(__builtin_bit_cast(at_bf16x8, __builtin_shufflevector(vlo[db], vhi[db], 0, 1, 2, 3, 4, 5, 6, 7)), pfrag, o[db]);
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // (the last step has waited for everything already)
+    }
+
+    // the four lane groups of a head hold disjoint keys: add their sums
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+    __syncthreads();   // every wavefront has left its ring: the memory becomes the merge buffers
+    if (h < G) {
+#pragma unroll
+        for (int db = 0; db < 8; ++db) *(at_f32x4*)&so[w][h][16 * db + 4 * gq] = o[db];
+        if (gq == 0) { sm[w][h] = m_run; sl[w][h] = l_run; }
+    }
+    __syncthreads();
+    finish_workgroup<G, 16, F16, APPEND, COHERENT>(a, seg, direct, slot_base, new_row, so, sm, sl);
+}
+
 // Attention of the G query heads of segment `seg` over its rows [t0, t1): the body shared by both kernels.
 // `direct`: normalise and write the output; otherwise the unnormalised accumulator and (max, sum) go to partial
 // slot `slot` of the workspace.  All 256 threads of the workgroup must call it together (it uses barriers).
@@ -189,7 +481,13 @@ __device__ __forceinline__ int segment_rows(const AttnArgs& a, int seg, int* new
 // GATED (with APPEND): log beta of the new row comes from the retention gate's partial sums (finish_gate), not from lb_new.
 template <int G, int ROW16, bool F16, bool APPEND, bool COHERENT = false, bool GATED = false>
 __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, int t1, bool direct, int64_t slot_base, int new_row) {
-    constexpr int D_REAL = ROW16 * 8;
+    // Rows of 128 features and five or more query heads per KV head: the MFMA form.  (Up to four heads the dot-product form
+    // below streams as fast or faster in the decode step -- 128 segments in two pieces: 29.4 against 30.5 us per launch --
+    // and from five on it loses to its own arithmetic: 52.2 against 51.4 us at five heads, 58.6 against 48.6 at eight.)
+    if constexpr (ROW16 == 16 && G >= 5 && TRIMKV_AT_MFMA) {
+        attend_rows_mfma<G, F16, APPEND, COHERENT, GATED>(a, seg, t0, t1, direct, slot_base, new_row);
+        return;
+    }
     using C = AttnCfg<G>;
     constexpr int NJ = C::NJ, NV = C::NV, NT = C::NT, TILE_ROWS = C::TILE_ROWS, PS = C::PSTRIDE;
 
@@ -499,37 +797,7 @@ __device__ __forceinline__ void attend_rows(const AttnArgs& a, int seg, int t0, 
         for (int g = 0; g < G; ++g) sm[w][g] = m_run[g];
     }
     __syncthreads();
-    if (APPEND && direct && tid == 0 && new_row >= 0) {
-        // one workgroup per segment: every wavefront read the old length before the barrier above, nobody else reads it
-        a.ap.seg_len[seg] = new_row + 1;
-        if (a.ap.cu) a.ap.cu[seg + 1] += seg + 1;     // cu[i] += i per appended token (cache_utils.py:678-680)
-    }
-    for (int i = tid; i < G * AT_D; i += AT_THREADS) {
-        const int g = i / AT_D, d = i - g * AT_D;
-        float mx = AT_NEG;
-#pragma unroll
-        for (int ww = 0; ww < AT_WAVES; ++ww) mx = fmaxf(mx, sm[ww][g]);
-        float acc = 0.0f, lsum = 0.0f;
-#pragma unroll
-        for (int ww = 0; ww < AT_WAVES; ++ww) {
-            const float f = __builtin_amdgcn_exp2f(sm[ww][g] - mx);
-            acc += f * so[ww][g][d];
-            lsum += f * sl[ww][g];
-        }
-        if (direct) {
-            const float y = lsum > 0.0f ? acc / lsum : 0.0f;
-            if (d < D_REAL) ((uint16_t*)a.out)[((int64_t)seg * G + g) * D_REAL + d] = to_kv_bits<F16>(y);
-        } else {
-            const int64_t slot = slot_base * G + g;
-            if (COHERENT) {
-                store_shared_partial(&a.ws_o[slot * AT_D + d], acc);
-                if (d == 0) { store_shared_partial(&a.ws_ml[slot * 2], mx); store_shared_partial(&a.ws_ml[slot * 2 + 1], lsum); }
-            } else {
-                a.ws_o[slot * AT_D + d] = acc;
-                if (d == 0) { a.ws_ml[slot * 2] = mx; a.ws_ml[slot * 2 + 1] = lsum; }
-            }
-        }
-    }
+    finish_workgroup<G, ROW16, F16, APPEND, COHERENT>(a, seg, direct, slot_base, new_row, so, sm, sl);
 }
 
 template <int G, int ROW16, bool F16, bool APPEND, bool GATED = false>
