@@ -782,9 +782,12 @@ def main():
                 "frac_basis": "HIP events recorded around the sampled calls on the launch stream: they include the dispatch gap in front "
                               "of the kernel, so frac is a little below the kernel's own (profile_frac, from the committed trace)",
                 "algorithmic_bytes_per_launch": int(avg_bytes),
-                "mfma_utilisation": 0.0,
-                "mfma_note": f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
-                             "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill) and the gate"}
+                "mfma_utilisation": 0.0 if G < 5 else None,
+                "mfma_note": (f"decode tiles are {G} query rows x 128 per KV segment (about 4 flop per byte): computed with v_dot2_f32_bf16 on the "
+                              "VALU, hidden under the loads; MFMA carries the chunk-prefill attention (bench.py --prefill), the gate, and the "
+                              "decode attention from five query heads per KV head on") if G < 5 else
+                             (f"decode tiles are {G} query rows x 128 per KV segment: v_mfma_f32_16x16x32 with the heads padded to 16 columns, "
+                              "16 MFMAs of 16 cycles per 16 KiB streamed and wavefront, i.e. a few per cent of the matrix pipes; the launch is HBM-bound")}
     if roof is not None and args.config == 3 and not args.gate:
         roof.update(profile_kernel_figures(3) or {})
     parity = attention_gate(cache, c, attn_fn, mod, T)

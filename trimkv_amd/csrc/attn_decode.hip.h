@@ -21,6 +21,9 @@
 //     otherwise segments are split and a second, tiny kernel merges the partials;
 //   * rows of 96 or 64 features keep their length in memory: the 16-lane row group then has 12 or 8
 //     loading lanes, the others repeat the last piece against q = 0.
+// With five or more query heads per KV head (rows of 128 features) the dot products start to cost and the
+// kernel body is another one (attend_rows_mfma): the same whole-row loads, but written straight into LDS,
+// and both products on v_mfma_f32_16x16x32 with the heads as the column index.
 #pragma once
 #include "common.hip.h"
 
