@@ -811,7 +811,8 @@ def main():
                    "launches_per_layer_step": (("2: trimkv_gate_hidden, then gate epilogue + append + attend in one launch (trimkv_append_attend_gated)" if args.gate
                                                 else "1: append + attend in one launch (trimkv_append_attend)") if cache.fuse_decode_append
                                                else ("3: trimkv_gate_hidden, trimkv_append_gated, trimkv_decode_attn" if args.gate else "2: trimkv_append, trimkv_decode_attn"))
-                                              + ("" if B * Hkv >= 256 else " + split-K merge"),
+                                              + ("" if B * Hkv >= 256 else (" (segments in equal pieces, merged inside the launch)" if cache.fuse_decode_append and not args.chunk
+                                                                            else " + split-K merge launch")),
                    **timing},
         "step_hbm": {"bytes_moved_per_step": int(bytes_per_step), "achieved_GBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9, 1),
                      "frac_of_8TBps": round(bytes_per_step / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
