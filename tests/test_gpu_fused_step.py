@@ -172,14 +172,17 @@ def test_ragged_fused_step_equals_separate_launches(G):
     assert lens.max() > 10 * lens.min()
 
 
-@pytest.mark.parametrize("D,dtype,lb_dtype", [(64, torch.bfloat16, torch.float32), (96, torch.float16, torch.float16), (128, torch.float16, torch.bfloat16)])
-def test_c_abi_append_attend_other_shapes_full_slabs_and_cu(D, dtype, lb_dtype):
+@pytest.mark.parametrize("D,dtype,lb_dtype,G", [(64, torch.bfloat16, torch.float32, 3), (96, torch.float16, torch.float16, 3), (128, torch.float16, torch.bfloat16, 3),
+                                                (128, torch.float16, torch.float32, 6), (128, torch.bfloat16, torch.bfloat16, 8), (96, torch.bfloat16, torch.float32, 8)])
+def test_c_abi_append_attend_other_shapes_full_slabs_and_cu(D, dtype, lb_dtype, G):
     """Straight through the C ABI: head_dim 64/96, fp16, 16-bit log beta, strided new rows ([B,1,H,D] transposed), cu_seqlens
-    advanced, and a segment whose slab is full (not appended, attends its old rows)."""
+    advanced, and a segment whose slab is full (not appended, attends its old rows); narrow groups (dot-product form of the
+    kernel) and wide ones (MFMA form at head_dim 128, dot-product form with q in LDS below it).  The fused output is also
+    held against fp32 softmax over the rows the launch should have seen."""
     from trimkv_amd import _lib as L
     lib = L.load()
     gen = torch.Generator().manual_seed(D)
-    B, H, G, cap = 3, 2, 3, 700
+    B, H, cap = 3, 2, 700
     nseg = B * H
     lens = np.array([699, 700, 0, 1, 350, 64], dtype=np.int32)      # segment 1 is full, segment 2 empty
     st = L.current_stream(torch.device(DEV))
@@ -220,3 +223,10 @@ def test_c_abi_append_attend_other_shapes_full_slabs_and_cu(D, dtype, lb_dtype):
         assert b["cu"].cpu().tolist() == a["cu"].cpu().tolist()     # cu[i+1] += i+1 for every segment that took a row
         for name in ("k", "v", "lb", "pos"):
             assert torch.equal(a[name], b[name]), name
+        for seg in range(nseg):
+            n = int(after[seg])
+            ks, vs = b["k"][seg, :n].float(), b["v"][seg, :n].float()
+            p = torch.softmax(q.view(nseg, G, D)[seg].float() @ ks.T * scale, -1)
+            ref = p @ vs
+            err = (got.view(nseg, G, D)[seg].float() - ref).abs()
+            assert bool((err <= 2e-2 + 1e-2 * ref.abs()).all()), (seg, float(err.max()))
