@@ -275,6 +275,8 @@ __device__ __forceinline__ void attend_rows_mfma(const AttnArgs& a, int seg, int
     // the rings; once every wavefront has left its loop, the merge buffers of finish_workgroup live in the same memory
     __shared__ __attribute__((aligned(1024))) char ring_all[AT_WAVES * ATM_RING_BYTES];
     static_assert(AT_WAVES * G * AT_D * 4 + 2 * AT_WAVES * 8 * 4 <= AT_WAVES * ATM_RING_BYTES, "merge buffers must fit into the rings");
+    __shared__ __attribute__((aligned(1024))) char q_all[AT_WAVES * 2048];   // per wavefront: q of 8 heads, [head][16 pieces of 16 bytes]
+    static_assert(G <= 8, "q staging holds eight heads");
     float (*so)[G][AT_D] = (float (*)[G][AT_D])ring_all;
     float (*sm)[8] = (float (*)[8])(ring_all + AT_WAVES * G * AT_D * 4);
     float (*sl)[8] = sm + AT_WAVES;
@@ -298,23 +300,10 @@ __device__ __forceinline__ void attend_rows_mfma(const AttnArgs& a, int seg, int
         knew = a.ap.k_new + off;
         vnew = a.ap.v_new + off;
     }
-    // q as the B operand of the score product: lane (head h, group gq) holds features 32 s + 8 gq .. + 7 of k-step s.
-    // These loads (and the new row's) are issued ahead of the stream's first requests: loads return in order, so the
-    // first use of q waits for nothing that the first step would not wait for anyway.
-    at_bf16x8 qb[4];
-    {
-        const uint4* qrow = a.q + ((int64_t)seg * G + min(h, G - 1)) * 16;
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            uint4 t = qrow[4 * s + gq];
-            if (h >= G) t = make_uint4(0u, 0u, 0u, 0u);   // padding columns
-            qb[s] = __builtin_bit_cast(at_bf16x8, t);
-        }
-    }
     uint4 kn = make_uint4(0u, 0u, 0u, 0u), vn = kn;
     float lbn = 0.0f, gate_bias = 0.0f;
     int64_t pn = 0;
-    if (APPEND) {   // fetched by every wavefront (unconditional loads), stored by the wavefront that owns the row
+    if (APPEND) {   // fetched by every wavefront (unconditional loads, ahead of the stream's requests), stored by the wavefront that owns the row
         kn = *(const uint4*)(knew + (h << 4));
         vn = *(const uint4*)(vnew + (h << 4));
         if (GATED) {
@@ -372,10 +361,28 @@ __device__ __forceinline__ void attend_rows_mfma(const AttnArgs& a, int seg, int
         // ring.  Sixteen loads are in flight at the top of a step; a tile is awaited ("all but the newest twelve loads have
         // landed"), read into registers, and its quarter is refilled with the same tile of the next step at once, so 12-16
         // KiB stay in flight.  The last step refills nothing and its waits count down instead.
+        // q takes the same road as K and V (two LDS-direct loads in front of the stream's first requests, then four reads):
+        // a register load here would be the only load the compiler knows of, and its wait for it -- s_waitcnt vmcnt(0), as
+        // far as it can tell -- would hold the wavefront until the whole first ring has landed.
+        const uint32_t q_addr = (uint32_t)(uintptr_t)((AT_LDS3 char*)q_all) + w * 2048;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int head = min(4 * i + gq, G - 1);   // lane (gq, h) fetches piece h of head 4 i + gq (past the last head: its copy, zeroed below)
+            atm_load_to_lds((const char*)(a.q + ((int64_t)seg * G + head) * 16 + h), q_addr + i * 1024);
+        }
         request(w0, 0, std::false_type{});
         request(w0, 1, std::false_type{});
         request(w0, 0, std::true_type{});
         request(w0, 1, std::true_type{});
+        // q as the B operand of the score product: lane (head h, group gq) holds features 32 s + 8 gq .. + 7 of k-step s
+        at_bf16x8 qb[4];
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");   // q has landed (the sixteen loads of the first step may be in flight)
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            at_u32x4 t = *(const AT_LDS3 at_u32x4*)((AT_LDS3 char*)q_all + w * 2048 + min(h, 7) * 256 + (4 * s + gq) * 16);
+            if (h >= G) t = at_u32x4{0u, 0u, 0u, 0u};   // padding columns
+            qb[s] = __builtin_bit_cast(at_bf16x8, t);
+        }
         if (APPEND && new_row >= w0 && new_row < w1) {   // wave-uniform: this wavefront owns the new row and writes it into the slabs
             const int64_t dst = row0 + new_row;
             if (gq == 0) {
