@@ -287,7 +287,7 @@ typedef short pf_s16x4 __attribute__((ext_vector_type(4)));
 
 constexpr int PF2_BN = 64;                          // keys per tile (two 32-key blocks)
 constexpr int PF2_NBUF = 4;                         // tiles in rotation: two being read, two on their way
-constexpr int PF2_TILE = PF2_BN * 256;              // bytes of one K (or V) tile
+constexpr int PF2_TILE = PF2_BN * PF_D * 2;         // bytes of one K (or V) tile: rows of 256 bytes
 constexpr int PF2_VBASE = PF2_NBUF * PF2_TILE;      // 65536: K tiles below, V tiles above
 constexpr int PF2_LDS = 2 * PF2_NBUF * PF2_TILE;    // 131072
 constexpr int PF2_PD = 3;                           // LDS operand reads in flight ahead of the MFMA that consumes them
