@@ -9,10 +9,11 @@ from tests.gpu_util import DEV
 pytestmark = pytest.mark.gpu
 
 
-def test_decode_step_replays_from_a_hip_graph():
+@pytest.mark.parametrize("G", [4, 8])   # the dot-product form of the attention kernel and the MFMA form (LDS-direct loads)
+def test_decode_step_replays_from_a_hip_graph(G):
     from trimkv_amd import _lib as L
     lib = L.load()
-    nlayers, B, H, G, D, cap, n0 = 3, 4, 8, 4, 128, 512, 300
+    nlayers, B, H, D, cap, n0 = 3, 4, 8, 128, 512, 300
     nseg = B * H
     gen = torch.Generator(device=DEV).manual_seed(0)
     rnd = lambda *s: torch.randn(*s, generator=gen, device=DEV)
@@ -74,7 +75,8 @@ def test_decode_step_replays_from_a_hip_graph():
                 assert torch.equal(a[key], b[key]), f"replay {it}: {key} differs"
 
 
-def test_decode_step_including_eviction_replays_from_a_hip_graph():
+@pytest.mark.parametrize("G", [4, 6])
+def test_decode_step_including_eviction_replays_from_a_hip_graph(G):
     """A whole decode step -- per layer trimkv_append_attend (append + attention in one launch), then trimkv_evict_layers for
     all layers -- captured once and replayed 40 times.  Nothing in it depends on host state: the lengths live on the device,
     the eviction kernel re-checks its trigger per segment (slack) and takes its query index from a device counter that the
@@ -83,7 +85,7 @@ def test_decode_step_including_eviction_replays_from_a_hip_graph():
     from trimkv_amd import _lib as L
     from trimkv_amd.cache_utils import _SlabBacked
     lib = L.load()
-    nlayers, B, H, G, D, M, buf = 3, 4, 8, 4, 128, 256, 16
+    nlayers, B, H, D, M, buf = 3, 4, 8, 128, 256, 16
     nseg, cap = B * H, M + buf
     n0 = cap - 5
     gen = torch.Generator(device=DEV).manual_seed(1)
