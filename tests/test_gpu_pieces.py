@@ -179,17 +179,18 @@ def test_append_attend_pieces_equals_append_then_attend():
         assert not ws_b[:32768].any()
 
 
-def test_alternating_layouts_reproduce_their_first_result():
+@pytest.mark.parametrize("G,launches", [(4, 2000), (8, 600)])   # the dot-product form of the kernel body, and the MFMA form (whose merge buffers reuse its LDS rings)
+def test_alternating_layouts_reproduce_their_first_result(G, launches):
     """The in-launch merge, attacked deterministically.  Three different piece lists take turns on ONE workspace, the host
     synchronising after every launch (each launch then starts on an idle GPU and the pieces of a segment finish almost
     together), and before every launch the partial slots are overwritten with NaN.  A merging workgroup that read a slot
     before its writer's stores had landed would therefore read NaN (or, without the poison, another layout's partial) and
     the output would differ from that layout's first launch, which was itself checked against the separate merge kernel:
-    every one of the 2000 launches must reproduce it bit for bit; the loop stops at the first that does not."""
+    every one of the launches must reproduce it bit for bit; the loop stops at the first that does not."""
     from trimkv_amd import _lib as L
     lib = L.load()
     rng = np.random.default_rng(0)
-    nseg, cap, G, D = 256, 8320, 4, 128
+    nseg, cap, D = 256, 8320, 128
     lens = (np.clip(np.round(np.exp(rng.normal(np.log(1024), 1.0, size=nseg))), 64, 8192) + 64).astype(np.int32)
     gen = torch.Generator().manual_seed(0)
     k = torch.randn(nseg, cap, D, generator=gen).to(torch.bfloat16).to(DEV)
@@ -213,7 +214,6 @@ def test_alternating_layouts_reproduce_their_first_result():
                                        nseg, cap, D, G, L.BF16, D ** -0.5, cap, 512, ws0.data_ptr(), ws0.numel(), st), "grid")
         grid.append(want)
     first = {}
-    launches = 2000
     print(f"alternating piece layouts with poisoned partial slots, {launches} launches", flush=True)
     for it in range(launches):
         li, qi = it % 3, (it // 3) % 2
