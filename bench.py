@@ -88,6 +88,41 @@ def profile_kernel_figures(config=3):
             "profile_source": os.path.relpath(path, ROOT)}
 
 
+def stream_ceiling(cache, bytes_per_launch, workgroups=512, reps=3):
+    """What a kernel that only reads gets on this GPU with this step's footprint: `trimkv_stream_probe` over the K and V
+    slabs of every layer, one launch per layer back to back like the attention launches, the same number of bytes per launch.
+    Returns GB/s (launch gaps included, as in the step) and the bytes it read per launch."""
+    import torch
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    slabs = cache._slabs
+    dev = slabs[0].k.device
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    st = L.current_stream(dev)
+    granule = lib.trimkv_stream_probe_granule(workgroups)
+    each = min(min(s.k.numel(), s.v.numel()) * slabs[0].k.element_size() for s in slabs)
+    each = (min(each, bytes_per_launch // 2) // granule) * granule
+    if each <= 0:
+        return None
+
+    def sweep():
+        for s in slabs:
+            L.check(lib.trimkv_stream_probe(s.k.data_ptr(), s.v.data_ptr(), each, workgroups, sink.data_ptr(), st), "trimkv_stream_probe")
+    sweep()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        sweep()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (reps * len(slabs))
+    return {"GBps": round(2 * each / us / 1e3, 1), "frac_of_peak": round(2 * each / us / 1e3 / HBM_PEAK_GBS, 4), "bytes_per_launch": int(2 * each),
+            "us_per_launch": round(us, 2), "launches": reps * len(slabs), "workgroups": workgroups,
+            "what": "trimkv_stream_probe: a load-only kernel (non-temporal 1 KiB loads, a contiguous share per workgroup) over the K and V slabs "
+                    "of every layer, one launch per layer back to back, launch gaps included"}
+
+
 def cpu_baseline(c, budget_s=20.0):
     """The oracle (the reference's pure-PyTorch CPU path restated) on ONE layer at full shape,
     extrapolated to the full step: t_step = L * (B / b) * (t_append_attend + t_evict / buffer)."""
@@ -413,6 +448,11 @@ def ragged_main(args):
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(avg_b / avg_s / 1e9 / HBM_PEAK_GBS, 4),
                 "traffic": None if ratio is None else int(avg_b * ratio), "traffic_source": src, "traffic_measured_in_run": False,
                 "avg_launch_us": round(avg_s * 1e6, 2), "launches_sampled": len(events), "algorithmic_bytes_per_launch": int(avg_b)}
+        if not args.no_stream_probe:
+            ceil = stream_ceiling(cache, int(avg_b))
+            if ceil is not None:
+                roof["stream_ceiling"] = ceil
+                roof["frac_of_stream_ceiling"] = round(roof["achieved"] / ceil["GBps"], 4)
     out_json = {
         "metric": "decode tokens/s (ragged append + varlen attn + per-head evict), Qwen3-4B shape", "value": round(B * args.steps / seconds, 1),
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(seconds * 1e3 / args.steps, 4),
@@ -531,6 +571,7 @@ def main():
     ap.add_argument("--config", type=int, default=3, choices=sorted(list(CONFIGS) + [4]),
                     help="BASELINE config: 3 = headline; 2, 5 = other dense shapes; 4 = ragged per-head budgets (secondary workload)")
     ap.add_argument("--chunk", type=int, default=0, help="split-K rows per workgroup for decode attention (0 = library default)")
+    ap.add_argument("--no-stream-probe", action="store_true", help="skip the load-only probe that measures what a pure read of the step's slabs gets")
     ap.add_argument("--dense-workgroups", type=int, default=0,
                     help="tuning knob: workgroups wanted per dense decode-attention launch (segments are cut into equal pieces to reach it)")
     ap.add_argument("--dense-groups", type=str, default="",
@@ -790,6 +831,11 @@ def main():
                               "16 MFMAs of 16 cycles per 16 KiB streamed and wavefront, i.e. a few per cent of the matrix pipes; the launch is HBM-bound")}
     if roof is not None and args.config == 3 and not args.gate:
         roof.update(profile_kernel_figures(3) or {})
+    if roof is not None and not args.no_stream_probe:
+        ceil = stream_ceiling(cache, int(roof["algorithmic_bytes_per_launch"]))
+        if ceil is not None:
+            roof["stream_ceiling"] = ceil
+            roof["frac_of_stream_ceiling"] = round(roof["achieved"] / ceil["GBps"], 4)
     parity = attention_gate(cache, c, attn_fn, mod, T)
     parity.update(evict_parity)
     timing = {"host_enqueue_ms_per_step": round(enqueue_seconds * 1e3 / args.steps, 4), "ms_append_attend": round(ms_window, 4), "ms_evict_round": round(ms_evict_round, 3), "evict_every_steps": buf}

@@ -507,6 +507,19 @@ int trimkv_decode_attn_static(const void* q, void* out, const void* k_slab, cons
                               int max_len, int chunk, void* stream);
 
 /*
+ * trimkv_stream_probe -- a measurement aid with no counterpart in the reference: a kernel that only reads.
+ * `workgroups` workgroups read the first floor(bytes_each / granule) * granule bytes of `src_a` and then of `src_b`
+ * (granule = trimkv_stream_probe_granule(workgroups)), each workgroup its own contiguous share of either, a quarter per
+ * wavefront, 1 KiB per load instruction, non-temporal: the access pattern of the decode attention (K slab, V slab)
+ * without its arithmetic.  Timed over the slabs a decode step reads, one launch per layer, it gives the share of the HBM
+ * peak that a pure read reaches with that footprint (bench.py: roofline.stream_ceiling).  `sink`: 16 writable bytes on the
+ * device (never written in practice; it keeps the loads alive).
+ * Returns TRIMKV_OK or a negative trimkv_status (null pointers, misaligned pointers, fewer bytes than one granule).
+ */
+int64_t trimkv_stream_probe_granule(int workgroups);
+int trimkv_stream_probe(const void* src_a, const void* src_b, int64_t bytes_each, int workgroups, void* sink, void* stream);
+
+/*
  * trimkv_prefill_attn -- GQA attention of a block of q_len queries (a prompt or prompt chunk)
  * over every segment's retained K/V, bottom-right causal: query t sees keys j <= n - q_len + t,
  * n = seg_len[seg] (the chunk's own tokens are already appended).  A query that sees no key

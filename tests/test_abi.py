@@ -61,6 +61,12 @@ def test_bad_arguments_are_refused_without_a_launch():
     assert attn(cap=4096, max_len=4096, chunk=256) == -5  # split-K needs a workspace
     assert attn(chunk=100) == -2
     assert lib.trimkv_decode_attn(None, one, one, one, one, None, None, None, 4, 64, 128, 4, _lib.BF16, 0.1, 64, 0, None, 0, None) == -1
+    # the load-only probe: null pointers, too few bytes, misaligned source
+    gran = lib.trimkv_stream_probe_granule(512)
+    assert gran == 512 * 4 * 1024 and lib.trimkv_stream_probe_granule(0) == 0
+    assert lib.trimkv_stream_probe(None, one, gran, 512, one, None) == -1 and lib.trimkv_stream_probe(one, one, gran, 512, None, None) == -1
+    assert lib.trimkv_stream_probe(one, one, gran - 1, 512, one, None) == -2 and lib.trimkv_stream_probe(one, one, gran, 0, one, None) == -2
+    assert lib.trimkv_stream_probe(ctypes.c_void_p(24), one, gran, 512, one, None) == -2
     # eviction: capacity, strategy, alignment of head_dim
     def evict(cap=64, D=128, keep=8, strat=0, rnd=0, max_len=64):
         return lib.trimkv_evict(one, one, one, one, one, 4, cap, D, _lib.BF16, _lib.F32, keep, None, 0, 100, strat, rnd, 0,

@@ -70,6 +70,8 @@ SIGNATURES = {
     "trimkv_plan_attn_pieces": (_i, [_p, _i, _i, _i, _p, _i]),
     "trimkv_decode_attn_static": (_i, [_p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _f, _i, _i, _p]),
     "trimkv_prefill_attn": (_i, [_p, _i64, _i64, _i64, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "trimkv_stream_probe_granule": (_i64, [_i]),
+    "trimkv_stream_probe": (_i, [_p, _p, _i64, _i, _p, _p]),
 }
 
 _lib = None
