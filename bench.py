@@ -316,6 +316,24 @@ def prefill_main(args):
                      "frac": round(flops / avg_s / 1e12 / 2500.0, 4), "traffic": None, "avg_launch_us": round(avg_s * 1e6, 1),
                      "launches_sampled": len(events), "algorithmic_flops_per_launch": int(flops)},
     }
+    if not args.no_stream_probe:
+        # for scale: what the vendor library's plain bf16 GEMM reaches on this GPU in this process (the chip's clock drops
+        # under MFMA load, so 2.5 PFLOP/s is not what a matrix kernel can be held against)
+        ng = 8192
+        ga = torch.randn(ng, ng, device=dev, dtype=torch.bfloat16)
+        gb = torch.randn(ng, ng, device=dev, dtype=torch.bfloat16)
+        for _ in range(5):
+            ga @ gb
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        g0.record()
+        for _ in range(30):
+            ga @ gb
+        g1.record()
+        torch.cuda.synchronize()
+        gemm = 2.0 * ng ** 3 * 30 / (g0.elapsed_time(g1) * 1e-3) / 1e12
+        out["roofline"]["vendor_gemm_bf16"] = {"TFLOPs": round(gemm, 1), "frac_of_peak": round(gemm / 2500.0, 4),
+                                               "what": "torch.matmul of two 8192 x 8192 bf16 matrices (the vendor GEMM library), 30 calls between two events"}
+        out["roofline"]["frac_of_vendor_gemm"] = round(out["roofline"]["achieved"] / gemm, 4)
     if args.layers:
         out["config"]["note"] = "layer count overridden: not the BASELINE configuration"
     print(json.dumps(out))
