@@ -1,0 +1,142 @@
+"""Decode steps of the thin decoders replayed from a HIP graph (trimkv_amd/graphed.py).
+
+A replayed step must be the eager step: the same launches with the same arguments.  So the strong check is bitwise: a
+twin model + cache runs the same tokens eagerly in the same device-side step mode (lengths read on the device), and
+after EVERY replay -- with that eager work and a synchronisation in between -- logits, slabs, lengths and the host
+mirrors of the two caches must be equal, across several evictions.  A second check compares with the ordinary eager
+step (lengths as launch arguments), whose attention launch merges in another order: logits within the attention
+tolerance, teacher-forced."""
+import copy
+
+import pytest
+import torch
+
+from tests.gpu_util import DEV
+from tests.test_gpu_qwen3_shell import _family, _tiny_config
+
+pytestmark = pytest.mark.gpu
+
+
+def _model(family, gate, **kw):
+    cfg = _tiny_config(family, retention_gate=gate, **kw)
+    torch.manual_seed(0)
+    model = _family(family)[1](cfg).to(torch.bfloat16).to(DEV).eval()
+    return cfg, model
+
+
+def _same_state(a, b, where):
+    assert a.get_seq_length() == b.get_seq_length(), where
+    for l, (sa, sb) in enumerate(zip(a._slabs, b._slabs)):
+        assert sa.max_len == sb.max_len and (sa.lens == sb.lens).all() and sa.total == sb.total, f"{where}: host mirrors of layer {l}"
+        assert a.n_seen_tokens[l] == b.n_seen_tokens[l], where
+        assert torch.equal(sa.seg_len, sb.seg_len), f"{where}: seg_len of layer {l}"
+        assert (sa.seg_len.cpu().numpy() == sa.lens).all(), f"{where}: mirror and device lengths of layer {l} disagree"
+        n = sa.max_len
+        for name in ("k", "v", "lb", "pos"):
+            assert torch.equal(getattr(sa, name)[:, :n], getattr(sb, name)[:, :n]), f"{where}: {name} of layer {l}"
+
+
+@pytest.mark.parametrize("family,gate", [("qwen3", "rg"), ("qwen3", "rg2"), ("qwen3", "rg3"), ("llama", "rg"), ("phi3", "rg2")])
+def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate):
+    from trimkv_amd.graphed import GraphedDecoder
+    cfg, model = _model(family, gate)
+    M, buf = cfg.memory_size, cfg.buffer_size
+    B, prompt, steps = 3, 90, 3 * buf + 5                     # three evictions inside the replays
+    gen = torch.Generator().manual_seed(1)
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps), generator=gen).to(DEV)
+    with torch.no_grad():
+        out_g = model(ids[:, :prompt], logits_to_keep=1)
+        out_e = model(ids[:, :prompt], logits_to_keep=1)
+    cache_g, cache_e = out_g.past_key_values, out_e.past_key_values
+    assert cache_g.get_cache_length(0) == M                   # the prompt was evicted to the budget
+    dec = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    cache_e.begin_device_steps(M, buf)                        # the eager twin issues the same launches
+    evictions = 0
+    for i in range(steps):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        before = cache_g.get_cache_length(0)
+        logits_g = dec(input_ids=tok).logits
+        with torch.no_grad():                                 # eager work between the replays
+            logits_e = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
+        torch.cuda.synchronize()
+        assert torch.equal(logits_g, logits_e), f"step {i}: logits of the replay differ from the eager step"
+        _same_state(cache_g, cache_e, f"step {i}")
+        evictions += cache_g.get_cache_length(0) < before
+    assert dec.graph is not None and dec.calls == steps
+    assert evictions == 3
+    assert cache_g.get_seq_length() == prompt + steps
+    dec.close()
+    assert not cache_g.lengths_on_device
+    # the cache goes on eagerly, sized from the host mirrors again
+    with torch.no_grad():
+        tok = ids[:, :1]
+        a = model(tok, past_key_values=cache_g, logits_to_keep=1).logits
+        cache_e.end_device_steps()
+        b = model(tok, past_key_values=cache_e, logits_to_keep=1).logits
+    assert torch.equal(a, b)
+
+
+def test_replayed_steps_match_the_ordinary_eager_steps():
+    """Against the step every other test pins (lengths as launch arguments, pieces merged inside the launch): the same
+    tokens, logits within the attention tolerance at every step, and the same lengths."""
+    from trimkv_amd.graphed import GraphedDecoder
+    cfg, model = _model("qwen3", "rg")
+    B, prompt, steps = 2, 90, 40
+    gen = torch.Generator().manual_seed(2)
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps), generator=gen).to(DEV)
+    with torch.no_grad():
+        cache_g = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+        cache_e = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+    dec = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    scale, worst = 0.0, 0.0
+    for i in range(steps):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        lg = dec(input_ids=tok).logits.float()
+        with torch.no_grad():
+            le = model(tok, past_key_values=cache_e, logits_to_keep=1).logits.float()
+        worst = max(worst, float((lg - le).abs().max()))
+        scale = max(scale, float(le.abs().max()))
+        assert cache_g.get_cache_length(0) == cache_e.get_cache_length(0)
+    assert worst <= 2e-2 + 1e-2 * scale, (worst, scale)
+
+
+def test_generate_with_a_graph_returns_the_eager_tokens():
+    """generate(use_graph=True) against a hand-written greedy loop over eager device-side steps: the same tokens."""
+    cfg, model = _model("qwen3", "rg")
+    B, prompt, new = 2, 50, 45
+    gen = torch.Generator().manual_seed(3)
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt), generator=gen).to(DEV)
+    got = model.generate(ids, new, use_graph=True)
+    with torch.no_grad():
+        out = model(ids, logits_to_keep=1)
+        cache = out.past_key_values
+        cache.begin_device_steps(cfg.memory_size, cfg.buffer_size)
+        toks = [ids]
+        for i in range(new):
+            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+            toks.append(nxt)
+            if i + 1 < new:
+                out = model(nxt, past_key_values=cache, logits_to_keep=1)
+    assert torch.equal(got, torch.cat(toks, dim=1))
+
+
+def test_graphed_decoder_refuses_what_it_cannot_replay():
+    from trimkv_amd import BatchedDynamicBudgetTrimKVCache, TrimKVCache
+    from trimkv_amd.graphed import GraphedDecoder
+    cfg, model = _model("qwen3", "rg")
+    with pytest.raises(TypeError):
+        GraphedDecoder(model, BatchedDynamicBudgetTrimKVCache())
+    with pytest.raises(RuntimeError):
+        GraphedDecoder(model, TrimKVCache())                  # no prompt yet
+    cfg2 = copy.copy(cfg)
+    cfg2.compress_memory = False
+    model2 = copy.copy(model)
+    model2.config = cfg2
+    with torch.no_grad():
+        cache = model(torch.zeros(1, 8, dtype=torch.int64, device=DEV)).past_key_values
+    with pytest.raises(ValueError):
+        GraphedDecoder(model2, cache)
+    dec = GraphedDecoder(model, cache)
+    with pytest.raises(ValueError):
+        dec(input_ids=torch.zeros(1, 2, dtype=torch.int64, device=DEV))
+    dec.close()

@@ -143,10 +143,11 @@ def decode_attention(query: torch.Tensor, k_rows: torch.Tensor, v_rows: torch.Te
 
 
 def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: int = 0,
-                  seg_order: Optional[torch.Tensor] = None, pieces=None, uniform_pps: int = 0) -> torch.Tensor:
+                  seg_order: Optional[torch.Tensor] = None, pieces=None, uniform_pps: int = 0, bound: int = 0) -> torch.Tensor:
     """The deferred one-token append of ``slab`` (a cache layer whose ``update`` ran with ``fuse_decode_append``) and the
     attention over the layer including that token, in one launch: ``trimkv_append_attend``.  ``query`` [nseg*group, D]
-    contiguous -> [nseg*group, D].  Clears the pending append."""
+    contiguous -> [nseg*group, D].  Clears the pending append.  ``bound`` > 0: the launch is sized for segments of up to
+    that many rows instead of the host's record of the longest one (a step that must not depend on host-side lengths)."""
     lib = _lib.load()
     nseg, d = slab.B * slab.H, slab.D
     out = torch.empty_like(query)
@@ -172,12 +173,13 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
             _lib.check(rc, "trimkv_append_attend_pieces_gated" if gated else "trimkv_append_attend_pieces")
         slab.pending = None
         return out
-    ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, slab.max_len, chunk)
+    max_len = bound if bound > 0 else slab.max_len
+    ws_bytes = lib.trimkv_decode_attn_workspace(nseg, group, d, max_len, chunk)
     ws = _workspace(query.device, ws_bytes, st) if ws_bytes else None
     # slab.pending[0] = the new row's addresses and strides, in the order of the entry point's parameters
     fn = lib.trimkv_append_attend_gated if gated else lib.trimkv_append_attend
     rc = fn(query.data_ptr(), out.data_ptr(), *slab.ptrs, None if seg_order is None else seg_order.data_ptr(), nseg, slab.H, slab.cap, d, group,
-            *slab.codes, *slab.pending[0], scale, slab.max_len, chunk, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
+            *slab.codes, *slab.pending[0], scale, max_len, chunk, None if ws is None else ws.data_ptr(), 0 if ws is None else ws.numel(), st)
     if rc:
         _lib.check(rc, "trimkv_append_attend_gated" if gated else "trimkv_append_attend")
     slab.pending = None
@@ -331,7 +333,9 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
     plain = not dropout and softcap is None        # what the kernels compute: softmax(q k^T * scale) v
     # every segment of a dense cache holds n rows: length and cut go to the kernel as launch arguments (pps pieces per segment)
     pps = 0
-    if Q == 1 and not dense_chunk and G <= _MAX_GROUP:
+    # a cache between begin_device_steps and end_device_steps: the launch must not depend on the host's record of the lengths
+    on_device = bool(flash_attn_kwargs and flash_attn_kwargs.get("lengths_on_device"))
+    if Q == 1 and not dense_chunk and G <= _MAX_GROUP and not on_device:
         pps = _uniform_cut(B * Hkv, n)
         if pps > 1 and G not in _DENSE_PIECES_GROUPS:
             pps = 0    # wide groups in pieces: the grid launch + merge kernel
@@ -342,7 +346,8 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
             q2 = q2.contiguous()
         if slab.cu is not None:
             pps = 0
-        return append_attend(slab, q2, G, scale, chunk=dense_chunk, uniform_pps=pps).view(B, 1, Hq, D), None, None
+        return append_attend(slab, q2, G, scale, chunk=dense_chunk, uniform_pps=pps,
+                             bound=slab.cap if on_device else 0).view(B, 1, Hq, D), None, None
     kernel_ok = plain and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128)
     seg_first = None
     if kernel_ok and Q == 1:
@@ -363,7 +368,8 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         seg_len = flash_attn_kwargs.get("seg_len") if flash_attn_kwargs else None
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
-        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, n, scale, chunk=dense_chunk, seg_first=seg_first, uniform_pps=pps)
+        out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, cap if on_device and seg_len is not None else n, scale,
+                               chunk=dense_chunk, seg_first=seg_first, uniform_pps=pps)
         return out.view(B, 1, Hq, D), None, None
     if kernel_ok and Q > 1 and attention_mask is None and window is None and causal:
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)

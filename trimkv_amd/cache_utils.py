@@ -470,6 +470,89 @@ class TrimKVCache(_SlabBacked):
 
     def __init__(self, max_seq_len: int = 20480, _distributed_cache_data: Iterable = None, device: str = "cuda") -> None:
         super().__init__(max_seq_len, _distributed_cache_data, device)
+        # Decode steps whose launches depend on no host-side length (begin_device_steps): what a HIP graph can replay.
+        self.lengths_on_device = False
+        self._seen_dev: Optional[torch.Tensor] = None   # device int64 [1]: tokens seen + 1, the query index of an eviction
+
+    # ---- decode steps that a HIP graph can replay ------------------------------------------------
+    def begin_device_steps(self, memory_size: int, buffer_size: int) -> None:
+        """From here on a decode step enqueues the same launches with the same arguments whatever the lengths are: the
+        attention launch reads the segment lengths on the device (``trimkv_append_attend`` with the slab capacity as the
+        bound, not the ``_uniform`` entry points that take the length as an argument), ``compress`` issues its launch at
+        every step and the kernel itself checks per segment whether ``memory_size + buffer_size`` rows have been reached
+        (``slack``), with the query index read from a device counter that ``update`` advances.  Such a step can be captured
+        once and replayed; ``advance_decode_mirrors`` then does the host bookkeeping of a replay.  The slabs are brought to
+        ``memory_size + buffer_size`` rows if they are smaller, so that no step has to move them."""
+        self._flush_all()
+        slabs = self._slabs
+        if not slabs or any(s is None for s in slabs):
+            raise RuntimeError("begin_device_steps: every layer must hold a prompt first")
+        if not self._layers_alike(list(range(len(slabs)))):
+            raise RuntimeError("begin_device_steps: all layers must have one shape, dtype and device")
+        hint = memory_size + buffer_size
+        if any(s.max_len >= hint for s in slabs):
+            raise RuntimeError(f"begin_device_steps: a layer already holds {hint} rows or more; compress() first")
+        if any(n != self._seen_tokens for n in self.n_seen_tokens):
+            raise RuntimeError("begin_device_steps: the layers have seen different numbers of tokens")
+        for s in slabs:
+            if s.cap < hint:
+                s.regrow(hint)
+        self._budget_hint = hint
+        self._seen_dev = torch.full((1,), self._seen_tokens + 1, dtype=torch.int64, device=slabs[0].k.device)
+        self.lengths_on_device = True
+
+    def end_device_steps(self) -> None:
+        """Back to launches sized from the host mirrors of the lengths."""
+        self._flush_all()
+        self.lengths_on_device, self._seen_dev = False, None
+
+    def _compress_on_device(self, strategy: str, memory_size: int, buffer_size: int, skip_layers: int, num_layers: int) -> None:
+        """compress() between begin_device_steps and end_device_steps: one ``trimkv_evict_layers`` launch over all layers
+        at every step; a segment is evicted to ``memory_size`` rows iff it holds ``memory_size + buffer_size`` or more."""
+        layers = list(range(skip_layers, num_layers))
+        if not layers:
+            return
+        s0 = self._slabs[layers[0]]
+        dev = s0.k.device
+        cap = min(self._slabs[l].cap for l in layers)
+        lib = _lib.load()
+        table = self._device_tables(layers)["slabs"]
+        ws = self._workspace(len(layers) * lib.trimkv_evict_workspace(s0.nseg, cap), dev)
+        rc = lib.trimkv_evict_layers(table.data_ptr(), len(layers), s0.nseg, s0.D, _lib.dtype_code(s0.k.dtype), _lib.dtype_code(s0.lb.dtype),
+                                     int(memory_size), None, 0, int(buffer_size), 0, self._seen_dev.data_ptr(),
+                                     self._dense_strategy_code(strategy), _lib.ROUND_UPCAST, int(self.sliding_window_size), cap,
+                                     _lib.ptr(ws), 0 if ws is None else ws.numel(), _lib.current_stream(dev))
+        _lib.check(rc, "trimkv_evict_layers")
+        for l in layers:
+            slab = self._slabs[l]
+            if slab.max_len >= memory_size + buffer_size:
+                slab.lens[:] = memory_size
+                slab.max_len = memory_size
+
+    def mirror_snapshot(self):
+        """The host-side bookkeeping (tokens seen, lengths) as a value that ``mirror_restore`` puts back: capturing a step
+        in a graph runs this class's Python, which advances the mirrors, without executing anything on the device."""
+        return (self._seen_tokens, list(self.n_seen_tokens), [(s.lens.copy(), s.max_len, s.total) for s in self._slabs])
+
+    def mirror_restore(self, snap) -> None:
+        self._seen_tokens, self.n_seen_tokens = snap[0], list(snap[1])
+        for s, (lens, max_len, total) in zip(self._slabs, snap[2]):
+            s.lens[:] = lens
+            s.max_len, s.total, s.pending = max_len, total, None
+
+    def advance_decode_mirrors(self, memory_size: int, buffer_size: int, skip_layers: int = 0) -> None:
+        """Host bookkeeping of one replayed decode step: what ``update`` of every layer (one token) and the ``compress``
+        after it do to the mirrors when they run eagerly."""
+        self._seen_tokens += 1
+        for l, s in enumerate(self._slabs):
+            self.n_seen_tokens[l] += 1
+            s.lens += 1
+            s.max_len += 1
+            s.total += s.lens.size
+        for s in self._slabs[skip_layers:]:
+            if s.max_len >= memory_size + buffer_size:
+                s.lens[:] = memory_size
+                s.max_len = memory_size
 
     # The reference exposes four per-layer lists; here they are live views of the slabs.
     @property
@@ -530,6 +613,8 @@ class TrimKVCache(_SlabBacked):
             seq_len = key_states.shape[-2]
             if layer_idx == 0:
                 self._seen_tokens += seq_len
+                if self._seen_dev is not None:
+                    self._seen_dev.add_(seq_len)
             self._ensure_layer(layer_idx)
             slab = self._slabs[layer_idx]
             if not (seq_len == 1 and self.fuse_decode_append and slab is not None
@@ -540,6 +625,8 @@ class TrimKVCache(_SlabBacked):
         if slab is None:
             return (*self._layer_tuple(layer_idx), {})
         extra = {"seg_len": slab.seg_len, "max_len": slab.max_len, "seg_cap": slab.cap}
+        if self.lengths_on_device:
+            extra["lengths_on_device"] = True
         if slab.pending is not None:
             # the last of the max_len rows is not in the slab yet: the attention call that receives this dictionary writes it
             extra["pending_append"] = (self, slab)
@@ -557,6 +644,8 @@ class TrimKVCache(_SlabBacked):
         heads = first.H if first is not None else 0
         num_key_value_heads = heads if num_key_value_heads is None else num_key_value_heads
         assert num_key_value_heads == heads, "Key and value caches must have the same number of heads"
+        if self.lengths_on_device:
+            return self._compress_on_device(strategy, memory_size, buffer_size, skip_layers, num_layers)
         self._budget_hint = memory_size + buffer_size
         todo = [l for l in range(skip_layers, num_layers) if memory_size + buffer_size <= self.get_cache_length(l)]
         if len(todo) > 1 and self._layers_alike(todo):   # the usual case: every layer is due at the same step -> one launch

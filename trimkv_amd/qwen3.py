@@ -387,18 +387,30 @@ class TrimKVQwen3ForCausalLM(nn.Module):
         return SimpleNamespace(logits=self.lm_head(h), past_key_values=out.past_key_values)
 
     @torch.no_grad()
-    def generate(self, input_ids: torch.Tensor, max_new_tokens: int, past_key_values=None, prefill_chunk: int = 0):
+    def generate(self, input_ids: torch.Tensor, max_new_tokens: int, past_key_values=None, prefill_chunk: int = 0,
+                 use_graph: bool = False):
         """Greedy decoding.  ``prefill_chunk`` > 0 streams the prompt in chunks of that many tokens, evicting after
-        each (the long-prompt mode of the reference's examples); returns prompt + new tokens."""
+        each (the long-prompt mode of the reference's examples); returns prompt + new tokens.  ``use_graph``: the decode
+        steps are captured in a HIP graph once and replayed (``trimkv_amd.graphed.GraphedDecoder``; dense cache with
+        ``compress_memory`` only); the cache goes back to host-sized launches when the call returns."""
         chunk = prefill_chunk or input_ids.shape[1]
         out = None
         for s in range(0, input_ids.shape[1], chunk):
             out = self(input_ids[:, s:s + chunk], past_key_values=past_key_values, logits_to_keep=1)
             past_key_values = out.past_key_values
+        step, graphed = self, None
+        if use_graph and max_new_tokens > 1:
+            from .graphed import GraphedDecoder
+            graphed = GraphedDecoder(self, past_key_values, logits_to_keep=1)
+            step = lambda ids, **_: graphed(input_ids=ids)
         tokens = [input_ids]
-        for i in range(max_new_tokens):
-            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
-            tokens.append(nxt)
-            if i + 1 < max_new_tokens:
-                out = self(nxt, past_key_values=past_key_values, logits_to_keep=1)
+        try:
+            for i in range(max_new_tokens):
+                nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+                tokens.append(nxt)
+                if i + 1 < max_new_tokens:
+                    out = step(nxt, past_key_values=past_key_values, logits_to_keep=1)
+        finally:
+            if graphed is not None:
+                graphed.close()
         return torch.cat(tokens, dim=1)
