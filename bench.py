@@ -494,7 +494,8 @@ def shell_main(args):
     """Secondary workload (--shell): decode steps of the thin Qwen3 decoder at the Qwen3-8B layer shape (hidden 4096, 32 query
     / 8 KV heads, MLP 12288, random bf16 weights, batch 64) on a cache in the steady state of config 3.  It measures what
     the `rg` retention gate costs a decode step inside a model: gate on a second stream beside the q/k/v projections (the
-    shell's default), gate on the main stream, and no gate at all (log beta a constant tensor), same cache contents."""
+    shell's opt-in), gate on the main stream, and no gate at all (log beta a constant tensor), same cache contents -- each
+    both eagerly ("gate" in the output) and with the step replayed from a HIP graph ("graph")."""
     import torch
     from trimkv_amd import TrimKVCache
     from trimkv_amd.qwen3 import TrimKVQwen3Attention, TrimKVQwen3Config, TrimKVQwen3Model
@@ -517,7 +518,7 @@ def shell_main(args):
     model.eval()
     gen = torch.Generator(device=dev).manual_seed(0)
     steps, warm = args.steps, args.warmup
-    n0 = M + max(1, (buf - 6 * (steps + warm) - 2) // 2)     # all runs (three variants, twice) fit inside one eviction cycle
+    n0 = M + max(1, (buf - 6 * (steps + warm) - 10) // 2)    # all runs of a cache (three variants, twice) fit inside one eviction cycle
 
     def fresh_cache():
         cache = TrimKVCache()
@@ -561,17 +562,56 @@ def shell_main(args):
     for kind in ("none", "side", "main", "none", "side", "main"):     # two rounds, alternating: the rows grow by one per step
         ms, enq = run(kind)
         res.setdefault(kind, []).append((ms, enq))
-    TrimKVQwen3Attention.gate_on_side_stream = True
+    TrimKVQwen3Attention.gate_on_side_stream = False
     assert cache.get_cache_length(0) < M + buf, "the window must not contain an eviction"
     best = {k: min(m for m, _ in v) for k, v in res.items()}
+
+    # The same three variants with the step captured in a HIP graph once and replayed (trimkv_amd.graphed.GraphedDecoder),
+    # on a fresh cache of the same contents.  The eviction launch is part of every replayed step (it finds nothing due).
+    from trimkv_amd.graphed import GraphedDecoder
+    del cache
+    torch.cuda.empty_cache()
+    cache = fresh_cache()
+    decoders = {}
+
+    def run_graph(kind):
+        dec = decoders.get(kind)
+        if dec is None:
+            for layer, g in zip(model.layers, gates):
+                layer.self_attn.retention_gate = NoGate() if kind == "none" else g
+            dec = decoders[kind] = GraphedDecoder(model, cache, gate_on_side_stream=kind == "side")
+            dec(inputs_embeds=x)        # eager, warms up the capture's stream
+            dec(inputs_embeds=x)        # captures, then replays
+        for _ in range(warm):
+            dec(inputs_embeds=x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            dec(inputs_embeds=x)
+        enq = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        sec = time.perf_counter() - t0
+        return sec * 1e3 / steps, enq * 1e3 / steps
+
+    gres = {}
+    for kind in ("none", "side", "main", "none", "side", "main"):
+        ms, enq = run_graph(kind)
+        gres.setdefault(kind, []).append((ms, enq))
+    assert cache.get_cache_length(0) < M + buf, "the window must not contain an eviction"
+    gbest = {k: min(m for m, _ in v) for k, v in gres.items()}
     out = {
-        "metric": "decode ms/step of the thin Qwen3 decoder at the Qwen3-8B layer shape: rg gate beside the projections vs no gate",
-        "value": round(best["side"], 4), "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(best["side"], 4),
+        "metric": "decode ms/step of the thin Qwen3 decoder at the Qwen3-8B layer shape, step replayed from a HIP graph, rg gate beside the projections",
+        "value": round(gbest["side"], 4), "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": round(gbest["side"], 4),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"thin TrimKV Qwen3 decoder, {L} layers of the Qwen3-8B shape (hidden {args.hidden}, {Hq} query / {Hkv} KV heads, "
                                f"head_dim {D}, MLP {3 * args.hidden}), random bf16 weights, batch {B}, cache of {cache.get_cache_length(0)} rows per head "
                                f"(memory_size {M}, buffer_size {buf}), fused append + attend, no eviction inside the window",
                    "note": "secondary workload; the headline metric is the default run"},
+        "graph": {"ms_per_step_gate_on_second_stream": round(gbest["side"], 4), "ms_per_step_gate_on_main_stream": round(gbest["main"], 4),
+                  "ms_per_step_without_gate": round(gbest["none"], 4),
+                  "gate_cost_second_stream_pct": round((gbest["side"] / gbest["none"] - 1) * 100, 2),
+                  "gate_cost_main_stream_pct": round((gbest["main"] / gbest["none"] - 1) * 100, 2),
+                  "all_runs_ms_and_host_enqueue_ms": {k: [(round(m, 4), round(e, 4)) for m, e in v] for k, v in gres.items()}},
         "gate": {"ms_per_step_gate_on_second_stream": round(best["side"], 4), "ms_per_step_gate_on_main_stream": round(best["main"], 4),
                  "ms_per_step_without_gate": round(best["none"], 4),
                  "gate_cost_second_stream_pct": round((best["side"] / best["none"] - 1) * 100, 2),

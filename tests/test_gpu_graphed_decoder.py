@@ -36,8 +36,10 @@ def _same_state(a, b, where):
             assert torch.equal(getattr(sa, name)[:, :n], getattr(sb, name)[:, :n]), f"{where}: {name} of layer {l}"
 
 
-@pytest.mark.parametrize("family,gate", [("qwen3", "rg"), ("qwen3", "rg2"), ("qwen3", "rg3"), ("llama", "rg"), ("phi3", "rg2")])
-def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate):
+@pytest.mark.parametrize("family,gate,fork", [("qwen3", "rg", False), ("qwen3", "rg", True), ("qwen3", "rg2", False), ("qwen3", "rg3", False),
+                                              ("llama", "rg", False), ("phi3", "rg2", False)])
+def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate, fork):
+    """``fork``: the `rg` gate runs on a second stream inside the graph, beside the projections."""
     from trimkv_amd.graphed import GraphedDecoder
     cfg, model = _model(family, gate)
     M, buf = cfg.memory_size, cfg.buffer_size
@@ -49,7 +51,7 @@ def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate):
         out_e = model(ids[:, :prompt], logits_to_keep=1)
     cache_g, cache_e = out_g.past_key_values, out_e.past_key_values
     assert cache_g.get_cache_length(0) == M                   # the prompt was evicted to the budget
-    dec = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    dec = GraphedDecoder(model, cache_g, gate_on_side_stream=fork, logits_to_keep=1)
     cache_e.begin_device_steps(M, buf)                        # the eager twin issues the same launches
     evictions = 0
     for i in range(steps):

@@ -7,8 +7,10 @@ once, and replays it per token.  What makes the step replayable is in the cache:
 ``end_device_steps`` a dense ``TrimKVCache`` enqueues launches that read the segment lengths, the position and the query
 index of the eviction on the device, so the same recorded launches are right at every step, eviction steps included.
 
-Inside the graph the `rg` gate is forked onto a second stream of the same priority and runs beside the q/k/v
-projections; a replay costs the host nothing for that.
+The `rg` gate stays on the stream of the step by default.  ``gate_on_side_stream=True`` forks it inside the graph onto a
+second stream of the same priority, beside the q/k/v projections; measured at the Qwen3-8B shape (36 layers, batch 64)
+that replay is slower, not faster (19.0 ms against 17.2 ms per step, 16.7 ms without a gate): a graph with 36 forks and
+joins replays through several queues with host-side hand-overs (16.5 ms of host time per replay against 5.5 ms).
 
 No counterpart in the reference (its decoders run eagerly under HF ``generate``); the call order of the captured step is
 the reference's (modeling_trimkv_qwen3.py:315-388, 751-760).
@@ -32,7 +34,7 @@ class GraphedDecoder:
     ``compress_memory`` on and the ``trimkv_hip`` attention; ``cache``: the dense ``TrimKVCache`` that holds the prompt.
     ``forward_kwargs`` are passed to every call of the model (e.g. ``logits_to_keep=1``)."""
 
-    def __init__(self, model, cache: TrimKVCache, gate_on_side_stream: bool = True, **forward_kwargs):
+    def __init__(self, model, cache: TrimKVCache, gate_on_side_stream: bool = False, **forward_kwargs):
         cfg = model.config
         if type(cache) is not TrimKVCache:
             raise TypeError("GraphedDecoder replays steps of the dense TrimKVCache only")
