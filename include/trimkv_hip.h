@@ -113,6 +113,23 @@ int trimkv_gate_hidden_swiglu(const void* x, const void* w_gate, const void* w_u
                               int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
 
 /*
+ * trimkv_gate_pack_weights / trimkv_gate_hidden_packed / trimkv_gate_hidden_swiglu_packed -- the first-layer
+ * weights of a gate (`linear1.weight`, :150; `gate_proj.weight` and `up_proj.weight`, :240-241), which are
+ * constants, stored once in the order the lanes of the decode-sized kernel read them, so that every load
+ * instruction fetches 1 KiB contiguous instead of 16 rows x 64 bytes (a 64-token call at hidden 4096,
+ * inter 512 takes about 2 us less).  trimkv_gate_pack_weights writes the packed copy of w [inter][hidden]
+ * (same size and dtype, 16-byte aligned, not in place); the *_packed calls take packed matrices where
+ * trimkv_gate_hidden(_swiglu) take row-major ones, compute the same bits, and serve ntok <= 256
+ * (TRIMKV_ERR_UNSUPPORTED beyond: prompts go through the row-major entry points).  The packed
+ * layout is private to this library version: pack again after an upgrade, never store it.
+ */
+int trimkv_gate_pack_weights(const void* w, void* packed, int hidden, int inter, int dtype, void* stream);
+int trimkv_gate_hidden_packed(const void* x, const void* w1_packed, const void* b1, const void* w2, float* part,
+                              int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
+int trimkv_gate_hidden_swiglu_packed(const void* x, const void* w_gate_packed, const void* w_up_packed, const void* w_down, float* part,
+                                     int ntok, int hidden, int inter, int kv_heads, int dtype, void* stream);
+
+/*
  * trimkv_append_gated -- trimkv_append whose log(beta) is produced inside the append kernel:
  *     lb[b][h][s] = logsigmoid( sum_j part[j][b*s_new + s][h] + gate_bias[h] )
  * rounded to lb_dtype (modeling_trimkv_qwen3.py:177-179, then the transpose at :333).

@@ -86,6 +86,11 @@ def test_bad_arguments_are_refused_without_a_launch():
     assert lib.trimkv_gate_hidden(one, one, one, one, one, 8, 4224, 512, 8, _lib.BF16, None) == -6
     assert lib.trimkv_gate_hidden_swiglu(one, one, None, one, one, 8, 2048, 512, 8, _lib.BF16, None) == -1   # no up_proj
     assert lib.trimkv_gate_hidden_swiglu(one, one, one, one, one, 8, 2048, 500, 8, _lib.BF16, None) == -6
+    assert lib.trimkv_gate_pack_weights(one, None, 4096, 512, _lib.BF16, None) == -1
+    assert lib.trimkv_gate_pack_weights(one, one, 4096, 512, _lib.BF16, None) == -2            # in place
+    assert lib.trimkv_gate_pack_weights(one, ctypes.c_void_p(32), 4100, 512, _lib.BF16, None) == -6
+    assert lib.trimkv_gate_hidden_packed(one, one, one, one, one, 300, 4096, 512, 8, _lib.BF16, None) == -6   # prompts: row-major weights
+    assert lib.trimkv_gate_hidden_swiglu_packed(one, one, None, one, one, 8, 2048, 512, 8, _lib.BF16, None) == -1
     # group selection
     assert lib.trimkv_group_threshold(one, one, None, one, 1, 8, 3, 64, 128, _lib.BF16, _lib.F32, 10, 0, 0.0, 5, 0, 1,
                                       one, one, one, one, None, None) == -2  # 3 does not divide 8

@@ -234,3 +234,52 @@ def test_gated_append_attend_refuses_more_than_64_slices():
     pieces = lambda nslice: lib.trimkv_append_attend_pieces_gated(one, one, one, one, one, one, one, None, one, 4, 8, 2, 64, 128, 4, L.BF16, L.BF16,
                                                                   one, one, 256, 128, one, nslice, one, one, 0, 0, 0.1, 64, one, 1 << 20, None)
     assert pieces(65) == -6
+
+
+@pytest.mark.parametrize("kind,hidden,ntok,dtype", [("rg", 4096, 64, torch.bfloat16), ("rg", 2560, 200, torch.bfloat16), ("rg", 512, 1, torch.float16),
+                                                      ("rg3", 2048, 64, torch.bfloat16), ("rg3", 1024, 256, torch.float16)])
+def test_packed_first_layer_weights_give_the_same_bits(kind, hidden, ntok, dtype):
+    """trimkv_gate_pack_weights + trimkv_gate_hidden(_swiglu)_packed against the row-major entry points through the C ABI:
+    the same partial sums bit for bit (only the addresses of the loads differ); the modules keep their packed copies in
+    step with the parameters."""
+    from trimkv_amd import _lib as L
+    lib = L.load()
+    inter, heads = 96, 4
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    rnd = lambda *s: (torch.randn(*s, generator=gen, device=DEV) * 0.05).to(dtype)
+    x = (torch.randn(ntok, hidden, generator=gen, device=DEV)).to(dtype)
+    w1, wu, b1, w2 = rnd(inter, hidden), rnd(inter, hidden), rnd(inter), rnd(heads, inter)
+    nsl = lib.trimkv_gate_slices(inter)
+    plain = torch.zeros(nsl, ntok, heads, device=DEV)
+    packed = torch.ones(nsl, ntok, heads, device=DEV)
+    w1p, wup = torch.empty_like(w1), torch.empty_like(wu)
+    code, st = L.dtype_code(dtype), L.current_stream(torch.device(DEV))
+    for src, dst in ((w1, w1p), (wu, wup)):
+        L.check(lib.trimkv_gate_pack_weights(src.data_ptr(), dst.data_ptr(), hidden, inter, code, st), "pack")
+    assert torch.equal(w1p.view(-1).sort().values, w1.view(-1).sort().values)       # a permutation of the matrix
+    if kind == "rg":
+        L.check(lib.trimkv_gate_hidden(x.data_ptr(), w1.data_ptr(), b1.data_ptr(), w2.data_ptr(), plain.data_ptr(), ntok, hidden, inter, heads, code, st), "plain")
+        L.check(lib.trimkv_gate_hidden_packed(x.data_ptr(), w1p.data_ptr(), b1.data_ptr(), w2.data_ptr(), packed.data_ptr(), ntok, hidden, inter, heads, code, st), "packed")
+    else:
+        L.check(lib.trimkv_gate_hidden_swiglu(x.data_ptr(), w1.data_ptr(), wu.data_ptr(), w2.data_ptr(), plain.data_ptr(), ntok, hidden, inter, heads, code, st), "plain")
+        L.check(lib.trimkv_gate_hidden_swiglu_packed(x.data_ptr(), w1p.data_ptr(), wup.data_ptr(), w2.data_ptr(), packed.data_ptr(), ntok, hidden, inter, heads, code, st), "packed")
+    torch.cuda.synchronize()
+    assert plain.abs().max() > 0 and torch.equal(plain, packed)
+    # more tokens than the packed kernel serves, packing in place
+    assert lib.trimkv_gate_hidden_packed(x.data_ptr(), w1p.data_ptr(), b1.data_ptr(), w2.data_ptr(), packed.data_ptr(), 257, hidden, inter, heads, code, st) == -6
+    assert lib.trimkv_gate_pack_weights(w1.data_ptr(), w1.data_ptr(), hidden, inter, code, st) == -2
+
+
+def test_gate_module_repacks_when_its_weights_change():
+    g = _gate(1024, 4, inter=64).to(DEV)
+    x = torch.randn(2, 1, 1024, device=DEV).to(torch.bfloat16)
+    a = g(x).materialize()
+    first = g._packed_w["w1"][1]
+    assert g(x).materialize().equal(a) and g._packed_w["w1"][1] is first          # cached
+    with torch.no_grad():
+        g.linear1.weight.mul_(0.5)                                                  # in place: the version counter moves
+    b = g(x).materialize()
+    assert g._packed_w["w1"][1] is not first
+    g.fused = False
+    want = g(x)                                                                     # the torch expression on the new weights
+    assert not torch.equal(a, b) and (b.float() - want.float()).abs().max() <= 3e-2 * want.float().abs().max() + 2e-3

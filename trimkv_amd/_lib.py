@@ -31,6 +31,9 @@ SIGNATURES = {
     "trimkv_gate_slices": (_i, [_i]),
     "trimkv_gate_hidden": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "trimkv_gate_hidden_swiglu": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "trimkv_gate_pack_weights": (_i, [_p, _p, _i, _i, _i, _p]),
+    "trimkv_gate_hidden_packed": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
+    "trimkv_gate_hidden_swiglu_packed": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "trimkv_append_gated": (_i, [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _p, _p, _i64, _i64, _i64,
                                  _p, _i, _p, _p, _i64, _i64, _i64, _i, _i, _p]),
     "trimkv_evict_workspace": (_sz, [_i, _i]),

@@ -6,8 +6,9 @@ Mirrors the reference's ``RetentionGate`` (src/trimkv/models/qwen3/modeling_trim
 parameter names match, so a reference checkpoint's gate weights load unchanged.
 
 On the GPU in eval mode ``forward`` launches ``trimkv_gate_hidden`` (MFMA first linear, SiLU,
-per-slice partial second linear) and returns a :class:`LazyLogBeta`; ``cache.update`` finishes it
-inside the append kernel.  Anywhere else (training, CPU, other activations) it is the plain torch
+per-slice partial second linear; decode-sized calls read the first-layer weights from a copy packed
+once in the kernel's operand order, ``trimkv_gate_hidden_packed``) and returns a :class:`LazyLogBeta`;
+``cache.update`` finishes it inside the append kernel.  Anywhere else (training, CPU, other activations) it is the plain torch
 expression.
 
 ``RetentionGate2`` (:182-224) is the same network on ``concat(K, V)`` after RoPE, all KV heads side by side
@@ -60,12 +61,34 @@ class RetentionGate(nn.Module):
             self._bias32, self._bias_version = bias32, self.bias._version
         return bias32
 
+    # Decode-sized calls (up to this many tokens) read the first-layer weights from a copy stored in the order the kernel's
+    # lanes want them (trimkv_gate_pack_weights): 1 KiB contiguous per load instruction instead of 16 rows x 64 bytes.
+    packed_max_tokens = 256
+
+    def _packed(self, lib, name: str, w: torch.Tensor) -> torch.Tensor:
+        """The packed copy of first-layer weight ``w``, rebuilt when the parameter has changed or moved."""
+        cache = self.__dict__.setdefault("_packed_w", {})
+        key = (w.data_ptr(), w._version, w.dtype, w.device)
+        hit = cache.get(name)
+        if hit is None or hit[0] != key:
+            src = w.detach()
+            if not src.is_contiguous():
+                src = src.contiguous()
+            packed = torch.empty_like(src)
+            rc = lib.trimkv_gate_pack_weights(src.data_ptr(), packed.data_ptr(), src.shape[1], src.shape[0], _lib.dtype_code(src.dtype),
+                                         _lib.current_stream(src.device))
+            _lib.check(rc, "trimkv_gate_pack_weights")
+            hit = cache[name] = (key, packed)
+        return hit[1]
+
     def _launch(self, lib, x2, part, ntok, hidden) -> None:
         w1, b1, w2 = self.linear1.weight, self.linear1.bias, self.linear2.weight
-        rc = lib.trimkv_gate_hidden(x2.data_ptr(), w1.data_ptr(), b1.data_ptr(), w2.data_ptr(), part.data_ptr(), ntok, hidden,
-                                    self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.dtype_code(x2.dtype),
-                                    _lib.current_stream(x2.device))
-        _lib.check(rc, "trimkv_gate_hidden")
+        args = (b1.data_ptr(), w2.data_ptr(), part.data_ptr(), ntok, hidden, self.retention_gate_intermediate_size,
+                self.num_key_value_heads, _lib.dtype_code(x2.dtype), _lib.current_stream(x2.device))
+        if ntok <= self.packed_max_tokens:
+            _lib.check(lib.trimkv_gate_hidden_packed(x2.data_ptr(), self._packed(lib, "w1", w1).data_ptr(), *args), "trimkv_gate_hidden_packed")
+        else:
+            _lib.check(lib.trimkv_gate_hidden(x2.data_ptr(), w1.data_ptr(), *args), "trimkv_gate_hidden")
 
     def forward(self, x: torch.Tensor):
         """x [B, S, hidden] -> log beta [B, S, Hkv] (a LazyLogBeta on the fused path)."""
@@ -135,11 +158,14 @@ class RetentionGate3(RetentionGate):
         return F.logsigmoid(self.down_proj(act(self.gate_proj(x)) * self.up_proj(x)) + self.bias)
 
     def _launch(self, lib, x2, part, ntok, hidden) -> None:
-        rc = lib.trimkv_gate_hidden_swiglu(x2.data_ptr(), self.gate_proj.weight.data_ptr(), self.up_proj.weight.data_ptr(),
-                                           self.down_proj.weight.data_ptr(), part.data_ptr(), ntok, hidden,
-                                           self.retention_gate_intermediate_size, self.num_key_value_heads, _lib.dtype_code(x2.dtype),
-                                           _lib.current_stream(x2.device))
-        _lib.check(rc, "trimkv_gate_hidden_swiglu")
+        args = (self.down_proj.weight.data_ptr(), part.data_ptr(), ntok, hidden, self.retention_gate_intermediate_size,
+                self.num_key_value_heads, _lib.dtype_code(x2.dtype), _lib.current_stream(x2.device))
+        wg, wu = self.gate_proj.weight, self.up_proj.weight
+        if ntok <= self.packed_max_tokens:
+            _lib.check(lib.trimkv_gate_hidden_swiglu_packed(x2.data_ptr(), self._packed(lib, "gate", wg).data_ptr(),
+                                                            self._packed(lib, "up", wu).data_ptr(), *args), "trimkv_gate_hidden_swiglu_packed")
+        else:
+            _lib.check(lib.trimkv_gate_hidden_swiglu(x2.data_ptr(), wg.data_ptr(), wu.data_ptr(), *args), "trimkv_gate_hidden_swiglu")
 
     def forward(self, x: torch.Tensor, transpose: bool = True):
         return super().forward(_heads_side_by_side(x, transpose))
