@@ -556,6 +556,34 @@ int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_stride_h, i
                         int batch, int kv_heads, int group, int q_len, int cap, int head_dim, int dtype, float scale,
                         int max_len, void* stream);
 
+/*
+ * trimkv_rmsnorm / trimkv_qk_norm_rope / trimkv_silu_mul -- the element-wise work of a decoder layer around the cache
+ * path, one launch each (a module-by-module decoder issues 5-16 small launches for each, and a decode step is bound
+ * by their number).  dtype: TRIMKV_BF16 or TRIMKV_F16; every intermediate is rounded where the torch modules round it.
+ *
+ * trimkv_rmsnorm (Qwen3RMSNorm, src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:89-103): out[t] = weight * round(h *
+ * rsqrt(mean(h^2) + eps)), h = fp32(x[t]); x rows x_stride elements apart, out [ntok][hidden].  With `residual`
+ * (rows residual_stride apart) h = fp32(round(x[t] + residual[t])) and that sum is written to sum_out [ntok][hidden]:
+ * the residual add in front of the norm (:431-435) in the same launch.  residual and sum_out are both given or both
+ * NULL; sum_out may be x or residual itself.  hidden and the strides are multiples of 8, all pointers 16-byte aligned.
+ *
+ * trimkv_qk_norm_rope (:328-329 and apply_rotary_pos_emb :125-151): q [batch*seq][q_heads][head_dim] with rows
+ * q_tok_stride elements apart (likewise k with kv_heads: slices of one fused projection are fine), optional per-head
+ * RMS-norm weights [head_dim] (both or neither), cos/sin [batch or 1][seq][rotary_dim] (cs_batch_stride 0 = shared by
+ * the batch), rotation of the first rotary_dim (even) features, the rest passed through; q_out [batch][q_heads][seq]
+ * [head_dim], k_out [batch][kv_heads][seq][head_dim].  head_dim <= 128.
+ *
+ * trimkv_silu_mul (Qwen3MLP :121): out[t][i] = round(silu(gate[t][i])) * up[t][i], rows gate_stride / up_stride
+ * elements apart (halves of one fused projection are fine), out [ntok][inter]; inter and strides multiples of 8.
+ */
+int trimkv_rmsnorm(const void* x, int64_t x_stride, const void* residual, int64_t residual_stride, const void* weight,
+                   void* out, void* sum_out, int ntok, int hidden, float eps, int dtype, void* stream);
+int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* q_weight, const void* k_weight,
+                        const void* cos, const void* sin, int64_t cs_batch_stride, void* q_out, void* k_out,
+                        int batch, int seq, int q_heads, int kv_heads, int head_dim, int rotary_dim, float eps, int dtype, void* stream);
+int trimkv_silu_mul(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
+                    int ntok, int inter, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,182 @@
+"""The fused element-wise launches of the decoder shells (trimkv_rmsnorm, trimkv_qk_norm_rope, trimkv_silu_mul) against
+the torch expressions they replace (reference: Qwen3RMSNorm, apply_rotary_pos_emb, Qwen3MLP,
+src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:89-151, 328-329, 431-437).  They round where the 16-bit torch modules
+round but sum in another order, so the comparison allows one unit in the last place of the 16-bit result (two where two
+rounded terms are added), and pins the mathematics against a float64 evaluation."""
+import pytest
+import torch
+
+from tests.gpu_util import DEV
+
+pytestmark = pytest.mark.gpu
+
+
+def _ulp(x: torch.Tensor, dtype) -> torch.Tensor:
+    """One unit in the last place of ``dtype`` at the magnitude of ``x`` (fp32 tensor)."""
+    bits = 8 if dtype == torch.bfloat16 else 11
+    return torch.clamp(x.abs(), min=2.0 ** -14).log2().floor().exp2() * 2.0 ** (1 - bits)
+
+
+def _torch_rmsnorm(x, w, eps):
+    h = x.float()
+    h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + eps)
+    return w * h.to(x.dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("ntok,hidden", [(64, 4096), (5, 2560), (300, 128), (1, 8)])
+def test_rmsnorm(dtype, ntok, hidden):
+    from trimkv_amd import decoder_ops
+    gen = torch.Generator(device=DEV).manual_seed(0)
+    x = (torch.randn(ntok, hidden, generator=gen, device=DEV) * 3).to(dtype)
+    w = (1 + 0.2 * torch.randn(hidden, generator=gen, device=DEV)).to(dtype)
+    got = decoder_ops.rmsnorm(x, w, 1e-6)
+    want = _torch_rmsnorm(x, w, 1e-6)
+    assert got.shape == want.shape and got.dtype == dtype
+    assert ((got.float() - want.float()).abs() <= _ulp(want.float(), dtype)).all()
+    assert (got != want).float().mean() < 0.02                      # the two differ only where a rounding tipped
+    x64 = x.double()
+    exact = w.double() * x64 * torch.rsqrt(x64.pow(2).mean(-1, keepdim=True) + 1e-6)
+    assert ((got.double() - exact).abs() <= 2.5 * _ulp(exact.float(), dtype).double()).all()
+    # rows that are not densely packed (a slice of a wider tensor)
+    wide = torch.zeros(ntok, hidden + 16, dtype=dtype, device=DEV)
+    wide[:, :hidden] = x
+    assert torch.equal(decoder_ops.rmsnorm(wide[:, :hidden], w, 1e-6), got)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_rmsnorm_with_the_residual_add(dtype):
+    from trimkv_amd import decoder_ops
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    x = torch.randn(3, 7, 1024, generator=gen, device=DEV).to(dtype)
+    r = (torch.randn(3, 7, 1024, generator=gen, device=DEV) * 4).to(dtype)
+    w = (1 + 0.2 * torch.randn(1024, generator=gen, device=DEV)).to(dtype)
+    got, total = decoder_ops.rmsnorm(x, w, 1e-5, r)
+    assert torch.equal(total, r + x)                                # the sum is element-wise: bit for bit
+    assert torch.equal(got, decoder_ops.rmsnorm(total, w, 1e-5))    # and the norm is the plain launch on it
+    want = _torch_rmsnorm(r + x, w, 1e-5)
+    assert ((got.float() - want.float()).abs() <= _ulp(want.float(), dtype)).all()
+
+
+def _torch_qk(q, k, qw, kw, cos, sin, eps):
+    from trimkv_amd.qwen3 import apply_rope
+    if qw is not None:
+        q, k = _torch_rmsnorm(q, qw, eps), _torch_rmsnorm(k, kw, eps)
+    return apply_rope(q.transpose(1, 2), cos, sin), apply_rope(k.transpose(1, 2), cos, sin)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,Hq,Hkv,D,R,norm,fused,per_batch", [
+    (64, 1, 32, 8, 128, 128, True, False, False),     # Qwen3-8B decode step
+    (2, 37, 8, 2, 128, 128, True, False, True),       # a prompt, positions per batch element
+    (3, 5, 6, 2, 128, 96, False, True, False),        # Phi-3: fused qkv projection, rotary on 3/4 of the features, no head norms
+    (2, 9, 4, 4, 96, 96, False, True, False),         # Phi-3-mini heads
+    (2, 3, 4, 2, 64, 64, True, False, False),
+    (1, 4, 2, 1, 128, 0, True, False, False),         # no rotation at all
+])
+def test_qk_norm_rope(dtype, B, S, Hq, Hkv, D, R, norm, fused, per_batch):
+    from trimkv_amd import decoder_ops
+    from trimkv_amd.qwen3 import rotary_tables
+    gen = torch.Generator(device=DEV).manual_seed(2)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device=DEV)
+    if fused:                                                       # q | k | v side by side in one projection output
+        qkv = (rnd(B, S, (Hq + 2 * Hkv) * D) * 2).to(dtype)
+        q, k, _ = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        q, k = q.view(B, S, Hq, D), k.view(B, S, Hkv, D)
+    else:
+        q, k = (rnd(B, S, Hq, D) * 2).to(dtype), (rnd(B, S, Hkv, D) * 2).to(dtype)
+    qw = (1 + 0.2 * rnd(D)).to(dtype) if norm else None
+    kw = (1 + 0.2 * rnd(D)).to(dtype) if norm else None
+    pos = torch.randint(0, 5000, (B if per_batch else 1, S), generator=gen, device=DEV)
+    if R:
+        cos, sin = rotary_tables(pos, D, 10000.0, dtype, R)
+    else:
+        cos = sin = torch.zeros(pos.shape[0], S, 0, dtype=dtype, device=DEV)
+    assert decoder_ops.qk_norm_rope_ok(q, k, cos, sin)
+    gq, gk = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, 1e-6)
+    if R:
+        wq, wk = _torch_qk(q, k, qw, kw, cos, sin, 1e-6)
+    else:
+        wq, wk = (_torch_rmsnorm(q, qw, 1e-6).transpose(1, 2), _torch_rmsnorm(k, kw, 1e-6).transpose(1, 2))
+    for got, want, H in ((gq, wq, Hq), (gk, wk, Hkv)):
+        assert got.shape == (B, H, S, D) and got.is_contiguous()
+        # a rotated feature is the sum of two rounded products, each within one unit of the torch module's
+        tol = 2 * _ulp(want.float(), dtype) + 2 * _ulp(torch.full_like(want.float(), 4.0), dtype) * norm
+        assert ((got.float() - want.float()).abs() <= tol).all(), float((got.float() - want.float()).abs().max())
+        assert (got != want).float().mean() < (0.05 if norm else 1e-9)   # without a norm nothing is summed: bit for bit
+    # float64: norm, then the rotation by the angle the tables encode
+    if R == D and norm:
+        q64 = q.double()
+        y = qw.double() * q64 * torch.rsqrt(q64.pow(2).mean(-1, keepdim=True) + 1e-6)
+        c, s_ = cos.double()[:, :, None, :], sin.double()[:, :, None, :]
+        rot = torch.cat([-y[..., D // 2:], y[..., :D // 2]], dim=-1)
+        exact = (y * c + rot * s_).transpose(1, 2)
+        assert (gq.double() - exact).abs().max() <= 0.05 * exact.abs().max()
+        assert (gq.double() - exact).abs().mean() <= 4e-3 * exact.abs().mean() * (8 if dtype == torch.bfloat16 else 1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_silu_mul(dtype):
+    from trimkv_amd import decoder_ops
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    g = (torch.randn(5, 3, 1536, generator=gen, device=DEV) * 3).to(dtype)
+    u = torch.randn(5, 3, 1536, generator=gen, device=DEV).to(dtype)
+    assert decoder_ops.silu_mul_ok(g, u)
+    got = decoder_ops.silu_mul(g, u)
+    want = torch.nn.functional.silu(g) * u
+    assert ((got.float() - want.float()).abs() <= _ulp(want.float(), dtype)).all()
+    assert (got != want).float().mean() < 0.01
+    exact = (g.double() * torch.sigmoid(g.double())) * u.double()
+    assert ((got.double() - exact).abs() <= 2.5 * _ulp(exact.float(), dtype).double()).all()
+    # the two halves of one fused projection (Phi-3's gate_up_proj)
+    both = torch.cat([g, u], dim=-1)
+    a, b = both.chunk(2, dim=-1)
+    assert decoder_ops.silu_mul_ok(a, b) and torch.equal(decoder_ops.silu_mul(a, b), got)
+    assert not decoder_ops.silu_mul_ok(g[..., :100], u[..., :100])
+
+
+@pytest.mark.parametrize("family", ["qwen3", "llama", "phi3", "phi3mini"])
+def test_decoder_with_and_without_the_fused_launches(family):
+    """The same model and tokens with the fused element-wise launches on and off: logits agree to 16-bit rounding noise,
+    and the fused path really runs fewer launches."""
+    from trimkv_amd import decoder_ops
+    from tests.test_gpu_qwen3_shell import _family, _tiny_config
+    cfg = _tiny_config(family, retention_gate="rg")
+    torch.manual_seed(0)
+    model = _family(family)[1](cfg).to(torch.bfloat16).to(DEV).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 40), generator=torch.Generator().manual_seed(4)).to(DEV)
+
+    def run():
+        with torch.no_grad():
+            out = model(ids[:, :30])
+            logits = [out.logits[:, -1]]
+            for i in range(30, 40):
+                out = model(ids[:, i:i + 1], past_key_values=out.past_key_values)
+                logits.append(out.logits[:, -1])
+        return torch.stack(logits).float()
+
+    assert decoder_ops.enabled
+    fused = run()
+    decoder_ops.enabled = False
+    try:
+        plain = run()
+    finally:
+        decoder_ops.enabled = True
+    assert (fused - plain).abs().max() <= 2e-2 + 2e-2 * plain.abs().max(), float((fused - plain).abs().max())
+
+
+def test_the_fused_launches_stay_out_of_training_and_cpu():
+    from trimkv_amd import decoder_ops
+    from trimkv_amd.qwen3 import RMSNorm
+    norm = RMSNorm(64, 1e-6).to(torch.bfloat16)
+    x = torch.randn(2, 64).to(torch.bfloat16)
+    assert not decoder_ops.usable(x, norm.weight)                   # CPU
+    norm, x = norm.to(DEV), x.to(DEV)
+    assert not decoder_ops.usable(x, norm.weight)                   # the weight wants a gradient
+    y = norm(x)
+    y.float().sum().backward()
+    assert norm.weight.grad is not None
+    with torch.no_grad():
+        assert decoder_ops.usable(x, norm.weight)
+        assert ((norm(x).float() - y.float()).abs() <= _ulp(y.float(), torch.bfloat16)).all()
+    assert not decoder_ops.usable(x.float(), norm.weight.float())   # fp32

@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 LIB_PATH = os.path.join(HERE, "libtrimkv_hip.so")
-SOURCES = ["api.hip", "append.hip", "evict.hip", "attn_decode.hip", "attn_decode_append.hip", "attn_decode_pieces.hip", "attn_decode_append_pieces.hip", "attn_decode_append_gated.hip", "attn_decode_append_pieces_gated.hip", "pieces_plan.hip", "attn_prefill.hip", "gate.hip", "stream_probe.hip"]
+SOURCES = ["api.hip", "append.hip", "evict.hip", "attn_decode.hip", "attn_decode_append.hip", "attn_decode_pieces.hip", "attn_decode_append_pieces.hip", "attn_decode_append_gated.hip", "attn_decode_append_pieces_gated.hip", "pieces_plan.hip", "attn_prefill.hip", "gate.hip", "stream_probe.hip", "decoder_ops.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + INCLUDE, "-I" + CSRC,

@@ -1,0 +1,107 @@
+"""The element-wise work of a decoder layer around the cache path on one HIP launch each: RMS norm (optionally with the
+residual add in front of it), per-head q/k norm + RoPE, SiLU-gated product.  A module-by-module decoder issues 5-16 small
+launches for each of them (reference: Qwen3RMSNorm, apply_rotary_pos_emb and Qwen3MLP,
+src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:89-151, 328-329, 431-437), and a decode step is bound by the number of
+launches.  Inference on the GPU in bf16/fp16 only: the callers in ``qwen3.py`` keep the torch expressions for everything
+else (training, CPU, fp32), and ``enabled = False`` switches these launches off altogether.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+enabled = True
+
+
+def usable(*tensors: Optional[torch.Tensor]) -> bool:
+    """Whether the fused launches can stand in for the torch expressions on these tensors."""
+    if not enabled:
+        return False
+    first = tensors[0]
+    if not first.is_cuda or first.dtype not in (torch.bfloat16, torch.float16):
+        return False
+    grad = torch.is_grad_enabled()
+    for t in tensors:
+        if t is None:
+            continue
+        if t.dtype != first.dtype or t.device != first.device or (grad and t.requires_grad):
+            return False
+    return True
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None):
+    """``weight * norm(x)`` over the last axis; with ``residual`` returns ``(weight * norm(x + residual), x + residual)``."""
+    hidden = x.shape[-1]
+    x2 = x.reshape(-1, hidden)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    out = torch.empty(x2.shape, dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    if residual is None:
+        rc = lib.trimkv_rmsnorm(x2.data_ptr(), x2.stride(0), None, 0, weight.data_ptr(), out.data_ptr(), None, x2.shape[0], hidden,
+                                float(eps), _lib.dtype_code(x.dtype), _lib.current_stream(x.device))
+        _lib.check(rc, "trimkv_rmsnorm")
+        return out.view(x.shape)
+    r2 = residual.reshape(-1, hidden)
+    if r2.stride(1) != 1 or r2.stride(0) % 8 or r2.data_ptr() % 16:
+        r2 = r2.contiguous()
+    total = torch.empty(x2.shape, dtype=x.dtype, device=x.device)
+    rc = lib.trimkv_rmsnorm(x2.data_ptr(), x2.stride(0), r2.data_ptr(), r2.stride(0), weight.data_ptr(), out.data_ptr(), total.data_ptr(),
+                            x2.shape[0], hidden, float(eps), _lib.dtype_code(x.dtype), _lib.current_stream(x.device))
+    _lib.check(rc, "trimkv_rmsnorm")
+    return out.view(x.shape), total.view(x.shape)
+
+
+def qk_norm_rope_ok(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> bool:
+    """q, k [B, S, H, D] views of projection outputs (D contiguous, heads D apart, batch = S tokens apart), cos/sin
+    [1 or B, S, R] contiguous with R even."""
+    B, S, _, D = q.shape
+    if D > 128 or cos.dim() != 3 or cos.shape != sin.shape or cos.shape[1] != S or cos.shape[0] not in (1, B):
+        return False
+    if cos.shape[2] % 2 or cos.shape[2] > D or not cos.is_contiguous() or not sin.is_contiguous() or cos.dtype != q.dtype:
+        return False
+    for t in (q, k):
+        if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != S * t.stride(1):
+            return False
+    return True
+
+
+def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
+                 cos: torch.Tensor, sin: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [B,S,Hq,D], k [B,S,Hkv,D] -> RMS-normed per head (when weights are given) and rotated, as [B,Hq,S,D], [B,Hkv,S,D]."""
+    B, S, Hq, D = q.shape
+    Hkv = k.shape[2]
+    q_out = torch.empty(B, Hq, S, D, dtype=q.dtype, device=q.device)
+    k_out = torch.empty(B, Hkv, S, D, dtype=q.dtype, device=q.device)
+    rc = _lib.load().trimkv_qk_norm_rope(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), _lib.ptr(q_weight), _lib.ptr(k_weight),
+                                         cos.data_ptr(), sin.data_ptr(), 0 if cos.shape[0] == 1 else cos.stride(0), q_out.data_ptr(), k_out.data_ptr(),
+                                         B, S, Hq, Hkv, D, cos.shape[2], float(eps), _lib.dtype_code(q.dtype), _lib.current_stream(q.device))
+    _lib.check(rc, "trimkv_qk_norm_rope")
+    return q_out, k_out
+
+
+def silu_mul_ok(gate: torch.Tensor, up: torch.Tensor) -> bool:
+    inter = gate.shape[-1]
+    if gate.shape != up.shape or inter % 8:
+        return False
+    for t in (gate, up):
+        if t.stride(-1) != 1 or t.data_ptr() % 16:
+            return False
+        rows = t.reshape(-1, inter) if t.dim() != 2 else t
+        if rows.stride(1) != 1 or rows.stride(0) % 8 or rows.data_ptr() != t.data_ptr():    # reshape had to copy: rows are not evenly spaced
+            return False
+    return True
+
+
+def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` over tensors whose rows are evenly spaced (halves of one fused projection are fine)."""
+    inter = gate.shape[-1]
+    g2, u2 = gate.reshape(-1, inter), up.reshape(-1, inter)
+    out = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    rc = _lib.load().trimkv_silu_mul(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), out.data_ptr(), g2.shape[0], inter,
+                                     _lib.dtype_code(gate.dtype), _lib.current_stream(gate.device))
+    _lib.check(rc, "trimkv_silu_mul")
+    return out

@@ -41,11 +41,7 @@ class TrimKVLlamaAttention(TrimKVQwen3Attention):
         self.v_proj = nn.Linear(hs, config.num_key_value_heads * d, bias=config.attention_bias)
         self.o_proj = nn.Linear(config.num_attention_heads * d, hs, bias=config.attention_bias)
 
-    def _qkv(self, hidden_states: torch.Tensor):
-        B, S, _ = hidden_states.shape
-        shape = (B, S, -1, self.head_dim)
-        return (self.q_proj(hidden_states).view(shape).transpose(1, 2), self.k_proj(hidden_states).view(shape).transpose(1, 2),
-                self.v_proj(hidden_states).view(shape).transpose(1, 2))
+    # no q_norm / k_norm modules: the base class's _head_norms() finds none, _qkv_rope() only rotates
 
 
 class TrimKVLlamaDecoderLayer(TrimKVQwen3DecoderLayer):

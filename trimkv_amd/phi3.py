@@ -14,6 +14,7 @@ import torch
 from torch import nn
 import torch.nn.functional as F
 
+from . import decoder_ops
 from .qwen3 import (TrimKVQwen3Attention, TrimKVQwen3Config, TrimKVQwen3DecoderLayer, TrimKVQwen3ForCausalLM, TrimKVQwen3Model)
 
 
@@ -44,6 +45,8 @@ class Phi3MLP(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         gate, up = self.gate_up_proj(x).chunk(2, dim=-1)
+        if decoder_ops.usable(gate, up) and decoder_ops.silu_mul_ok(gate, up):
+            return self.down_proj(decoder_ops.silu_mul(gate, up))
         return self.down_proj(up * F.silu(gate))
 
 
@@ -56,12 +59,12 @@ class TrimKVPhi3Attention(TrimKVQwen3Attention):
         self.qkv_proj = nn.Linear(config.hidden_size, (self.num_heads + 2 * self.num_key_value_heads) * d, bias=False)
         self.o_proj = nn.Linear(self.num_heads * d, config.hidden_size, bias=False)
 
-    def _qkv(self, hidden_states: torch.Tensor):
+    def _projections(self, hidden_states: torch.Tensor):
         B, S, _ = hidden_states.shape
         d = self.head_dim
         q, k, v = self.qkv_proj(hidden_states).split([self.num_heads * d, self.num_key_value_heads * d, self.num_key_value_heads * d], dim=-1)
         shape = (B, S, -1, d)
-        return q.view(shape).transpose(1, 2), k.view(shape).transpose(1, 2), v.view(shape).transpose(1, 2)
+        return q.view(shape), k.view(shape), v.view(shape)
 
 
 class TrimKVPhi3DecoderLayer(TrimKVQwen3DecoderLayer):

@@ -24,6 +24,7 @@ import torch
 from torch import nn
 import torch.nn.functional as F
 
+from . import decoder_ops
 from .attn import get_attention_interface
 from .cache_utils import LazyLogBeta, TrimKVCache
 from .gate import RetentionGate, RetentionGate2, RetentionGate3
@@ -85,9 +86,18 @@ class RMSNorm(nn.Module):
         self.variance_epsilon = eps
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if decoder_ops.usable(x, self.weight) and x.shape[-1] % 8 == 0:
+            return decoder_ops.rmsnorm(x, self.weight, self.variance_epsilon)      # one launch instead of eight
         h = x.float()
         h = h * torch.rsqrt(h.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
         return self.weight * h.to(x.dtype)
+
+    def add_norm(self, x: torch.Tensor, residual: torch.Tensor):
+        """``(norm(x + residual), x + residual)``: the residual add in front of a norm (qwen3:431-435), in the norm's launch."""
+        if decoder_ops.usable(x, residual, self.weight) and x.shape[-1] % 8 == 0 and x.shape == residual.shape:
+            return decoder_ops.rmsnorm(x, self.weight, self.variance_epsilon, residual)
+        total = residual + x
+        return self.forward(total), total
 
 
 class MLP(nn.Module):
@@ -99,7 +109,10 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=bias)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+        gate, up = self.gate_proj(x), self.up_proj(x)
+        if decoder_ops.usable(gate, up) and decoder_ops.silu_mul_ok(gate, up):
+            return self.down_proj(decoder_ops.silu_mul(gate, up))
+        return self.down_proj(F.silu(gate) * up)
 
 
 def rotary_tables(position_ids: torch.Tensor, head_dim: int, theta: float, dtype: torch.dtype,
@@ -180,14 +193,28 @@ class TrimKVQwen3Attention(nn.Module):
             return RetentionGate(config.hidden_size, *common)
         return (RetentionGate2 if kind == "rg2" else RetentionGate3)(config.head_dim, *common)
 
-    def _qkv(self, hidden_states: torch.Tensor):
-        """q [B,Hq,S,D], k and v [B,Hkv,S,D] before RoPE (qwen3:326-328, 335-337: per-head RMS norm on q and k)."""
+    def _projections(self, hidden_states: torch.Tensor):
+        """The outputs of the q, k and v projections as [B,S,H,D] views (qwen3:326-328), before any norm."""
         B, S, _ = hidden_states.shape
         shape = (B, S, -1, self.head_dim)
-        q = self.q_norm(self.q_proj(hidden_states).view(shape)).transpose(1, 2)
-        k = self.k_norm(self.k_proj(hidden_states).view(shape)).transpose(1, 2)
-        v = self.v_proj(hidden_states).view(shape).transpose(1, 2)
-        return q, k, v
+        return self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape), self.v_proj(hidden_states).view(shape)
+
+    def _head_norms(self):
+        """The per-head RMS norms of q and k (qwen3:328-329), or (None, None) for a family without them."""
+        return getattr(self, "q_norm", None), getattr(self, "k_norm", None)
+
+    def _qkv_rope(self, hidden_states: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
+        """q [B,Hq,S,D] and k [B,Hkv,S,D] after the per-head norm and RoPE, v [B,Hkv,S,D] (qwen3:326-337, 341-343).  On the GPU
+        at inference norm and rotation of q and k are one launch (trimkv_qk_norm_rope)."""
+        q, k, v = self._projections(hidden_states)
+        qn, kn = self._head_norms()
+        qw, kw = (None, None) if qn is None else (qn.weight, kn.weight)
+        if decoder_ops.usable(q, k, cos, sin, qw, kw) and decoder_ops.qk_norm_rope_ok(q, k, cos, sin):
+            q, k = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps)
+            return q, k, v.transpose(1, 2)
+        if qn is not None:
+            q, k = qn(q), kn(k)
+        return apply_rope(q.transpose(1, 2), cos, sin), apply_rope(k.transpose(1, 2), cos, sin), v.transpose(1, 2)
 
     # `rg` depends on nothing but the normed hidden state, as the q/k/v projections do.  With this flag its first linear
     # (trimkv_gate_hidden) is issued on a second stream of the same priority and joined by an event before update(), so that
@@ -226,9 +253,8 @@ class TrimKVQwen3Attention(nn.Module):
             else:
                 retention = self.retention_gate(hidden_states)
             retention = retention.transpose(1, 2)
-        q, k, v = self._qkv(hidden_states)
         cos, sin = position_embeddings
-        q, k = apply_rope(q, cos, sin), apply_rope(k, cos, sin)
+        q, k, v = self._qkv_rope(hidden_states, cos, sin)
         if self.config.retention_gate in ("rg2", "rg3"):   # these see concat(K, V) after RoPE (qwen3:345-347)
             retention = self.retention_gate(torch.cat([k, v], dim=-1)).transpose(1, 2)
         offset = past_key_values.get_seq_length(self.layer_idx)
@@ -255,9 +281,9 @@ class TrimKVQwen3DecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
     def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
-        hidden_states = hidden_states + self.self_attn(self.input_layernorm(hidden_states), position_embeddings, attention_mask,
-                                                       past_key_values, cache_position)
-        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+        attn_out = self.self_attn(self.input_layernorm(hidden_states), position_embeddings, attention_mask, past_key_values, cache_position)
+        normed, hidden_states = self.post_attention_layernorm.add_norm(attn_out, hidden_states)   # qwen3:431-435
+        return hidden_states + self.mlp(normed)
 
 
 class TrimKVQwen3Model(nn.Module):
