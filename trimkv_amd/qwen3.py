@@ -280,10 +280,16 @@ class TrimKVQwen3DecoderLayer(nn.Module):
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
-    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position):
-        attn_out = self.self_attn(self.input_layernorm(hidden_states), position_embeddings, attention_mask, past_key_values, cache_position)
+    def forward(self, hidden_states, position_embeddings, attention_mask, past_key_values, cache_position, pending=None):
+        """``pending``: the MLP output of the layer below, not yet added to ``hidden_states`` -- the add (qwen3:437) then rides
+        in this layer's first norm.  Returns ``(hidden_states, mlp_out)`` with the same add left to whoever comes next."""
+        if pending is None:
+            normed = self.input_layernorm(hidden_states)
+        else:
+            normed, hidden_states = self.input_layernorm.add_norm(pending, hidden_states)
+        attn_out = self.self_attn(normed, position_embeddings, attention_mask, past_key_values, cache_position)
         normed, hidden_states = self.post_attention_layernorm.add_norm(attn_out, hidden_states)   # qwen3:431-435
-        return hidden_states + self.mlp(normed)
+        return hidden_states, self.mlp(normed)
 
 
 class TrimKVQwen3Model(nn.Module):
@@ -316,9 +322,10 @@ class TrimKVQwen3Model(nn.Module):
         position_embeddings = rotary_tables(position_ids, c.head_dim, c.rope_theta, inputs_embeds.dtype,
                                             int(c.head_dim * getattr(c, "partial_rotary_factor", 1.0)), getattr(c, "rope_scaling", None))
         hidden_states = inputs_embeds
+        pending = None    # the last MLP output; its residual add rides in the next norm
         for layer in self.layers:
-            hidden_states = layer(hidden_states, position_embeddings, attention_mask, past_key_values, cache_position)
-        hidden_states = self.norm(hidden_states)
+            hidden_states, pending = layer(hidden_states, position_embeddings, attention_mask, past_key_values, cache_position, pending)
+        hidden_states = self.norm(hidden_states) if pending is None else self.norm.add_norm(pending, hidden_states)[0]
         c = self.config
         if c.compress_memory:   # qwen3:751-760: after every forward, prompt or decode step
             past_key_values.compress(strategy=c.compress_strategy, memory_size=c.memory_size, buffer_size=c.buffer_size,
