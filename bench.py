@@ -502,6 +502,8 @@ def shell_main(args):
     if args.config not in CONFIGS:
         raise SystemExit("--shell runs on the dense cache: --config 2, 3 or 5 (with the matching --hidden)")
     c = dict(CONFIGS[args.config])
+    if args.batch:
+        c["B"] = args.batch
     L = args.layers or c["L"]
     B, Hkv, Hq, M, buf = c["B"], c["Hkv"], c["Hq"], c["M"], c["buf"]
     dev = torch.device("cuda:0")
@@ -649,6 +651,7 @@ def main():
                     help="produce log beta with the fused `rg` retention gate (MFMA first linear + epilogue inside the append "
                          "kernel) from a random hidden state per layer instead of appending drawn values; reported as a "
                          "variant, the BASELINE configs draw beta directly")
+    ap.add_argument("--batch", type=int, default=0, help="--shell only: override the config's batch size (e.g. 1 for single-stream latency)")
     ap.add_argument("--hidden", type=int, default=4096, help="hidden size for --gate (Qwen3-8B: 4096)")
     ap.add_argument("--gate-stream", choices=("side", "main"), default="main",
                     help="with --gate: run the gate's first linear on the main stream in front of the launch that needs it, or on a "

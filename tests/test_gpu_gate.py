@@ -280,6 +280,14 @@ def test_gate_module_repacks_when_its_weights_change():
         g.linear1.weight.mul_(0.5)                                                  # in place: the version counter moves
     b = g(x).materialize()
     assert g._packed_w["w1"][1] is not first
+    g.linear1.weight.data.mul_(2.0)                                                 # through .data: no trace in the version counter
+    stale = g._packed_w["w1"][1]
+    g.invalidate_packed()
+    c = g(x).materialize()
+    assert g._packed_w["w1"][1] is not stale and not torch.equal(b, c)
+    g.linear1.weight.data.mul_(0.5)
+    g.invalidate_packed()
+    assert torch.equal(g(x).materialize(), b)
     g.fused = False
     want = g(x)                                                                     # the torch expression on the new weights
     assert not torch.equal(a, b) and (b.float() - want.float()).abs().max() <= 3e-2 * want.float().abs().max() + 2e-3

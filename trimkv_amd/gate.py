@@ -65,6 +65,13 @@ class RetentionGate(nn.Module):
     # lanes want them (trimkv_gate_pack_weights): 1 KiB contiguous per load instruction instead of 16 rows x 64 bytes.
     packed_max_tokens = 256
 
+    def invalidate_packed(self) -> None:
+        """Drop the derived copies of the parameters (packed first-layer weights, fp32 bias).  They are rebuilt by themselves
+        when a parameter is replaced, moved or written in place (its version counter moves: ``copy_``, ``load_state_dict``,
+        an optimizer step); a write through ``param.data`` leaves no trace, so call this after one."""
+        self.__dict__.pop("_packed_w", None)
+        self.__dict__.pop("_bias32", None)
+
     def _packed(self, lib, name: str, w: torch.Tensor) -> torch.Tensor:
         """The packed copy of first-layer weight ``w``, rebuilt when the parameter has changed or moved."""
         cache = self.__dict__.setdefault("_packed_w", {})
