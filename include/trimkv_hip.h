@@ -571,15 +571,18 @@ int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_stride_h, i
  * q_tok_stride elements apart (likewise k with kv_heads: slices of one fused projection are fine), optional per-head
  * RMS-norm weights [head_dim] (both or neither), cos/sin [batch or 1][seq][rotary_dim] (cs_batch_stride 0 = shared by
  * the batch), rotation of the first rotary_dim (even) features, the rest passed through; q_out [batch][q_heads][seq]
- * [head_dim], k_out [batch][kv_heads][seq][head_dim].  head_dim <= 128.
+ * [head_dim], k_out [batch][kv_heads][seq][head_dim].  head_dim <= 128.  v / v_out (both or neither): v, laid out like k,
+ * is copied unchanged into v_out [batch][kv_heads][seq][head_dim] by the same launch, so that a slice of a fused q|k|v
+ * projection reaches the cache with k's strides (what trimkv_append_attend* require of k_new and v_new).
  *
  * trimkv_silu_mul (Qwen3MLP :121): out[t][i] = round(silu(gate[t][i])) * up[t][i], rows gate_stride / up_stride
  * elements apart (halves of one fused projection are fine), out [ntok][inter]; inter and strides multiples of 8.
  */
 int trimkv_rmsnorm(const void* x, int64_t x_stride, const void* residual, int64_t residual_stride, const void* weight,
                    void* out, void* sum_out, int ntok, int hidden, float eps, int dtype, void* stream);
-int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* q_weight, const void* k_weight,
-                        const void* cos, const void* sin, int64_t cs_batch_stride, void* q_out, void* k_out,
+int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* v, int64_t v_tok_stride,
+                        const void* q_weight, const void* k_weight, const void* cos, const void* sin, int64_t cs_batch_stride,
+                        void* q_out, void* k_out, void* v_out,
                         int batch, int seq, int q_heads, int kv_heads, int head_dim, int rotary_dim, float eps, int dtype, void* stream);
 int trimkv_silu_mul(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
                     int ntok, int inter, int dtype, void* stream);

@@ -81,8 +81,8 @@ def test_qk_norm_rope(dtype, B, S, Hq, Hkv, D, R, norm, fused, per_batch):
     rnd = lambda *s: torch.randn(*s, generator=gen, device=DEV)
     if fused:                                                       # q | k | v side by side in one projection output
         qkv = (rnd(B, S, (Hq + 2 * Hkv) * D) * 2).to(dtype)
-        q, k, _ = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
-        q, k = q.view(B, S, Hq, D), k.view(B, S, Hkv, D)
+        q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+        q, k, v = q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
     else:
         q, k = (rnd(B, S, Hq, D) * 2).to(dtype), (rnd(B, S, Hkv, D) * 2).to(dtype)
     qw = (1 + 0.2 * rnd(D)).to(dtype) if norm else None
@@ -104,6 +104,10 @@ def test_qk_norm_rope(dtype, B, S, Hq, Hkv, D, R, norm, fused, per_batch):
         tol = 2 * _ulp(want.float(), dtype) + 2 * _ulp(torch.full_like(want.float(), 4.0), dtype) * norm
         assert ((got.float() - want.float()).abs() <= tol).all(), float((got.float() - want.float()).abs().max())
         assert (got != want).float().mean() < (0.05 if norm else 1e-9)   # without a norm nothing is summed: bit for bit
+    if fused:   # v rides along: copied into k's layout by the same launch, q and k as without it
+        q3, k3, v3 = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, 1e-6, v)
+        assert torch.equal(q3, gq) and torch.equal(k3, gk)
+        assert v3.is_contiguous() and torch.equal(v3, v.transpose(1, 2))
     # float64: norm, then the rotation by the angle the tables encode
     if R == D and norm:
         q64 = q.double()
@@ -156,13 +160,33 @@ def test_decoder_with_and_without_the_fused_launches(family):
         return torch.stack(logits).float()
 
     assert decoder_ops.enabled
+    before = dict(decoder_ops.counts)
     fused = run()
+    L, calls = cfg.num_hidden_layers, 11                           # one prompt call + ten decode steps
+    issued = {k: decoder_ops.counts[k] - before[k] for k in before}
+    assert issued == {"rmsnorm": calls * (2 * L + 1), "qk_norm_rope": calls * L, "silu_mul": calls * L}, issued
+    # q, k, v and gate, up are one product each: the parameters are views of one buffer, under their own names
+    attn, mlp = model.model.layers[0].self_attn, model.model.layers[0].mlp
+    if hasattr(attn, "q_proj"):
+        w = attn._qkv_rows.weight
+        assert attn.q_proj.weight.data_ptr() == w.data_ptr() and attn.v_proj.weight.data_ptr() == w[-attn.v_proj.out_features:].data_ptr()
+        assert "model.layers.0.self_attn.k_proj.weight" in model.state_dict()
+    if hasattr(mlp, "gate_proj"):
+        assert mlp.up_proj.weight.data_ptr() == mlp._gate_up.weight[mlp.gate_proj.out_features:].data_ptr()
+    # every decode step appended inside its attention launch (k and v reach the cache with common strides)
     decoder_ops.enabled = False
     try:
         plain = run()
+        assert {k: decoder_ops.counts[k] - before[k] for k in before} == issued     # nothing more was launched
     finally:
         decoder_ops.enabled = True
     assert (fused - plain).abs().max() <= 2e-2 + 2e-2 * plain.abs().max(), float((fused - plain).abs().max())
+    # moving the model replaces the parameters: the fused buffers follow
+    model.to(torch.float16)
+    with torch.no_grad():
+        model(ids[:, :4])
+    if hasattr(attn, "q_proj"):
+        assert attn._qkv_rows.weight.dtype == torch.float16 and attn.q_proj.weight.data_ptr() == attn._qkv_rows.weight.data_ptr()
 
 
 def test_the_fused_launches_stay_out_of_training_and_cpu():

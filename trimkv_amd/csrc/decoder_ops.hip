@@ -5,7 +5,9 @@
 //                        (Qwen3RMSNorm, src/trimkv/models/qwen3/modeling_trimkv_qwen3.py:89-103; with `residual` also the
 //                        add in front of it, :431-435, whose sum is written too)
 //   trimkv_qk_norm_rope  per-head RMS norm of q and k (:328-329; weights optional: the Llama and Phi-3 files have none) and
-//                        RoPE on the first rotary_dim features (apply_rotary_pos_emb, :125-151), written as [B, H, S, D]
+//                        RoPE on the first rotary_dim features (apply_rotary_pos_emb, :125-151), written as [B, H, S, D];
+//                        optionally v is copied into the same layout (a slice of a fused q|k|v projection becomes a tensor
+//                        with k's strides, which the fused append wants)
 //   trimkv_silu_mul      out = round(silu(gate)) * up  (Qwen3MLP, :121)
 //
 // Every intermediate is rounded to the 16-bit dtype where the torch modules round it; sums run in another order than
@@ -71,9 +73,9 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(NormArgs a) {
 
 // ---- per-head norm + RoPE, one wavefront per (token, head) -----------------------------------
 struct RopeArgs {
-    const uint16_t* q; const uint16_t* k; const uint16_t* qw; const uint16_t* kw; const uint16_t* cos; const uint16_t* sin;
-    uint16_t* q_out; uint16_t* k_out;
-    int64_t q_tok_stride, k_tok_stride, cs_batch_stride, units;
+    const uint16_t* q; const uint16_t* k; const uint16_t* v; const uint16_t* qw; const uint16_t* kw; const uint16_t* cos; const uint16_t* sin;
+    uint16_t* q_out; uint16_t* k_out; uint16_t* v_out;
+    int64_t q_tok_stride, k_tok_stride, v_tok_stride, cs_batch_stride, units;
     int seq, hq, hkv, d, rd; float eps;
 };
 
@@ -82,15 +84,16 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(RopeArgs a) {
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= a.units) return;
-    const int heads = a.hq + a.hkv;
+    const int heads = a.hq + a.hkv + (a.v ? a.hkv : 0);
     const int64_t t = unit / heads;
     const int h = (int)(unit - t * heads);
-    const bool is_k = h >= a.hq;
-    const int head = is_k ? h - a.hq : h, nh = is_k ? a.hkv : a.hq;
-    const uint16_t* src = is_k ? a.k + t * a.k_tok_stride + (int64_t)head * a.d : a.q + t * a.q_tok_stride + (int64_t)head * a.d;
-    const uint16_t* w = is_k ? a.kw : a.qw;
+    const int kind = h < a.hq ? 0 : h < a.hq + a.hkv ? 1 : 2;      // q, k, or v (copied as it is: no norm, no rotation)
+    const int head = kind == 0 ? h : kind == 1 ? h - a.hq : h - a.hq - a.hkv, nh = kind == 0 ? a.hq : a.hkv;
+    const uint16_t* src = (kind == 0 ? a.q + t * a.q_tok_stride : kind == 1 ? a.k + t * a.k_tok_stride : a.v + t * a.v_tok_stride) + (int64_t)head * a.d;
+    const uint16_t* w = kind == 0 ? a.qw : kind == 1 ? a.kw : nullptr;
+    const int rd = kind == 2 ? 0 : a.rd;
     const int64_t b = t / a.seq, s = t - b * a.seq;
-    uint16_t* dst = (is_k ? a.k_out : a.q_out) + ((b * nh + head) * a.seq + s) * a.d;
+    uint16_t* dst = (kind == 0 ? a.q_out : kind == 1 ? a.k_out : a.v_out) + ((b * nh + head) * a.seq + s) * a.d;
     // the lane holds features lane and lane + 64
     const int e0 = lane, e1 = lane + 64;
     const bool in0 = e0 < a.d, in1 = e1 < a.d;
@@ -101,22 +104,22 @@ __global__ __launch_bounds__(256) void qk_norm_rope_kernel(RopeArgs a) {
         if (in1) y1 = dop_round<F16>(dop_load<F16>(w[e1]) * dop_round<F16>(y1 * inv));
     }
     // rotate_half: feature i < rd pairs with i + rd/2 (negated) or i - rd/2
-    const int half = a.rd >> 1;
+    const int half = rd >> 1;
     const int p0 = e0 < half ? e0 + half : e0 - half, p1 = e1 < half ? e1 + half : e1 - half;   // partners (meaningful below rd)
     const int q0 = min(max(p0, 0), 127), q1 = min(max(p1, 0), 127);
     const float a0 = __shfl(y0, q0 & 63, 64), b0 = __shfl(y1, q0 & 63, 64);
     const float a1 = __shfl(y0, q1 & 63, 64), b1 = __shfl(y1, q1 & 63, 64);
     const float r0 = q0 < 64 ? a0 : b0, r1 = q1 < 64 ? a1 : b1;
-    const uint16_t* cs = a.cos + b * a.cs_batch_stride + s * a.rd;
+    const uint16_t* cs = a.cos + b * a.cs_batch_stride + s * a.rd;     // not touched when rd == 0
     const uint16_t* sn = a.sin + b * a.cs_batch_stride + s * a.rd;
     if (in0) {
         float o = y0;
-        if (e0 < a.rd) o = dop_round<F16>(y0 * dop_load<F16>(cs[e0])) + dop_round<F16>((e0 < half ? -r0 : r0) * dop_load<F16>(sn[e0]));
+        if (e0 < rd) o = dop_round<F16>(y0 * dop_load<F16>(cs[e0])) + dop_round<F16>((e0 < half ? -r0 : r0) * dop_load<F16>(sn[e0]));
         dst[e0] = dop_bits<F16>(o);
     }
     if (in1) {
         float o = y1;
-        if (e1 < a.rd) o = dop_round<F16>(y1 * dop_load<F16>(cs[e1])) + dop_round<F16>((e1 < half ? -r1 : r1) * dop_load<F16>(sn[e1]));
+        if (e1 < rd) o = dop_round<F16>(y1 * dop_load<F16>(cs[e1])) + dop_round<F16>((e1 < half ? -r1 : r1) * dop_load<F16>(sn[e1]));
         dst[e1] = dop_bits<F16>(o);
     }
 }
@@ -168,11 +171,14 @@ extern "C" int trimkv_rmsnorm(const void* x, int64_t x_stride, const void* resid
     return launch_status(fn);
 }
 
-extern "C" int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* q_weight, const void* k_weight,
-                                   const void* cos, const void* sin, int64_t cs_batch_stride, void* q_out, void* k_out,
+extern "C" int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* v, int64_t v_tok_stride,
+                                   const void* q_weight, const void* k_weight, const void* cos, const void* sin, int64_t cs_batch_stride,
+                                   void* q_out, void* k_out, void* v_out,
                                    int batch, int seq, int q_heads, int kv_heads, int head_dim, int rotary_dim, float eps, int dtype, void* stream) {
     const char* fn = "trimkv_qk_norm_rope";
     if (!q || !k || !q_out || !k_out || (rotary_dim > 0 && (!cos || !sin))) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
+    if ((v != nullptr) != (v_out != nullptr)) return fail(TRIMKV_ERR_NULL, "%s: v and v_out come together or not at all", fn);
+    if (v && v_tok_stride < (int64_t)kv_heads * head_dim) return fail(TRIMKV_ERR_SHAPE, "%s: the token stride of v must cover its heads (%lld)", fn, (long long)v_tok_stride);
     if ((q_weight != nullptr) != (k_weight != nullptr)) return fail(TRIMKV_ERR_NULL, "%s: the two norm weights come together or not at all", fn);
     if (int rc = dop_dtype(fn, dtype)) return rc;
     if (batch <= 0 || seq <= 0 || q_heads <= 0 || kv_heads <= 0 || head_dim <= 0 || head_dim > 128 || rotary_dim < 0 || rotary_dim > head_dim || rotary_dim % 2)
@@ -180,9 +186,9 @@ extern "C" int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const vo
                     kv_heads, head_dim, rotary_dim);
     if (q_tok_stride < (int64_t)q_heads * head_dim || k_tok_stride < (int64_t)kv_heads * head_dim || cs_batch_stride < 0)
         return fail(TRIMKV_ERR_SHAPE, "%s: token strides must cover the heads (%lld, %lld)", fn, (long long)q_tok_stride, (long long)k_tok_stride);
-    RopeArgs a{(const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)q_weight, (const uint16_t*)k_weight, (const uint16_t*)cos, (const uint16_t*)sin,
-               (uint16_t*)q_out, (uint16_t*)k_out, q_tok_stride, k_tok_stride, cs_batch_stride, (int64_t)batch * seq * (q_heads + kv_heads),
-               seq, q_heads, kv_heads, head_dim, rotary_dim, eps};
+    RopeArgs a{(const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_weight, (const uint16_t*)k_weight, (const uint16_t*)cos,
+               (const uint16_t*)sin, (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)v_out, q_tok_stride, k_tok_stride, v_tok_stride, cs_batch_stride,
+               (int64_t)batch * seq * (q_heads + kv_heads + (v ? kv_heads : 0)), seq, q_heads, kv_heads, head_dim, rotary_dim, eps};
     const int64_t blocks = (a.units + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(TRIMKV_ERR_SHAPE, "%s: too many (token, head) pairs", fn);
     hipStream_t st = (hipStream_t)stream;

@@ -14,6 +14,7 @@ import torch
 from . import _lib
 
 enabled = True
+counts = {"rmsnorm": 0, "qk_norm_rope": 0, "silu_mul": 0}   # launches issued so far (tests check that a decoder really takes this path)
 
 
 def usable(*tensors: Optional[torch.Tensor]) -> bool:
@@ -40,6 +41,7 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optiona
         x2 = x2.contiguous()
     out = torch.empty(x2.shape, dtype=x.dtype, device=x.device)
     lib = _lib.load()
+    counts["rmsnorm"] += 1
     if residual is None:
         rc = lib.trimkv_rmsnorm(x2.data_ptr(), x2.stride(0), None, 0, weight.data_ptr(), out.data_ptr(), None, x2.shape[0], hidden,
                                 float(eps), _lib.dtype_code(x.dtype), _lib.current_stream(x.device))
@@ -63,24 +65,38 @@ def qk_norm_rope_ok(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: to
         return False
     if cos.shape[2] % 2 or cos.shape[2] > D or not cos.is_contiguous() or not sin.is_contiguous() or cos.dtype != q.dtype:
         return False
-    for t in (q, k):
-        if t.stride(3) != 1 or t.stride(2) != D or t.stride(0) != S * t.stride(1):
-            return False
-    return True
+    return all(token_stride(t) is not None for t in (q, k))
+
+
+def token_stride(t: torch.Tensor) -> Optional[int]:
+    """Elements between consecutive tokens of ``t`` [B, S, H, D] when D is contiguous, the heads lie D apart and the B*S
+    tokens are evenly spaced (what trimkv_qk_norm_rope reads), else None.  (The stride of an axis of length 1 means nothing.)"""
+    B, S, H, D = t.shape
+    if t.stride(3) != 1 or (H > 1 and t.stride(2) != D):
+        return None
+    if S == 1:
+        return t.stride(0) if B > 1 else H * D
+    if B > 1 and t.stride(0) != S * t.stride(1):
+        return None
+    return t.stride(1)
 
 
 def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
-                 cos: torch.Tensor, sin: torch.Tensor, eps: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    """q [B,S,Hq,D], k [B,S,Hkv,D] -> RMS-normed per head (when weights are given) and rotated, as [B,Hq,S,D], [B,Hkv,S,D]."""
+                 cos: torch.Tensor, sin: torch.Tensor, eps: float, v: Optional[torch.Tensor] = None):
+    """q [B,S,Hq,D], k [B,S,Hkv,D] -> RMS-normed per head (when weights are given) and rotated, as [B,Hq,S,D], [B,Hkv,S,D].
+    With ``v`` [B,S,Hkv,D] (laid out like k) a third tensor comes back: v copied into [B,Hkv,S,D] by the same launch."""
     B, S, Hq, D = q.shape
     Hkv = k.shape[2]
     q_out = torch.empty(B, Hq, S, D, dtype=q.dtype, device=q.device)
     k_out = torch.empty(B, Hkv, S, D, dtype=q.dtype, device=q.device)
-    rc = _lib.load().trimkv_qk_norm_rope(q.data_ptr(), q.stride(1), k.data_ptr(), k.stride(1), _lib.ptr(q_weight), _lib.ptr(k_weight),
-                                         cos.data_ptr(), sin.data_ptr(), 0 if cos.shape[0] == 1 else cos.stride(0), q_out.data_ptr(), k_out.data_ptr(),
+    v_out = None if v is None else torch.empty(B, Hkv, S, D, dtype=q.dtype, device=q.device)
+    rc = _lib.load().trimkv_qk_norm_rope(q.data_ptr(), token_stride(q), k.data_ptr(), token_stride(k), _lib.ptr(v), 0 if v is None else token_stride(v),
+                                         _lib.ptr(q_weight), _lib.ptr(k_weight), cos.data_ptr(), sin.data_ptr(),
+                                         0 if cos.shape[0] == 1 else cos.stride(0), q_out.data_ptr(), k_out.data_ptr(), _lib.ptr(v_out),
                                          B, S, Hq, Hkv, D, cos.shape[2], float(eps), _lib.dtype_code(q.dtype), _lib.current_stream(q.device))
     _lib.check(rc, "trimkv_qk_norm_rope")
-    return q_out, k_out
+    counts["qk_norm_rope"] += 1
+    return (q_out, k_out) if v is None else (q_out, k_out, v_out)
 
 
 def silu_mul_ok(gate: torch.Tensor, up: torch.Tensor) -> bool:
@@ -104,4 +120,5 @@ def silu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     rc = _lib.load().trimkv_silu_mul(g2.data_ptr(), g2.stride(0), u2.data_ptr(), u2.stride(0), out.data_ptr(), g2.shape[0], inter,
                                      _lib.dtype_code(gate.dtype), _lib.current_stream(gate.device))
     _lib.check(rc, "trimkv_silu_mul")
+    counts["silu_mul"] += 1
     return out

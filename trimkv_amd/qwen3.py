@@ -100,6 +100,65 @@ class RMSNorm(nn.Module):
         return self.forward(total), total
 
 
+class FusedRows:
+    """Several ``nn.Linear`` modules over the same input as ONE matrix product (a decode step is bound by the number of
+    launches, and the vendor library runs three skinny products far below the rate of one wider one: q, k and v of a
+    Qwen3-8B layer at 64 tokens take 68 us apart and about 20 us together).  On first use the weights (and biases) are
+    moved into one buffer of which the modules' parameters become views, so nothing is held twice and ``state_dict`` /
+    ``load_state_dict`` keep working on the original names; if the parameters are replaced later (``.to()``, a new
+    ``nn.Parameter``) the buffer is rebuilt.  Inference on the GPU only; otherwise ``None`` comes back and the caller
+    runs the modules one by one."""
+
+    def __init__(self, *linears: nn.Linear):
+        self.linears = linears
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def _in_place(self) -> bool:
+        w = self.weight
+        if w is None:
+            return False
+        off, esz = 0, w.element_size()
+        for lin in self.linears:
+            p = lin.weight
+            if p.data_ptr() != w.data_ptr() + off * esz or p.dtype != w.dtype or p.device != w.device:
+                return False
+            off += p.numel()
+        if self.bias is not None:
+            off = 0
+            for lin in self.linears:
+                if lin.bias.data_ptr() != self.bias.data_ptr() + off * esz:
+                    return False
+                off += lin.bias.numel()
+        return True
+
+    def _fuse(self) -> None:
+        ws = [lin.weight for lin in self.linears]
+        self.weight = torch.cat([w.detach() for w in ws], dim=0)
+        off = 0
+        for w in ws:
+            w.data = self.weight[off:off + w.shape[0]]
+            off += w.shape[0]
+        self.bias = None
+        if self.linears[0].bias is not None:
+            bs = [lin.bias for lin in self.linears]
+            self.bias = torch.cat([b.detach() for b in bs], dim=0)
+            off = 0
+            for b in bs:
+                b.data = self.bias[off:off + b.shape[0]]
+                off += b.shape[0]
+
+    def __call__(self, x: torch.Tensor):
+        first = self.linears[0]
+        if not decoder_ops.usable(x, *(lin.weight for lin in self.linears)):
+            return None
+        if any((lin.bias is None) != (first.bias is None) or lin.in_features != first.in_features for lin in self.linears):
+            return None
+        if not self._in_place():
+            self._fuse()
+        return F.linear(x, self.weight, self.bias).split([lin.out_features for lin in self.linears], dim=-1)
+
+
 class MLP(nn.Module):
     def __init__(self, config: TrimKVQwen3Config):
         super().__init__()
@@ -109,7 +168,11 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=bias)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        gate, up = self.gate_proj(x), self.up_proj(x)
+        fused = self.__dict__.get("_gate_up")
+        if fused is None:
+            fused = self.__dict__["_gate_up"] = FusedRows(self.gate_proj, self.up_proj)
+        both = fused(x)
+        gate, up = both if both is not None else (self.gate_proj(x), self.up_proj(x))
         if decoder_ops.usable(gate, up) and decoder_ops.silu_mul_ok(gate, up):
             return self.down_proj(decoder_ops.silu_mul(gate, up))
         return self.down_proj(F.silu(gate) * up)
@@ -197,7 +260,13 @@ class TrimKVQwen3Attention(nn.Module):
         """The outputs of the q, k and v projections as [B,S,H,D] views (qwen3:326-328), before any norm."""
         B, S, _ = hidden_states.shape
         shape = (B, S, -1, self.head_dim)
-        return self.q_proj(hidden_states).view(shape), self.k_proj(hidden_states).view(shape), self.v_proj(hidden_states).view(shape)
+        fused = self.__dict__.get("_qkv_rows")
+        if fused is None:
+            fused = self.__dict__["_qkv_rows"] = FusedRows(self.q_proj, self.k_proj, self.v_proj)
+        qkv = fused(hidden_states)        # one product; q, k, v are slices of its output
+        if qkv is None:
+            qkv = (self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states))
+        return qkv[0].view(shape), qkv[1].view(shape), qkv[2].view(shape)
 
     def _head_norms(self):
         """The per-head RMS norms of q and k (qwen3:328-329), or (None, None) for a family without them."""
@@ -210,6 +279,11 @@ class TrimKVQwen3Attention(nn.Module):
         qn, kn = self._head_norms()
         qw, kw = (None, None) if qn is None else (qn.weight, kn.weight)
         if decoder_ops.usable(q, k, cos, sin, qw, kw) and decoder_ops.qk_norm_rope_ok(q, k, cos, sin):
+            v_stride = decoder_ops.token_stride(v)
+            if v_stride is not None and v_stride != v.shape[2] * v.shape[3] and v.dtype == q.dtype:
+                # v is a slice of a wider projection output: the same launch copies it into k's layout (the fused append takes
+                # k and v with common strides)
+                return decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps, v)
             q, k = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps)
             return q, k, v.transpose(1, 2)
         if qn is not None:
