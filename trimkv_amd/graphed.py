@@ -1,7 +1,7 @@
 """Decode steps replayed from a HIP graph.
 
-A decode step of the thin decoders in this package is some fifteen launches per layer, and at small batch sizes the host
-that enqueues them is slower than the GPU that runs them (Qwen3-1.7B shape, batch 16: 8.0 ms per eager step, 3.6 ms
+A decode step of the thin decoders in this package is some ten launches per layer, and at small batch sizes the host
+that enqueues them is slower than the GPU that runs them (Qwen3-1.7B shape, batch 16: 6.7 ms per eager step, 2.7 ms
 replayed; at batch 64 of the Qwen3-8B shape the host keeps up and a replay gains nothing).  ``GraphedDecoder`` captures one step -- every layer's retention gate,
 projections, RoPE, the append + attention launch, the MLP, the final norm (and the LM head), then the eviction launch --
 once, and replays it per token.  What makes the step replayable is in the cache: between ``begin_device_steps`` and
@@ -10,8 +10,8 @@ index of the eviction on the device, so the same recorded launches are right at 
 
 The `rg` gate stays on the stream of the step by default.  ``gate_on_side_stream=True`` forks it inside the graph onto a
 second stream of the same priority, beside the q/k/v projections; measured at the Qwen3-8B shape (36 layers, batch 64)
-that replay is slower, not faster (13.4 ms against 12.7 ms per step, 12.4 ms without a gate): a graph with 36 forks and
-joins replays through several queues with host-side hand-overs (3.2 ms of host time per replay against 0.2 ms).
+that replay is slower, not faster (12.3 ms against 11.7 ms per step, 11.3 ms without a gate): a graph with 36 forks and
+joins replays through several queues with host-side hand-overs (0.9 ms of host time per replay against 0.1 ms).
 
 No counterpart in the reference (its decoders run eagerly under HF ``generate``); the call order of the captured step is
 the reference's (modeling_trimkv_qwen3.py:315-388, 751-760).
