@@ -142,3 +142,39 @@ def test_graphed_decoder_refuses_what_it_cannot_replay():
     with pytest.raises(ValueError):
         dec(input_ids=torch.zeros(1, 2, dtype=torch.int64, device=DEV))
     dec.close()
+
+
+def test_two_decoders_over_one_cache_take_turns():
+    """Two captured steps over the same cache (as a caller holds who switches between sampling set-ups): both advance the one
+    device-side token counter, so evictions fire at the right step whichever decoder replays, and a decoder made after
+    another was closed starts from the right count."""
+    from trimkv_amd.graphed import GraphedDecoder
+    cfg, model = _model("qwen3", "rg")
+    M, buf = cfg.memory_size, cfg.buffer_size
+    B, prompt, steps = 2, 90, 2 * buf + 6
+    gen = torch.Generator().manual_seed(7)
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps + 4), generator=gen).to(DEV)
+    with torch.no_grad():
+        cache_g = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+        cache_e = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+    a = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    b = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    cache_e.begin_device_steps(M, buf)
+    for i in range(steps):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        lg = (a if (i // 3) % 2 == 0 else b)(input_ids=tok).logits
+        with torch.no_grad():
+            le = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
+        torch.cuda.synchronize()
+        assert torch.equal(lg, le), f"step {i}"
+        _same_state(cache_g, cache_e, f"step {i}")
+    assert a.graph is not None and b.graph is not None
+    a.close()                                                 # ends the device-side phase of the cache
+    c = GraphedDecoder(model, cache_g, logits_to_keep=1)      # ... and a new decoder starts another
+    for i in range(steps, steps + 4):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        lg = c(input_ids=tok).logits
+        with torch.no_grad():
+            le = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
+        assert torch.equal(lg, le), f"step {i}"
+    _same_state(cache_g, cache_e, "end")

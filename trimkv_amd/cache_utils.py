@@ -498,13 +498,18 @@ class TrimKVCache(_SlabBacked):
             if s.cap < hint:
                 s.regrow(hint)
         self._budget_hint = hint
-        self._seen_dev = torch.full((1,), self._seen_tokens + 1, dtype=torch.int64, device=slabs[0].k.device)
+        dev = slabs[0].k.device
+        if self._seen_dev is None or self._seen_dev.device != dev:
+            self._seen_dev = torch.empty(1, dtype=torch.int64, device=dev)
+        # the counter keeps its address for the life of the cache: graphs captured in an earlier device-side phase, or by
+        # another decoder over this cache, go on advancing and reading the same word
+        self._seen_dev.fill_(self._seen_tokens + 1)
         self.lengths_on_device = True
 
     def end_device_steps(self) -> None:
         """Back to launches sized from the host mirrors of the lengths."""
         self._flush_all()
-        self.lengths_on_device, self._seen_dev = False, None
+        self.lengths_on_device = False
 
     def _compress_on_device(self, strategy: str, memory_size: int, buffer_size: int, skip_layers: int, num_layers: int) -> None:
         """compress() between begin_device_steps and end_device_steps: one ``trimkv_evict_layers`` launch over all layers
@@ -613,7 +618,7 @@ class TrimKVCache(_SlabBacked):
             seq_len = key_states.shape[-2]
             if layer_idx == 0:
                 self._seen_tokens += seq_len
-                if self._seen_dev is not None:
+                if self.lengths_on_device:
                     self._seen_dev.add_(seq_len)
             self._ensure_layer(layer_idx)
             slab = self._slabs[layer_idx]
