@@ -36,14 +36,16 @@ def _same_state(a, b, where):
             assert torch.equal(getattr(sa, name)[:, :n], getattr(sb, name)[:, :n]), f"{where}: {name} of layer {l}"
 
 
-@pytest.mark.parametrize("family,gate,fork", [("qwen3", "rg", False), ("qwen3", "rg", True), ("qwen3", "rg2", False), ("qwen3", "rg3", False),
-                                              ("llama", "rg", False), ("phi3", "rg2", False)])
-def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate, fork):
-    """``fork``: the `rg` gate runs on a second stream inside the graph, beside the projections."""
+@pytest.mark.parametrize("family,gate,fork,long", [("qwen3", "rg", False, False), ("qwen3", "rg", True, False), ("qwen3", "rg2", False, False),
+                                                   ("qwen3", "rg3", False, False), ("llama", "rg", False, False), ("phi3", "rg2", False, False),
+                                                   ("qwen3", "rg", False, True), ("phi3", "rg", False, True)])
+def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate, fork, long):
+    """``fork``: the `rg` gate runs on a second stream inside the graph, beside the projections.  ``long``: segments long
+    enough that the attention launch cuts each into pieces (a static piece list, merged inside the launch)."""
     from trimkv_amd.graphed import GraphedDecoder
-    cfg, model = _model(family, gate)
+    cfg, model = _model(family, gate, **(dict(memory_size=1100, buffer_size=8) if long else {}))
     M, buf = cfg.memory_size, cfg.buffer_size
-    B, prompt, steps = 3, 90, 3 * buf + 5                     # three evictions inside the replays
+    B, prompt, steps = 3, (1200 if long else 90), 3 * buf + 5  # three evictions inside the replays
     gen = torch.Generator().manual_seed(1)
     ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps), generator=gen).to(DEV)
     with torch.no_grad():
@@ -53,6 +55,9 @@ def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate, fork):
     assert cache_g.get_cache_length(0) == M                   # the prompt was evicted to the budget
     dec = GraphedDecoder(model, cache_g, gate_on_side_stream=fork, logits_to_keep=1)
     cache_e.begin_device_steps(M, buf)                        # the eager twin issues the same launches
+    assert (cache_g._device_pieces is not None) == long
+    if long:
+        assert cache_g._device_pieces[1] == 3 * cache_g._slabs[0].nseg
     evictions = 0
     for i in range(steps):
         tok = ids[:, prompt + i:prompt + i + 1]

@@ -168,7 +168,7 @@ def append_attend(slab, query: torch.Tensor, group: int, scale: float, chunk: in
         ws = _workspace_zeroed(query.device, lib.trimkv_decode_attn_pieces_workspace(npieces, group), st)
         fn = lib.trimkv_append_attend_pieces_gated if gated else lib.trimkv_append_attend_pieces
         rc = fn(query.data_ptr(), out.data_ptr(), *slab.ptrs, plist.data_ptr(), npieces, nseg, slab.H, slab.cap, d, group, *slab.codes,
-                *slab.pending[0], scale, slab.max_len, ws.data_ptr(), ws.numel(), st)
+                *slab.pending[0], scale, bound if bound > 0 else slab.max_len, ws.data_ptr(), ws.numel(), st)
         if rc:
             _lib.check(rc, "trimkv_append_attend_pieces_gated" if gated else "trimkv_append_attend_pieces")
         slab.pending = None
@@ -339,14 +339,17 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         pps = _uniform_cut(B * Hkv, n)
         if pps > 1 and G not in _DENSE_PIECES_GROUPS:
             pps = 0    # wide groups in pieces: the grid launch + merge kernel
-    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None and window is None and plain, True if pps > 1 else None)
+    # ... and where its segments are cut, the cuts come from a list that names pieces, not rows (merged inside the launch)
+    dev_pieces = flash_attn_kwargs.get("device_pieces") if on_device and not dense_chunk and G in _FUSED_PIECES_GROUPS else None
+    slab = _take_pending(flash_attn_kwargs, query, key, G, Q == 1 and attention_mask is None and window is None and plain,
+                         True if pps > 1 or dev_pieces is not None else None)
     if slab is not None:
         q2 = query.reshape(B * Hq, D)
         if not q2.is_contiguous():
             q2 = q2.contiguous()
         if slab.cu is not None:
             pps = 0
-        return append_attend(slab, q2, G, scale, chunk=dense_chunk, uniform_pps=pps,
+        return append_attend(slab, q2, G, scale, chunk=dense_chunk, uniform_pps=pps, pieces=dev_pieces,
                              bound=slab.cap if on_device else 0).view(B, 1, Hq, D), None, None
     kernel_ok = plain and query.dtype in (torch.bfloat16, torch.float16) and D in (64, 96, 128)
     seg_first = None
@@ -369,7 +372,8 @@ def dense_attention_forward(module: nn.Module, query: torch.Tensor, key: torch.T
         if seg_len is not None and (flash_attn_kwargs.get("max_len") != n or seg_len.numel() != B * Hkv):
             seg_len = None
         out = decode_attention(q2, key, value, B * Hkv, G, seg_len, None, cap, cap if on_device and seg_len is not None else n, scale,
-                               chunk=dense_chunk, seg_first=seg_first, uniform_pps=pps)
+                               chunk=dense_chunk, seg_first=seg_first, uniform_pps=pps,
+                               pieces=dev_pieces if seg_len is not None and cap == flash_attn_kwargs.get("seg_cap") else None)
         return out.view(B, 1, Hq, D), None, None
     if kernel_ok and Q > 1 and attention_mask is None and window is None and causal:
         ok = (key.stride(3) == 1 and key.stride(2) == D and key.stride(0) == Hkv * key.stride(1)

@@ -473,6 +473,7 @@ class TrimKVCache(_SlabBacked):
         # Decode steps whose launches depend on no host-side length (begin_device_steps): what a HIP graph can replay.
         self.lengths_on_device = False
         self._seen_dev: Optional[torch.Tensor] = None   # device int64 [1]: tokens seen + 1, the query index of an eviction
+        self._device_pieces = None                      # (device piece list, entries) of the attention launch in that mode
 
     # ---- decode steps that a HIP graph can replay ------------------------------------------------
     def begin_device_steps(self, memory_size: int, buffer_size: int) -> None:
@@ -504,6 +505,18 @@ class TrimKVCache(_SlabBacked):
         # the counter keeps its address for the life of the cache: graphs captured in an earlier device-side phase, or by
         # another decoder over this cache, go on advancing and reading the same word
         self._seen_dev.fill_(self._seen_tokens + 1)
+        # few segments: each is attended in equal pieces merged inside the launch.  The list names (segment, piece) only and
+        # the kernel cuts by the length it finds on the device, so one list serves every step (built here: an upload must
+        # not happen while a graph is being captured)
+        from .attn import hip_attn
+        s0 = slabs[0]
+        pps = hip_attn._uniform_cut(s0.nseg, hint)
+        self._device_pieces = None
+        if pps > 1 and s0.nseg <= 8192:
+            seg = np.arange(s0.nseg, dtype=np.int32)
+            rows = [np.stack([seg, np.full_like(seg, p), np.full_like(seg, pps), seg * pps], axis=1) for p in range(pps)]
+            plist = torch.from_numpy(np.concatenate(rows, axis=0)).to(dev)      # piece-major: the segment is the fast axis
+            self._device_pieces = (plist, s0.nseg * pps)
         self.lengths_on_device = True
 
     def end_device_steps(self) -> None:
@@ -632,6 +645,7 @@ class TrimKVCache(_SlabBacked):
         extra = {"seg_len": slab.seg_len, "max_len": slab.max_len, "seg_cap": slab.cap}
         if self.lengths_on_device:
             extra["lengths_on_device"] = True
+            extra["device_pieces"] = self._device_pieces
         if slab.pending is not None:
             # the last of the max_len rows is not in the slab yet: the attention call that receives this dictionary writes it
             extra["pending_append"] = (self, slab)
