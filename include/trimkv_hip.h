@@ -574,6 +574,11 @@ int trimkv_prefill_attn(const void* q, int64_t q_stride_b, int64_t q_stride_h, i
  * [head_dim], k_out [batch][kv_heads][seq][head_dim].  head_dim <= 128.  v / v_out (both or neither): v, laid out like k,
  * is copied unchanged into v_out [batch][kv_heads][seq][head_dim] by the same launch, so that a slice of a fused q|k|v
  * projection reaches the cache with k's strides (what trimkv_append_attend* require of k_new and v_new).
+ * gate_hidden / gate_w2 / gate_part (all or none): the `rg` retention gate whose first linear ran in the same matrix
+ * product as q, k and v.  gate_hidden [batch*seq][gate_inter] (rows gate_tok_stride apart) = round(W1 x + b1) in `dtype`,
+ * gate_w2 [kv_heads][gate_inter]; the launch writes gate_part f32 [gate_inter/16][batch*seq][kv_heads], the per-slice
+ * sums that trimkv_gate_hidden would have written (:175-176), for trimkv_append_gated / trimkv_append_attend*_gated
+ * to finish.  gate_inter is a multiple of 16.
  *
  * trimkv_silu_mul (Qwen3MLP :121): out[t][i] = round(silu(gate[t][i])) * up[t][i], rows gate_stride / up_stride
  * elements apart (halves of one fused projection are fine), out [ntok][inter]; inter and strides multiples of 8.
@@ -583,6 +588,7 @@ int trimkv_rmsnorm(const void* x, int64_t x_stride, const void* residual, int64_
 int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* v, int64_t v_tok_stride,
                         const void* q_weight, const void* k_weight, const void* cos, const void* sin, int64_t cs_batch_stride,
                         void* q_out, void* k_out, void* v_out,
+                        const void* gate_hidden, int64_t gate_tok_stride, const void* gate_w2, float* gate_part, int gate_inter,
                         int batch, int seq, int q_heads, int kv_heads, int head_dim, int rotary_dim, float eps, int dtype, void* stream);
 int trimkv_silu_mul(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
                     int ntok, int inter, int dtype, void* stream);

@@ -27,3 +27,16 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _decoder_switches_restored():
+    """Tests flip the decoders' class-level switches (fused element-wise launches, gate placement); a failing test must not
+    leave them flipped for the tests after it."""
+    yield
+    mods = sys.modules
+    if "trimkv_amd.decoder_ops" in mods:
+        mods["trimkv_amd.decoder_ops"].enabled = True
+    if "trimkv_amd.qwen3" in mods:
+        attn = mods["trimkv_amd.qwen3"].TrimKVQwen3Attention
+        attn.fold_gate, attn.gate_on_side_stream = True, False

@@ -91,11 +91,13 @@ def test_bad_arguments_are_refused_without_a_launch():
     assert lib.trimkv_rmsnorm(one, 64, one, 64, one, one, None, 4, 64, 1e-6, _lib.BF16, None) == -1       # residual without sum_out
     assert lib.trimkv_rmsnorm(one, 64, None, 0, one, one, None, 4, 64, 1e-6, _lib.F32, None) == -3
     assert lib.trimkv_rmsnorm(ctypes.c_void_p(8), 64, None, 0, one, one, None, 4, 64, 1e-6, _lib.BF16, None) == -2   # misaligned
-    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, one, None, one, one, 0, one, one, None, 1, 1, 4, 2, 128, 128, 1e-6, _lib.BF16, None) == -1
-    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, 1, 1, 4, 2, 256, 128, 1e-6, _lib.BF16, None) == -2
-    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, 1, 1, 4, 2, 128, 63, 1e-6, _lib.BF16, None) == -2
-    assert lib.trimkv_qk_norm_rope(one, 256, one, 256, None, 0, None, None, one, one, 0, one, one, None, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -2   # q rows overlap
-    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, one, 256, None, None, one, one, 0, one, one, None, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -1   # v without v_out
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, one, None, one, one, 0, one, one, None, None, 0, None, None, 0, 1, 1, 4, 2, 128, 128, 1e-6, _lib.BF16, None) == -1
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, None, 0, None, None, 0, 1, 1, 4, 2, 256, 128, 1e-6, _lib.BF16, None) == -2
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, None, 0, None, None, 0, 1, 1, 4, 2, 128, 63, 1e-6, _lib.BF16, None) == -2
+    assert lib.trimkv_qk_norm_rope(one, 256, one, 256, None, 0, None, None, one, one, 0, one, one, None, None, 0, None, None, 0, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -2   # q rows overlap
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, one, 256, None, None, one, one, 0, one, one, None, None, 0, None, None, 0, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -1   # v without v_out
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, one, 512, None, one, 512, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -1   # gate without w2
+    assert lib.trimkv_qk_norm_rope(one, 512, one, 256, None, 0, None, None, one, one, 0, one, one, None, one, 512, one, one, 500, 1, 1, 4, 2, 128, 64, 1e-6, _lib.BF16, None) == -2
     assert lib.trimkv_silu_mul(one, 64, one, 64, None, 4, 64, _lib.BF16, None) == -1
     assert lib.trimkv_silu_mul(one, 64, one, 60, one, 4, 64, _lib.BF16, None) == -2
     assert lib.trimkv_gate_pack_weights(one, None, 4096, 512, _lib.BF16, None) == -1

@@ -169,7 +169,8 @@ def test_decoder_with_and_without_the_fused_launches(family):
     attn, mlp = model.model.layers[0].self_attn, model.model.layers[0].mlp
     if hasattr(attn, "q_proj"):
         w = attn._qkv_rows.weight
-        assert attn.q_proj.weight.data_ptr() == w.data_ptr() and attn.v_proj.weight.data_ptr() == w[-attn.v_proj.out_features:].data_ptr()
+        at_v = attn.q_proj.out_features + attn.k_proj.out_features      # q | k | v (| the `rg` gate's first linear)
+        assert attn.q_proj.weight.data_ptr() == w.data_ptr() and attn.v_proj.weight.data_ptr() == w[at_v:].data_ptr()
         assert "model.layers.0.self_attn.k_proj.weight" in model.state_dict()
     if hasattr(mlp, "gate_proj"):
         assert mlp.up_proj.weight.data_ptr() == mlp._gate_up.weight[mlp.gate_proj.out_features:].data_ptr()
@@ -204,3 +205,47 @@ def test_the_fused_launches_stay_out_of_training_and_cpu():
         assert decoder_ops.usable(x, norm.weight)
         assert ((norm(x).float() - y.float()).abs() <= _ulp(y.float(), torch.bfloat16)).all()
     assert not decoder_ops.usable(x.float(), norm.weight.float())   # fp32
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("B,S,hidden,inter,Hkv", [(64, 1, 4096, 512, 8), (2, 37, 1024, 96, 4), (1, 1, 512, 16, 2)])
+def test_gate_second_half_inside_the_norm_rope_launch(dtype, B, S, hidden, inter, Hkv):
+    """The `rg` gate without a launch of its own: first linear in one product with q, k, v (here: torch's linear on
+    concatenated weights), second half in trimkv_qk_norm_rope.  Against the torch expression of the whole gate, against the
+    stand-alone kernel's partial sums, and q/k/v must come out as without the gate."""
+    from trimkv_amd import LazyLogBeta, decoder_ops, _lib as L
+    from trimkv_amd.qwen3 import rotary_tables
+    gen = torch.Generator(device=DEV).manual_seed(6)
+    rnd = lambda *s: torch.randn(*s, generator=gen, device=DEV)
+    Hq, D = 2 * Hkv, 128
+    x = rnd(B, S, hidden).to(dtype)
+    wq, wk, wv = (rnd(Hq * D, hidden) * 0.03).to(dtype), (rnd(Hkv * D, hidden) * 0.03).to(dtype), (rnd(Hkv * D, hidden) * 0.03).to(dtype)
+    w1, b1, w2 = (rnd(inter, hidden) * 0.03).to(dtype), (rnd(inter) * 0.1).to(dtype), (rnd(Hkv, inter) * 0.05).to(dtype)
+    bias = (rnd(Hkv) + 2).to(dtype)
+    fused_bias = torch.cat([torch.zeros((Hq + 2 * Hkv) * D, dtype=dtype, device=DEV), b1])
+    y = torch.nn.functional.linear(x, torch.cat([wq, wk, wv, w1]), fused_bias)
+    q, k, v, gh = y.split([Hq * D, Hkv * D, Hkv * D, inter], dim=-1)
+    q, k, v = q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
+    cos, sin = rotary_tables(torch.arange(S, device=DEV)[None], D, 10000.0, dtype)
+    assert decoder_ops.gate_rows_ok(gh, w2, B, S, Hkv)
+    q1, k1, v1, part = decoder_ops.qk_norm_rope(q, k, None, None, cos, sin, 1e-6, v, (gh, w2))
+    q0, k0, v0 = decoder_ops.qk_norm_rope(q, k, None, None, cos, sin, 1e-6, v)
+    assert torch.equal(q1, q0) and torch.equal(k1, k0) and torch.equal(v1, v0)
+    assert part.shape == (inter // 16, B * S, Hkv) and part.dtype == torch.float32
+    got = LazyLogBeta(part, bias.float(), B, S, Hkv, dtype).materialize().float()
+    # the module in torch ops on the same first-layer outputs (bias added and rounded by the product, as nn.Linear does)
+    want16 = torch.nn.functional.logsigmoid(torch.nn.functional.linear(torch.nn.functional.silu(gh), w2) + bias).float()
+    h64 = x.double() @ w1.double().T + b1.double()
+    want64 = torch.nn.functional.logsigmoid((h64 * torch.sigmoid(h64)) @ w2.double().T + bias.double()).float()
+    tol = 3e-2 * want64.abs() + 4e-3
+    assert ((got - want64).abs() <= tol).all(), float((got - want64).abs().max())
+    assert (got - want16).abs().mean() <= (want16 - want64).abs().mean() * 2 + 1e-4
+    # the stand-alone kernel on the same inputs: the same slices, sums that differ by the rounding of h only
+    if hidden % 512 == 0:
+        lib = L.load()
+        ref = torch.zeros_like(part)
+        x2 = x.reshape(B * S, hidden)
+        L.check(lib.trimkv_gate_hidden(x2.data_ptr(), w1.data_ptr(), b1.data_ptr(), w2.data_ptr(), ref.data_ptr(), B * S, hidden, inter, Hkv,
+                                       L.dtype_code(dtype), L.current_stream(torch.device(DEV))), "gate_hidden")
+        torch.cuda.synchronize()
+        assert (part - ref).abs().max() <= 2e-2 * ref.abs().max() + 1e-3

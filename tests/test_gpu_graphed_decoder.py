@@ -43,6 +43,9 @@ def test_replayed_steps_equal_eager_steps_bit_for_bit(family, gate, fork, long):
     """``fork``: the `rg` gate runs on a second stream inside the graph, beside the projections.  ``long``: segments long
     enough that the attention launch cuts each into pieces (a static piece list, merged inside the launch)."""
     from trimkv_amd.graphed import GraphedDecoder
+    from trimkv_amd.qwen3 import TrimKVQwen3Attention
+    if fork:    # the forked gate is a launch of its own (trimkv_gate_hidden): the eager twin must run that kernel too
+        TrimKVQwen3Attention.fold_gate = False
     cfg, model = _model(family, gate, **(dict(memory_size=1100, buffer_size=8) if long else {}))
     M, buf = cfg.memory_size, cfg.buffer_size
     B, prompt, steps = 3, (1200 if long else 90), 3 * buf + 5  # three evictions inside the replays
@@ -158,7 +161,7 @@ def test_two_decoders_over_one_cache_take_turns():
     M, buf = cfg.memory_size, cfg.buffer_size
     B, prompt, steps = 2, 90, 2 * buf + 6
     gen = torch.Generator().manual_seed(7)
-    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps + 4), generator=gen).to(DEV)
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps + 7), generator=gen).to(DEV)
     with torch.no_grad():
         cache_g = model(ids[:, :prompt], logits_to_keep=1).past_key_values
         cache_e = model(ids[:, :prompt], logits_to_keep=1).past_key_values
@@ -174,6 +177,20 @@ def test_two_decoders_over_one_cache_take_turns():
         assert torch.equal(lg, le), f"step {i}"
         _same_state(cache_g, cache_e, f"step {i}")
     assert a.graph is not None and b.graph is not None
+    # parameters of some decoder were moved into another buffer (here: only said so): the recorded addresses may be stale,
+    # so the next call runs eagerly and the one after captures anew -- with the same results
+    from trimkv_amd import decoder_ops
+    decoder_ops.layout_epoch += 1
+    old_graph = a.graph
+    for i in range(steps, steps + 3):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        lg = a(input_ids=tok).logits
+        assert (a.graph is None) == (i == steps)
+        with torch.no_grad():
+            le = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
+        assert torch.equal(lg, le), f"step {i}"
+    assert a.graph is not old_graph
+    steps += 3
     a.close()                                                 # ends the device-side phase of the cache
     c = GraphedDecoder(model, cache_g, logits_to_keep=1)      # ... and a new decoder starts another
     for i in range(steps, steps + 4):

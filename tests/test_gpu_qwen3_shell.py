@@ -202,11 +202,28 @@ def test_shell_decode_keeps_one_launch_per_layer_with_the_fused_gate(gate):
     hidden size: the deferred append must engage all the same (the attention launch finishes the gate), and the logits
     must equal, bit for bit, those of a run whose cache appends in a launch of its own."""
     from trimkv_amd import LazyLogBeta, TrimKVCache
+    from trimkv_amd.qwen3 import TrimKVQwen3Attention
     torch.manual_seed(3)
     cfg = _tiny_config("qwen3", retention_gate=gate)
     assert cfg.hidden_size % 512 == 0
     model = _family("qwen3")[1](cfg).to(torch.bfloat16).to(DEV).eval()
     B, P, STEPS = 2, 70, 24
+    folded = None
+    if gate == "rg":
+        # `rg` by default has no launch of its own (first linear in the product of q, k, v, second half in the norm + RoPE
+        # launch): the step must still be one cache launch per layer, and agree with the stand-alone gate to rounding noise
+        cache = TrimKVCache()
+        cache.fuse_decode_append = True
+        ids0 = torch.randint(0, cfg.vocab_size, (B, P + STEPS), generator=torch.Generator().manual_seed(4)).to(DEV)
+        with torch.no_grad():
+            model(ids0[:, :P], past_key_values=cache)
+            folded = []
+            for t in range(STEPS):
+                folded.append(model(ids0[:, P + t:P + t + 1], past_key_values=cache).logits)
+                assert all(s is None or s.pending is None for s in cache._slabs)
+        folded = torch.cat(folded, dim=1)
+        assert model.model.layers[0].self_attn._qkv_rows.weight.shape[0] == (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim + cfg.retention_gate_intermediate_size
+        TrimKVQwen3Attention.fold_gate = False       # below: the gate as a launch of its own, wherever it runs the same bits
     ids = torch.randint(0, cfg.vocab_size, (B, P + STEPS), generator=torch.Generator().manual_seed(4)).to(DEV)
     runs = {}
     for fuse in (True, False):
@@ -230,8 +247,9 @@ def test_shell_decode_keeps_one_launch_per_layer_with_the_fused_gate(gate):
                 logits.append(out.logits)
                 assert all(s is None or s.pending is None for s in cache._slabs)     # every attention call carried its append out
         runs[fuse] = (torch.cat(logits, dim=1), deferred, [cache.kv_positions[l].clone() for l in range(cfg.num_hidden_layers)])
-    if gate == "rg":   # the gate beside the projections on a second stream (opt-in) or in front of them (default): the same bits
-        from trimkv_amd.qwen3 import TrimKVQwen3Attention
+    if gate == "rg":   # the gate beside the projections on a second stream (opt-in) or in front of them: the same bits
+        TrimKVQwen3Attention.fold_gate = True
+        assert (folded.float() - runs[True][0].float()).abs().max() <= 2e-2 + 2e-2 * runs[True][0].float().abs().max()
         TrimKVQwen3Attention.gate_on_side_stream = True
         try:
             cache = TrimKVCache()

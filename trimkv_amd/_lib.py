@@ -33,7 +33,8 @@ SIGNATURES = {
     "trimkv_gate_hidden_swiglu": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "trimkv_gate_pack_weights": (_i, [_p, _p, _i, _i, _i, _p]),
     "trimkv_rmsnorm": (_i, [_p, _i64, _p, _i64, _p, _p, _p, _i, _i, _f, _i, _p]),
-    "trimkv_qk_norm_rope": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p]),
+    "trimkv_qk_norm_rope": (_i, [_p, _i64, _p, _i64, _p, _i64, _p, _p, _p, _p, _i64, _p, _p, _p, _p, _i64, _p, _p, _i,
+                                 _i, _i, _i, _i, _i, _i, _f, _i, _p]),
     "trimkv_silu_mul": (_i, [_p, _i64, _p, _i64, _p, _i, _i, _i, _p]),
     "trimkv_gate_hidden_packed": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),
     "trimkv_gate_hidden_swiglu_packed": (_i, [_p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _p]),

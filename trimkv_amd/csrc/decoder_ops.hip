@@ -7,7 +7,9 @@
 //   trimkv_qk_norm_rope  per-head RMS norm of q and k (:328-329; weights optional: the Llama and Phi-3 files have none) and
 //                        RoPE on the first rotary_dim features (apply_rotary_pos_emb, :125-151), written as [B, H, S, D];
 //                        optionally v is copied into the same layout (a slice of a fused q|k|v projection becomes a tensor
-//                        with k's strides, which the fused append wants)
+//                        with k's strides, which the fused append wants), and the second half of the `rg` retention gate
+//                        (:175-176: SiLU and the per-slice second linear) is taken on first-layer outputs that came out of
+//                        the same matrix product as q, k and v
 //   trimkv_silu_mul      out = round(silu(gate)) * up  (Qwen3MLP, :121)
 //
 // Every intermediate is rounded to the 16-bit dtype where the torch modules round it; sums run in another order than
@@ -77,16 +79,53 @@ struct RopeArgs {
     uint16_t* q_out; uint16_t* k_out; uint16_t* v_out;
     int64_t q_tok_stride, k_tok_stride, v_tok_stride, cs_batch_stride, units;
     int seq, hq, hkv, d, rd; float eps;
+    // second half of the `rg` retention gate on first-layer outputs that came out of the same product as q, k and v
+    const uint16_t* gate_h; const uint16_t* gate_w2; float* gate_part;
+    int64_t gate_tok_stride; int gate_inter; int ntok;
 };
+
+// part[slice][t][head] = sum over the 16 units u of the slice of w2[head][u] * round(silu(h[t][u])): what gate_hidden_kernel
+// leaves for the append (same slices, same butterfly order within a slice), from h = round(W1 x + b1) computed elsewhere.
+// One wavefront takes 64 units (four slices) of one token for all heads; the loads of a batch of eight heads are issued
+// together (a wavefront that walked units and heads one after the other spent a memory round trip on each: 20 us).
+template <bool F16>
+__device__ __forceinline__ void gate_second_half(const RopeArgs& a, int64_t t, int chunk, int lane) {
+    const int u = chunk * 64 + lane;
+    const bool in = u < a.gate_inter;
+    float act = 0.0f;
+    if (in) {
+        const float x = dop_load<F16>(a.gate_h[t * a.gate_tok_stride + u]);
+        act = dop_round<F16>(x / (1.0f + __expf(-x)));
+    }
+    for (int h0 = 0; h0 < a.hkv; h0 += 8) {
+        float w[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[i] = in && h0 + i < a.hkv ? dop_load<F16>(a.gate_w2[(int64_t)(h0 + i) * a.gate_inter + u]) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float p = act * w[i];
+            p += __shfl_xor(p, 1, 64);
+            p += __shfl_xor(p, 2, 64);
+            p += __shfl_xor(p, 4, 64);
+            p += __shfl_xor(p, 8, 64);
+            if (in && (lane & 15) == 0 && h0 + i < a.hkv) a.gate_part[((int64_t)(u >> 4) * a.ntok + t) * a.hkv + h0 + i] = p;
+        }
+    }
+}
 
 template <bool F16>
 __global__ __launch_bounds__(256) void qk_norm_rope_kernel(RopeArgs a) {
     const int lane = threadIdx.x & 63;
     const int64_t unit = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (unit >= a.units) return;
-    const int heads = a.hq + a.hkv + (a.v ? a.hkv : 0);
+    const int kv_units = a.hq + a.hkv + (a.v ? a.hkv : 0);
+    const int heads = kv_units + (a.gate_h ? (a.gate_inter + 63) >> 6 : 0);
     const int64_t t = unit / heads;
     const int h = (int)(unit - t * heads);
+    if (h >= kv_units) {            // only with a gate: the token's extra wavefronts, 64 units each
+        gate_second_half<F16>(a, t, h - kv_units, lane);
+        return;
+    }
     const int kind = h < a.hq ? 0 : h < a.hq + a.hkv ? 1 : 2;      // q, k, or v (copied as it is: no norm, no rotation)
     const int head = kind == 0 ? h : kind == 1 ? h - a.hq : h - a.hq - a.hkv, nh = kind == 0 ? a.hq : a.hkv;
     const uint16_t* src = (kind == 0 ? a.q + t * a.q_tok_stride : kind == 1 ? a.k + t * a.k_tok_stride : a.v + t * a.v_tok_stride) + (int64_t)head * a.d;
@@ -174,8 +213,15 @@ extern "C" int trimkv_rmsnorm(const void* x, int64_t x_stride, const void* resid
 extern "C" int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const void* k, int64_t k_tok_stride, const void* v, int64_t v_tok_stride,
                                    const void* q_weight, const void* k_weight, const void* cos, const void* sin, int64_t cs_batch_stride,
                                    void* q_out, void* k_out, void* v_out,
+                                   const void* gate_hidden, int64_t gate_tok_stride, const void* gate_w2, float* gate_part, int gate_inter,
                                    int batch, int seq, int q_heads, int kv_heads, int head_dim, int rotary_dim, float eps, int dtype, void* stream) {
     const char* fn = "trimkv_qk_norm_rope";
+    if (gate_hidden || gate_w2 || gate_part) {
+        if (!gate_hidden || !gate_w2 || !gate_part) return fail(TRIMKV_ERR_NULL, "%s: gate_hidden, gate_w2 and gate_part come together or not at all", fn);
+        if (gate_inter <= 0 || gate_inter % 16 || gate_tok_stride < gate_inter)
+            return fail(TRIMKV_ERR_SHAPE, "%s: gate_inter=%d must be a positive multiple of 16 and the token stride must cover it (%lld)", fn, gate_inter,
+                        (long long)gate_tok_stride);
+    }
     if (!q || !k || !q_out || !k_out || (rotary_dim > 0 && (!cos || !sin))) return fail(TRIMKV_ERR_NULL, "%s: null pointer argument", fn);
     if ((v != nullptr) != (v_out != nullptr)) return fail(TRIMKV_ERR_NULL, "%s: v and v_out come together or not at all", fn);
     if (v && v_tok_stride < (int64_t)kv_heads * head_dim) return fail(TRIMKV_ERR_SHAPE, "%s: the token stride of v must cover its heads (%lld)", fn, (long long)v_tok_stride);
@@ -188,7 +234,8 @@ extern "C" int trimkv_qk_norm_rope(const void* q, int64_t q_tok_stride, const vo
         return fail(TRIMKV_ERR_SHAPE, "%s: token strides must cover the heads (%lld, %lld)", fn, (long long)q_tok_stride, (long long)k_tok_stride);
     RopeArgs a{(const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)q_weight, (const uint16_t*)k_weight, (const uint16_t*)cos,
                (const uint16_t*)sin, (uint16_t*)q_out, (uint16_t*)k_out, (uint16_t*)v_out, q_tok_stride, k_tok_stride, v_tok_stride, cs_batch_stride,
-               (int64_t)batch * seq * (q_heads + kv_heads + (v ? kv_heads : 0)), seq, q_heads, kv_heads, head_dim, rotary_dim, eps};
+               (int64_t)batch * seq * (q_heads + kv_heads + (v ? kv_heads : 0) + (gate_hidden ? (gate_inter + 63) / 64 : 0)), seq, q_heads, kv_heads, head_dim, rotary_dim, eps,
+               (const uint16_t*)gate_hidden, (const uint16_t*)gate_w2, gate_part, gate_tok_stride, gate_inter, batch * seq};
     const int64_t blocks = (a.units + 3) / 4;
     if (blocks > 0x7fffffffLL) return fail(TRIMKV_ERR_SHAPE, "%s: too many (token, head) pairs", fn);
     hipStream_t st = (hipStream_t)stream;

@@ -14,6 +14,9 @@ import torch
 from . import _lib
 
 enabled = True
+# Bumped whenever the decoders move parameters into another buffer (FusedRows in qwen3.py).  A captured graph holds the
+# addresses it was recorded with: GraphedDecoder remembers the epoch of its capture and refuses to replay after a move.
+layout_epoch = 0
 counts = {"rmsnorm": 0, "qk_norm_rope": 0, "silu_mul": 0}   # launches issued so far (tests check that a decoder really takes this path)
 
 
@@ -81,22 +84,45 @@ def token_stride(t: torch.Tensor) -> Optional[int]:
     return t.stride(1)
 
 
+def gate_rows_ok(gate_hidden: torch.Tensor, w2: torch.Tensor, batch: int, seq: int, kv_heads: int) -> bool:
+    """gate_hidden [B, S, I] with I contiguous and evenly spaced tokens (a slice of a fused projection is fine), w2 [Hkv, I]
+    contiguous, I a multiple of 16: what the gate's second half inside trimkv_qk_norm_rope reads."""
+    if gate_hidden.dim() != 3 or tuple(gate_hidden.shape[:2]) != (batch, seq) or gate_hidden.stride(2) != 1:
+        return False
+    inter = gate_hidden.shape[2]
+    if inter % 16 or tuple(w2.shape) != (kv_heads, inter) or not w2.is_contiguous() or w2.dtype != gate_hidden.dtype:
+        return False
+    return seq == 1 or batch == 1 or gate_hidden.stride(0) == seq * gate_hidden.stride(1)
+
+
 def qk_norm_rope(q: torch.Tensor, k: torch.Tensor, q_weight: Optional[torch.Tensor], k_weight: Optional[torch.Tensor],
-                 cos: torch.Tensor, sin: torch.Tensor, eps: float, v: Optional[torch.Tensor] = None):
+                 cos: torch.Tensor, sin: torch.Tensor, eps: float, v: Optional[torch.Tensor] = None, gate=None):
     """q [B,S,Hq,D], k [B,S,Hkv,D] -> RMS-normed per head (when weights are given) and rotated, as [B,Hq,S,D], [B,Hkv,S,D].
-    With ``v`` [B,S,Hkv,D] (laid out like k) a third tensor comes back: v copied into [B,Hkv,S,D] by the same launch."""
+    With ``v`` [B,S,Hkv,D] (laid out like k) a third tensor comes back: v copied into [B,Hkv,S,D] by the same launch.
+    With ``gate = (gate_hidden [B,S,I], w2 [Hkv,I])`` -- the first-layer outputs of the `rg` retention gate, bias added and
+    rounded, out of the same product as q, k, v -- the last tensor that comes back holds the gate's per-slice partial sums
+    f32 [I/16, B*S, Hkv] (what ``trimkv_gate_hidden`` leaves for the append to finish)."""
     B, S, Hq, D = q.shape
     Hkv = k.shape[2]
     q_out = torch.empty(B, Hq, S, D, dtype=q.dtype, device=q.device)
     k_out = torch.empty(B, Hkv, S, D, dtype=q.dtype, device=q.device)
     v_out = None if v is None else torch.empty(B, Hkv, S, D, dtype=q.dtype, device=q.device)
+    gh = w2 = part = None
+    g_stride = inter = 0
+    if gate is not None:
+        gh, w2 = gate
+        inter = gh.shape[2]
+        g_stride = gh.stride(1) if S > 1 else (gh.stride(0) if B > 1 else inter)
+        part = torch.empty(inter // 16, B * S, Hkv, dtype=torch.float32, device=q.device)
     rc = _lib.load().trimkv_qk_norm_rope(q.data_ptr(), token_stride(q), k.data_ptr(), token_stride(k), _lib.ptr(v), 0 if v is None else token_stride(v),
                                          _lib.ptr(q_weight), _lib.ptr(k_weight), cos.data_ptr(), sin.data_ptr(),
                                          0 if cos.shape[0] == 1 else cos.stride(0), q_out.data_ptr(), k_out.data_ptr(), _lib.ptr(v_out),
+                                         _lib.ptr(gh), g_stride, _lib.ptr(w2), _lib.ptr(part), inter,
                                          B, S, Hq, Hkv, D, cos.shape[2], float(eps), _lib.dtype_code(q.dtype), _lib.current_stream(q.device))
     _lib.check(rc, "trimkv_qk_norm_rope")
     counts["qk_norm_rope"] += 1
-    return (q_out, k_out) if v is None else (q_out, k_out, v_out)
+    out = (q_out, k_out) if v is None else (q_out, k_out, v_out)
+    return out if gate is None else out + (part,)
 
 
 def silu_mul_ok(gate: torch.Tensor, up: torch.Tensor) -> bool:

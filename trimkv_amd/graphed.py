@@ -22,6 +22,7 @@ from typing import Optional
 
 import torch
 
+from . import decoder_ops
 from .cache_utils import TrimKVCache
 
 
@@ -56,6 +57,7 @@ class GraphedDecoder:
         self.by_ids = True
         self.out = None
         self.calls = 0
+        self._epoch = -1
         self._fork_gate = bool(gate_on_side_stream) and cfg.retention_gate == "rg"
 
     def _forward(self):
@@ -87,6 +89,10 @@ class GraphedDecoder:
         self.static_in.copy_(x)
         self.position.fill_(cache.get_seq_length())
         self.calls += 1
+        if self.graph is not None and self._epoch != decoder_ops.layout_epoch:
+            # some decoder's parameters were moved into another buffer since the capture (a module replaced, a model moved):
+            # the recorded addresses may be stale.  This step runs eagerly, the next one is captured anew.
+            self.graph, self.out, self.calls = None, None, 1
         if self.calls == 1:
             # eager, on the capture's stream: first-use allocations (workspaces, address tables, library handles) happen here
             cur = torch.cuda.current_stream(self.device)
@@ -106,6 +112,7 @@ class GraphedDecoder:
                 self._set_fork(False)
                 cache.mirror_restore(snap)       # the capture ran the cache's Python but nothing on the device
             self.graph = graph
+            self._epoch = decoder_ops.layout_epoch
         self.graph.replay()
         cache.advance_decode_mirrors(self.memory_size, self.buffer_size)
         return self.out

@@ -52,6 +52,7 @@ class Phi3MLP(nn.Module):
 
 class TrimKVPhi3Attention(TrimKVQwen3Attention):
     gate_kinds = ("rg", "rg2")
+    fold_gate = False     # q | k | v are one module here (qkv_proj): the gate keeps its own launch
 
     def _build_projections(self, config) -> None:
         d = config.head_dim

@@ -112,7 +112,7 @@ class FusedRows:
     def __init__(self, *linears: nn.Linear):
         self.linears = linears
         self.weight: Optional[torch.Tensor] = None
-        self.bias: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None      # rows of modules without a bias hold zeros (adding zero changes no bit)
 
     def _in_place(self) -> bool:
         w = self.weight
@@ -123,40 +123,46 @@ class FusedRows:
             p = lin.weight
             if p.data_ptr() != w.data_ptr() + off * esz or p.dtype != w.dtype or p.device != w.device:
                 return False
+            if lin.bias is not None and (self.bias is None or lin.bias.data_ptr() != self.bias.data_ptr() + (off // lin.in_features) * esz):
+                return False
             off += p.numel()
-        if self.bias is not None:
-            off = 0
-            for lin in self.linears:
-                if lin.bias.data_ptr() != self.bias.data_ptr() + off * esz:
-                    return False
-                off += lin.bias.numel()
         return True
 
     def _fuse(self) -> None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("FusedRows: parameters would have to move while a graph is being captured (a module was replaced "
+                               "after the eager warm-up step); run one eager step first")
+        decoder_ops.layout_epoch += 1      # parameters are about to move: captured graphs that read them are stale
         ws = [lin.weight for lin in self.linears]
         self.weight = torch.cat([w.detach() for w in ws], dim=0)
-        off = 0
-        for w in ws:
-            w.data = self.weight[off:off + w.shape[0]]
-            off += w.shape[0]
         self.bias = None
-        if self.linears[0].bias is not None:
-            bs = [lin.bias for lin in self.linears]
-            self.bias = torch.cat([b.detach() for b in bs], dim=0)
-            off = 0
-            for b in bs:
-                b.data = self.bias[off:off + b.shape[0]]
-                off += b.shape[0]
+        if any(lin.bias is not None for lin in self.linears):
+            self.bias = torch.cat([(torch.zeros_like(lin.weight[:, 0]) if lin.bias is None else lin.bias.detach()) for lin in self.linears], dim=0)
+        off = 0
+        for lin in self.linears:
+            n = lin.out_features
+            lin.weight.data = self.weight[off:off + n]
+            if lin.bias is not None:
+                lin.bias.data = self.bias[off:off + n]
+            off += n
 
-    def __call__(self, x: torch.Tensor):
-        first = self.linears[0]
+    def __call__(self, x: torch.Tensor, first: Optional[int] = None):
+        """The outputs of the modules for ``x`` as slices of one product, or None when that cannot be done here (training,
+        CPU, fp32, differing input widths).  ``first``: only the leading ``first`` modules (a prefix of the buffer)."""
         if not decoder_ops.usable(x, *(lin.weight for lin in self.linears)):
             return None
-        if any((lin.bias is None) != (first.bias is None) or lin.in_features != first.in_features for lin in self.linears):
+        if any(lin.in_features != self.linears[0].in_features or (lin.bias is not None and lin.bias.dtype != x.dtype) for lin in self.linears):
             return None
         if not self._in_place():
             self._fuse()
-        return F.linear(x, self.weight, self.bias).split([lin.out_features for lin in self.linears], dim=-1)
+        sizes = [lin.out_features for lin in self.linears[:first]]
+        rows = sum(sizes)
+        bias = self.bias
+        if bias is not None and not any(lin.bias is not None for lin in self.linears[:first]):
+            bias = None
+        elif bias is not None:
+            bias = bias[:rows]
+        return F.linear(x, self.weight[:rows], bias).split(sizes, dim=-1)
 
 
 class MLP(nn.Module):
@@ -256,39 +262,66 @@ class TrimKVQwen3Attention(nn.Module):
             return RetentionGate(config.hidden_size, *common)
         return (RetentionGate2 if kind == "rg2" else RetentionGate3)(config.head_dim, *common)
 
-    def _projections(self, hidden_states: torch.Tensor):
-        """The outputs of the q, k and v projections as [B,S,H,D] views (qwen3:326-328), before any norm."""
+    def _projections(self, hidden_states: torch.Tensor, with_gate: bool = False):
+        """The outputs of the q, k and v projections as [B,S,H,D] views (qwen3:326-328), before any norm.  ``with_gate``: the
+        first linear of the `rg` gate (qwen3:171-174: the same input, a bias of its own) rides in the same product; a fourth
+        tensor [B,S,I] comes back, or None where the product cannot be shared (then the caller runs the gate by itself)."""
         B, S, _ = hidden_states.shape
         shape = (B, S, -1, self.head_dim)
+        linears = [self.q_proj, self.k_proj, self.v_proj]
+        if isinstance(self.retention_gate, RetentionGate) and self.config.retention_gate == "rg":
+            linears.append(self.retention_gate.linear1)
         fused = self.__dict__.get("_qkv_rows")
-        if fused is None:
-            fused = self.__dict__["_qkv_rows"] = FusedRows(self.q_proj, self.k_proj, self.v_proj)
-        qkv = fused(hidden_states)        # one product; q, k, v are slices of its output
+        # kept while the modules wanted now are the leading ones of the buffer (a gate taken away later leaves q | k | v where
+        # they are: moving the weights would pull the ground from under every captured graph that reads them)
+        if fused is None or len(fused.linears) < len(linears) or any(a is not b for a, b in zip(fused.linears, linears)):
+            fused = self.__dict__["_qkv_rows"] = FusedRows(*linears)      # first use, or a module was replaced or added
+        n = 4 if with_gate and len(linears) == 4 else 3
+        qkv = fused(hidden_states, n)     # one product; q, k, v (and the gate's hidden layer) are slices of its output
         if qkv is None:
             qkv = (self.q_proj(hidden_states), self.k_proj(hidden_states), self.v_proj(hidden_states))
-        return qkv[0].view(shape), qkv[1].view(shape), qkv[2].view(shape)
+        out = (qkv[0].view(shape), qkv[1].view(shape), qkv[2].view(shape))
+        return out + ((qkv[3] if len(qkv) == 4 else None),) if with_gate else out
 
     def _head_norms(self):
         """The per-head RMS norms of q and k (qwen3:328-329), or (None, None) for a family without them."""
         return getattr(self, "q_norm", None), getattr(self, "k_norm", None)
 
-    def _qkv_rope(self, hidden_states: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
+    def _qkv_rope(self, hidden_states: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, fold_gate: bool = False):
         """q [B,Hq,S,D] and k [B,Hkv,S,D] after the per-head norm and RoPE, v [B,Hkv,S,D] (qwen3:326-337, 341-343).  On the GPU
-        at inference norm and rotation of q and k are one launch (trimkv_qk_norm_rope)."""
-        q, k, v = self._projections(hidden_states)
+        at inference norm and rotation of q and k are one launch (trimkv_qk_norm_rope).  ``fold_gate``: a fourth value comes
+        back, the `rg` gate's log beta for these tokens as a LazyLogBeta [B,S,Hkv] -- its first linear computed in the product
+        of q, k, v and its second half in that same launch -- or None where that cannot be done."""
+        gate_h = None
+        if fold_gate:
+            q, k, v, gate_h = self._projections(hidden_states, True)
+        else:
+            q, k, v = self._projections(hidden_states)
+        lazy = None
         qn, kn = self._head_norms()
         qw, kw = (None, None) if qn is None else (qn.weight, kn.weight)
         if decoder_ops.usable(q, k, cos, sin, qw, kw) and decoder_ops.qk_norm_rope_ok(q, k, cos, sin):
+            B, S = q.shape[:2]
             v_stride = decoder_ops.token_stride(v)
-            if v_stride is not None and v_stride != v.shape[2] * v.shape[3] and v.dtype == q.dtype:
-                # v is a slice of a wider projection output: the same launch copies it into k's layout (the fused append takes
-                # k and v with common strides)
-                return decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps, v)
-            q, k = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps)
-            return q, k, v.transpose(1, 2)
-        if qn is not None:
-            q, k = qn(q), kn(k)
-        return apply_rope(q.transpose(1, 2), cos, sin), apply_rope(k.transpose(1, 2), cos, sin), v.transpose(1, 2)
+            # v as a slice of a wider projection output: the same launch copies it into k's layout (the fused append takes k
+            # and v with common strides)
+            v_in = v if v_stride is not None and v_stride != v.shape[2] * v.shape[3] and v.dtype == q.dtype else None
+            gate = None
+            if gate_h is not None:
+                w2 = self.retention_gate.linear2.weight
+                if decoder_ops.usable(gate_h, w2) and decoder_ops.gate_rows_ok(gate_h, w2, B, S, k.shape[2]):
+                    gate = (gate_h, w2)
+            res = decoder_ops.qk_norm_rope(q, k, qw, kw, cos, sin, self.config.rms_norm_eps, v_in, gate)
+            if gate is not None:
+                g = self.retention_gate
+                lazy = LazyLogBeta(res[-1], g._bias_f32(q.device), B, S, g.num_key_value_heads, q.dtype)
+            q, k = res[0], res[1]
+            v = res[2] if v_in is not None else v.transpose(1, 2)
+        else:
+            if qn is not None:
+                q, k = qn(q), kn(k)
+            q, k, v = apply_rope(q.transpose(1, 2), cos, sin), apply_rope(k.transpose(1, 2), cos, sin), v.transpose(1, 2)
+        return (q, k, v, lazy) if fold_gate else (q, k, v)
 
     # `rg` depends on nothing but the normed hidden state, as the q/k/v projections do.  With this flag its first linear
     # (trimkv_gate_hidden) is issued on a second stream of the same priority and joined by an event before update(), so that
@@ -297,6 +330,11 @@ class TrimKVQwen3Attention(nn.Module):
     # host runs far ahead of the GPU; this eager decoder is host-bound at decode batch sizes (measured at the Qwen3-8B
     # shape, batch 64: 18.9 ms per step with the gate on the main stream, 23.6 ms with the fork, 18.1 ms without a gate).
     gate_on_side_stream = False
+    # The `rg` gate without a launch of its own: its first linear is one more block of rows in the product that computes q, k
+    # and v (the same input), its second half (SiLU, the per-slice second linear) a few more wavefronts of the norm + RoPE
+    # launch.  The vendor library's product sums in another order than trimkv_gate_hidden's MFMA kernel, so log beta agrees
+    # with the stand-alone gate to rounding noise, not bit for bit.
+    fold_gate = True
 
     def _gate_beside_projections(self, hidden_states):
         """The `rg` gate of this layer on the side stream; returns (log beta, event to wait for before it is read)."""
@@ -321,14 +359,22 @@ class TrimKVQwen3Attention(nn.Module):
         B, S, _ = hidden_states.shape
         # `rg` sees the normed hidden state, before RoPE (qwen3:332-333); on the GPU this is a LazyLogBeta
         retention, gate_done = None, None
+        cos, sin = position_embeddings
         if self.config.retention_gate == "rg":
             if self.gate_on_side_stream and hidden_states.is_cuda and not self.training:
                 retention, gate_done = self._gate_beside_projections(hidden_states)
+                q, k, v = self._qkv_rope(hidden_states, cos, sin)
+            elif self.fold_gate and getattr(self.retention_gate, "_use_hip", lambda x: False)(hidden_states):
+                # the gate's first linear in the product of q, k, v, its second half in the norm + RoPE launch: no launch of its own
+                q, k, v, retention = self._qkv_rope(hidden_states, cos, sin, True)
+                if retention is None:
+                    retention = self.retention_gate(hidden_states)
             else:
                 retention = self.retention_gate(hidden_states)
+                q, k, v = self._qkv_rope(hidden_states, cos, sin)
             retention = retention.transpose(1, 2)
-        cos, sin = position_embeddings
-        q, k, v = self._qkv_rope(hidden_states, cos, sin)
+        else:
+            q, k, v = self._qkv_rope(hidden_states, cos, sin)
         if self.config.retention_gate in ("rg2", "rg3"):   # these see concat(K, V) after RoPE (qwen3:345-347)
             retention = self.retention_gate(torch.cat([k, v], dim=-1)).transpose(1, 2)
         offset = past_key_values.get_seq_length(self.layer_idx)
