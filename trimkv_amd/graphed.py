@@ -8,9 +8,10 @@ once, and replays it per token.  What makes the step replayable is in the cache:
 ``end_device_steps`` a dense ``TrimKVCache`` enqueues launches that read the segment lengths, the position and the query
 index of the eviction on the device, so the same recorded launches are right at every step, eviction steps included.
 
-The `rg` gate stays on the stream of the step by default.  ``gate_on_side_stream=True`` forks it inside the graph onto a
+The `rg` gate stays on the stream of the step by default (in the Qwen3 and Llama shells it has no launch of its own: its
+first linear rides in the product of q, k and v, its second half in the norm + RoPE launch).  ``gate_on_side_stream=True`` forks it inside the graph onto a
 second stream of the same priority, beside the q/k/v projections; measured at the Qwen3-8B shape (36 layers, batch 64)
-that replay is slower, not faster (12.3 ms against 11.7 ms per step, 11.3 ms without a gate): a graph with 36 forks and
+that replay is slower, not faster (12.3 ms against 11.4 ms per step, 11.3 ms without a gate): a graph with 36 forks and
 joins replays through several queues with host-side hand-overs (0.9 ms of host time per replay against 0.1 ms).
 
 No counterpart in the reference (its decoders run eagerly under HF ``generate``); the call order of the captured step is

@@ -323,12 +323,12 @@ class TrimKVQwen3Attention(nn.Module):
             q, k, v = apply_rope(q.transpose(1, 2), cos, sin), apply_rope(k.transpose(1, 2), cos, sin), v.transpose(1, 2)
         return (q, k, v, lazy) if fold_gate else (q, k, v)
 
-    # `rg` depends on nothing but the normed hidden state, as the q/k/v projections do.  With this flag its first linear
-    # (trimkv_gate_hidden) is issued on a second stream of the same priority and joined by an event before update(), so that
-    # it runs beside the projections, the head norms and RoPE instead of in front of them.  Off by default: the fork and
-    # join cost the host about 45 us per layer (stream switch, two events) to hide an 11 us kernel, which only pays when the
-    # host runs far ahead of the GPU; this eager decoder is host-bound at decode batch sizes (measured at the Qwen3-8B
-    # shape, batch 64: 18.9 ms per step with the gate on the main stream, 23.6 ms with the fork, 18.1 ms without a gate).
+    # `rg` depends on nothing but the normed hidden state, as the q/k/v projections do.  With this flag its first linear runs
+    # as a launch of its own (trimkv_gate_hidden) on a second stream of the same priority, joined by an event before update(),
+    # beside the projections, the head norms and RoPE instead of in front of them.  Off by default: the fork and join cost the
+    # host about 45 us per layer (stream switch, two events) to hide an 8 us kernel, and the decoder has no host time to spare
+    # (Qwen3-8B shape, batch 64: 11.7 ms per step with the fork against 11.3 ms with that kernel on the step's stream and
+    # 11.0 ms with the gate folded into the projections, see fold_gate).
     gate_on_side_stream = False
     # The `rg` gate without a launch of its own: its first linear is one more block of rows in the product that computes q, k
     # and v (the same input), its second half (SiLU, the per-slice second linear) a few more wavefronts of the norm + RoPE
