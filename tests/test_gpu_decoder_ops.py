@@ -249,3 +249,44 @@ def test_gate_second_half_inside_the_norm_rope_launch(dtype, B, S, hidden, inter
                                        L.dtype_code(dtype), L.current_stream(torch.device(DEV))), "gate_hidden")
         torch.cuda.synchronize()
         assert (part - ref).abs().max() <= 2e-2 * ref.abs().max() + 1e-3
+
+
+def test_fused_rows_survive_training_steps_and_reloads():
+    """After inference has moved q, k, v (and the gate's first linear) into one buffer the parameters are views of it:
+    autograd, an optimizer step and load_state_dict must keep working on them, and inference must see the new values."""
+    from tests.test_gpu_qwen3_shell import _family, _tiny_config
+    cfg = _tiny_config("qwen3", retention_gate="rg")
+    torch.manual_seed(0)
+    model = _family("qwen3")[1](cfg).to(torch.bfloat16).to(DEV).eval()
+    ids = torch.randint(0, cfg.vocab_size, (2, 12), generator=torch.Generator().manual_seed(5)).to(DEV)
+    with torch.no_grad():
+        before = model(ids).logits.float()
+    attn = model.model.layers[0].self_attn
+    fused = attn._qkv_rows
+    assert len(fused.linears) == 4 and attn.retention_gate.linear1.weight.data_ptr() == fused.weight[-cfg.retention_gate_intermediate_size:].data_ptr()
+    assert attn.retention_gate.linear1.bias.data_ptr() == fused.bias[-cfg.retention_gate_intermediate_size:].data_ptr()
+    saved = {k: v.clone() for k, v in model.state_dict().items()}
+    # a training step: the torch expressions run (no fused launch takes a tensor that wants a gradient)
+    model.train()
+    opt = torch.optim.SGD(model.parameters(), lr=0.05)
+    loss = model(ids).logits.float().square().mean()
+    loss.backward()
+    # (the HIP attention has no backward: gradients reach what lies behind it -- the MLPs, whose gate_proj and up_proj are
+    # views of one buffer too -- and the residual stream)
+    mlp = model.model.layers[0].mlp
+    for lin in (mlp.gate_proj, mlp.up_proj, mlp.down_proj):
+        assert lin.weight.grad is not None and lin.weight.grad.abs().max() > 0
+    opt.step()
+    with torch.no_grad():
+        attn.q_proj.weight.mul_(1.05)                                        # q, k, v get no gradient here: step them by hand
+    model.eval()
+    assert attn.q_proj.weight.data_ptr() == fused.weight.data_ptr()          # updated in place: still the one buffer
+    assert mlp.up_proj.weight.data_ptr() == mlp._gate_up.weight[mlp.gate_proj.out_features:].data_ptr()
+    with torch.no_grad():
+        after = model(ids).logits.float()
+    assert attn._qkv_rows is fused and (after - before).abs().max() > 1e-3    # inference reads the stepped weights
+    # ... and a checkpoint written before the step restores the first answer
+    model.load_state_dict(saved)
+    with torch.no_grad():
+        again = model(ids).logits.float()
+    assert attn.q_proj.weight.data_ptr() == fused.weight.data_ptr() and torch.equal(again, before)
