@@ -73,6 +73,8 @@ def _torch_qk(q, k, qw, kw, cos, sin, eps):
     (2, 9, 4, 4, 96, 96, False, True, False),         # Phi-3-mini heads
     (2, 3, 4, 2, 64, 64, True, False, False),
     (1, 4, 2, 1, 128, 0, True, False, False),         # no rotation at all
+    (2, 3, 4, 2, 128, 40, True, False, False),        # a rotary width the 16-byte kernel does not take: the 2-byte one runs
+    (5, 7, 5, 5, 72, 48, True, True, True),           # 72 features per head: nine of a row's sixteen lanes busy
 ])
 def test_qk_norm_rope(dtype, B, S, Hq, Hkv, D, R, norm, fused, per_batch):
     from trimkv_amd import decoder_ops
