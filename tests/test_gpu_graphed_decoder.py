@@ -200,3 +200,41 @@ def test_two_decoders_over_one_cache_take_turns():
             le = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
         assert torch.equal(lg, le), f"step {i}"
     _same_state(cache_g, cache_e, "end")
+
+
+@pytest.mark.parametrize("B", [1, 16, 64])
+def test_replays_at_the_real_layer_shape(B):
+    """The Qwen3-8B layer shape (hidden 4096, 32 / 8 heads, MLP 12288; two layers): the vendor library picks other GEMM kernels
+    here than at the toy sizes above, and a library call that records a memset node into a graph has given wrong results
+    on replays after the first.  So: several replays with eager work and synchronisations in between, every one compared
+    bit for bit with the eager twin."""
+    from trimkv_amd.graphed import GraphedDecoder
+    from trimkv_amd.qwen3 import TrimKVQwen3Config, TrimKVQwen3ForCausalLM
+    cfg = TrimKVQwen3Config(vocab_size=2048, hidden_size=4096, intermediate_size=12288, num_hidden_layers=2, num_attention_heads=32,
+                            num_key_value_heads=8, head_dim=128, retention_gate="rg", retention_gate_intermediate_size=512,
+                            retention_gate_bias_init=2.0, memory_size=256, buffer_size=8)
+    torch.manual_seed(0)
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        with torch.device(DEV):
+            model = TrimKVQwen3ForCausalLM(cfg).eval()
+    finally:
+        torch.set_default_dtype(torch.float32)
+    prompt, steps = 300, 20
+    ids = torch.randint(0, cfg.vocab_size, (B, prompt + steps), generator=torch.Generator().manual_seed(8)).to(DEV)
+    with torch.no_grad():
+        cache_g = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+        cache_e = model(ids[:, :prompt], logits_to_keep=1).past_key_values
+    dec = GraphedDecoder(model, cache_g, logits_to_keep=1)
+    cache_e.begin_device_steps(cfg.memory_size, cfg.buffer_size)
+    for i in range(steps):
+        tok = ids[:, prompt + i:prompt + i + 1]
+        lg = dec(input_ids=tok).logits
+        with torch.no_grad():
+            le = model(tok, past_key_values=cache_e, cache_position=torch.tensor([prompt + i], device=DEV), logits_to_keep=1).logits
+        torch.cuda.synchronize()
+        assert torch.isfinite(lg.float()).all()
+        assert torch.equal(lg, le), f"step {i}: the replay differs from the eager step by {float((lg.float() - le.float()).abs().max())}"
+        _same_state(cache_g, cache_e, f"step {i}")
+    assert dec.graph is not None
+    dec.close()
