@@ -292,3 +292,37 @@ def test_fused_rows_survive_training_steps_and_reloads():
     with torch.no_grad():
         again = model(ids).logits.float()
     assert attn.q_proj.weight.data_ptr() == fused.weight.data_ptr() and torch.equal(again, before)
+
+
+def test_prompt_sized_launches():
+    """Sizes of a prompt chunk: more 16-byte pieces than the SiLU launch has threads (its grid is capped and strides), a norm
+    over tens of thousands of rows, a rotation over a million (token, head) rows -- values against the torch expressions."""
+    from trimkv_amd import decoder_ops
+    from trimkv_amd.qwen3 import rotary_tables
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    dtype = torch.bfloat16
+    g = (torch.randn(20000, 8192, generator=gen, device=DEV) * 2).to(dtype)
+    u = torch.randn(20000, 8192, generator=gen, device=DEV).to(dtype)
+    assert g.numel() // 8 > 65536 * 256
+    got, want = decoder_ops.silu_mul(g, u), torch.nn.functional.silu(g) * u
+    assert ((got.float() - want.float()).abs() <= _ulp(want.float(), dtype)).all() and (got != want).float().mean() < 0.01
+    del g, u, got, want
+    x = (torch.randn(30000, 4096, generator=gen, device=DEV) * 2).to(dtype)
+    w = (1 + 0.1 * torch.randn(4096, generator=gen, device=DEV)).to(dtype)
+    got, want = decoder_ops.rmsnorm(x, w, 1e-6), _torch_rmsnorm(x, w, 1e-6)
+    err, ulp = (got.float() - want.float()).abs(), _ulp(want.float(), dtype)
+    # two roundings in a row (the normed value, then its product with the weight): among 10^8 values a few tip twice
+    assert (err <= 2 * ulp).all() and (err > ulp).float().mean() < 1e-4 and (got != want).float().mean() < 0.02
+    del x, got, want, err, ulp
+    B, S, Hq, Hkv, D = 4, 8192, 32, 8, 128
+    qkv = torch.randn(B, S, (Hq + 2 * Hkv) * D, generator=gen, device=DEV).to(dtype)
+    q, k, v = qkv.split([Hq * D, Hkv * D, Hkv * D], dim=-1)
+    q, k, v = q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
+    qw = (1 + 0.1 * torch.randn(D, generator=gen, device=DEV)).to(dtype)
+    cos, sin = rotary_tables(torch.arange(S, device=DEV)[None], D, 1e6, dtype)
+    gq, gk, gv = decoder_ops.qk_norm_rope(q, k, qw, qw, cos, sin, 1e-6, v)
+    wq, wk = _torch_qk(q, k, qw, qw, cos, sin, 1e-6)
+    assert torch.equal(gv, v.transpose(1, 2))
+    for got, want in ((gq, wq), (gk, wk)):
+        tol = 2 * _ulp(want.float(), dtype) + 2 * _ulp(torch.full_like(want.float(), 4.0), dtype)
+        assert ((got.float() - want.float()).abs() <= tol).all()
