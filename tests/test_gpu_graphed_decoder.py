@@ -238,3 +238,47 @@ def test_replays_at_the_real_layer_shape(B):
         _same_state(cache_g, cache_e, f"step {i}")
     assert dec.graph is not None
     dec.close()
+
+
+def test_checkpoint_to_tokens_with_and_without_a_graph(tmp_path):
+    """The whole way a user goes: a base checkpoint directory + a TrimKV directory on disk -> from_pretrained -> GPU ->
+    generate with chunked prefill; replayed from a graph and eagerly the same tokens, and saving the state afterwards gives
+    back what was loaded (the parameters have meanwhile become views of fused buffers)."""
+    import json
+    from safetensors.torch import save_file
+    from trimkv_amd.qwen3 import TrimKVQwen3Config, TrimKVQwen3ForCausalLM
+    torch.manual_seed(0)
+    hf = dict(vocab_size=256, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8, num_key_value_heads=2,
+              head_dim=128, rms_norm_eps=1e-6, rope_parameters={"rope_theta": 10000.0, "rope_type": "default"}, architectures=["Qwen3ForCausalLM"])
+    src = TrimKVQwen3ForCausalLM(TrimKVQwen3Config.from_dict(dict(hf, retention_gate="rg", retention_gate_intermediate_size=64)))
+    for p in src.parameters():
+        p.data.normal_(0, 0.05)
+    full = {k: v.clone().to(torch.bfloat16) for k, v in src.state_dict().items()}
+    gate = {k: v for k, v in full.items() if "retention_gate" in k}
+    base_dir, trim_dir = tmp_path / "base", tmp_path / "trimkv"
+    base_dir.mkdir(); trim_dir.mkdir()
+    save_file({k: v.contiguous() for k, v in full.items() if k not in gate}, str(base_dir / "model.safetensors"))
+    (base_dir / "config.json").write_text(json.dumps(hf))
+    (trim_dir / "config.json").write_text(json.dumps(dict(hf, base_model=str(base_dir), retention_gate="rg", memory_size=64, buffer_size=16,
+                                                          retention_gate_intermediate_size=64, trainable_params="retention_gate")))
+    torch.save(gate, str(trim_dir / "trimkv_weights.pth"))
+    model = TrimKVQwen3ForCausalLM.from_pretrained(str(trim_dir)).to(DEV)
+    ids = torch.randint(0, 256, (2, 150), generator=torch.Generator().manual_seed(11)).to(DEV)
+    graphed = model.generate(ids, 40, prefill_chunk=64, use_graph=True)
+    assert graphed.shape == (2, 190) and torch.equal(graphed[:, :150], ids)
+    # eagerly, on launches that read the lengths on the device as the replayed ones do
+    with torch.no_grad():
+        out = None
+        for s in range(0, 150, 64):
+            out = model(ids[:, s:s + 64], past_key_values=None if out is None else out.past_key_values, logits_to_keep=1)
+        cache = out.past_key_values
+        cache.begin_device_steps(model.config.memory_size, model.config.buffer_size)
+        toks = [ids]
+        for i in range(40):
+            nxt = out.logits[:, -1].argmax(-1, keepdim=True)
+            toks.append(nxt)
+            if i + 1 < 40:
+                out = model(nxt, past_key_values=cache, logits_to_keep=1)
+    assert torch.equal(graphed, torch.cat(toks, dim=1))
+    after = model.state_dict()
+    assert set(after) == set(full) and all(torch.equal(after[k].cpu(), full[k]) for k in full)
