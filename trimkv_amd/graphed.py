@@ -101,6 +101,9 @@ class GraphedDecoder:
             with torch.cuda.stream(self.stream):
                 out = self._forward()
             cur.wait_stream(self.stream)
+            for t in vars(out).values():          # allocated on the capture's stream, read by the caller on its own
+                if torch.is_tensor(t):
+                    t.record_stream(cur)
             return out
         if self.graph is None:
             snap = cache.mirror_snapshot()
